@@ -1,0 +1,255 @@
+// paged_attention (decode) on AMD Instinct MI355X: descriptor, launch plan and launches.
+// Takes the place of the reference's nvidia backend host code
+// (src/infiniop/ops/paged_attention/nvidia/paged_attention_nvidia.cu:182-443 and
+// nvidia/paged_attention_hd128.cu:424-923) for the AMD device.
+#include "paged_attention_amd.h"
+#include "../../../handle.h"
+#include "../../../../utils/check.h"
+#include "../../../devices/amd/amd_device.h"
+#include "decode_common.h"
+#include "decode_generic.h"
+#include "decode_reduce.h"
+#include "decode_tiled.h"
+#include <cstdlib>
+#include <cstring>
+
+namespace op::paged_attention::amd {
+
+namespace {
+
+// Decided once, at descriptor creation, from shapes and the device alone (sequence lengths live in
+// device memory and are never read on the host).
+struct Plan {
+    bool tiled;            // tiled matrix-core kernel (head 128, power-of-two pages >= 16, 16-byte aligned strides)
+    int partition_tokens;  // tokens per unit of work
+    int max_partitions;    // partitions the longest representable sequence needs
+    int dims_per_lane;     // generic / reduce kernels: ceil(max(head_size, value_size) / 64)
+    size_t acc_bytes, ml_bytes; // workspace carve-up: [acc][m][l], each region 256-byte aligned
+};
+
+size_t alignUp(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+int floorPow2(long long x) {
+    int p = 1;
+    while (2LL * p <= x) {
+        p *= 2;
+    }
+    return p;
+}
+
+bool multipleOf8(ptrdiff_t x) { return (x % 8) == 0; }
+
+Plan makePlan(const PagedAttentionInfo &in, const device::amd::DeviceInfo &dev) {
+    Plan plan{};
+    const long long bs = static_cast<long long>(in.page_block_size);
+    const long long max_tokens = static_cast<long long>(in.max_num_blocks_per_seq) * bs;
+    const bool pow2_page = bs >= 16 && (bs & (bs - 1)) == 0;
+
+    plan.tiled = in.head_size == kTiledHead && in.value_size == kTiledHead && pow2_page
+              && multipleOf8(in.q_stride) && multipleOf8(in.q_head_stride) && multipleOf8(in.o_stride)
+              && multipleOf8(in.o_head_stride) && multipleOf8(in.k_batch_stride) && multipleOf8(in.k_head_stride)
+              && multipleOf8(in.k_row_stride) && multipleOf8(in.v_batch_stride) && multipleOf8(in.v_head_stride)
+              && multipleOf8(in.v_row_stride) && in.num_blocks > 0 && in.num_blocks <= 0x7fffffff;
+    if (const char *env = std::getenv("INFINIOP_AMD_PA_KERNEL")) {
+        if (std::strcmp(env, "generic") == 0) {
+            plan.tiled = false;
+        }
+    }
+
+    // Units of work the kernel is launched with = sequences x KV heads (x query heads for the
+    // generic kernel) x partitions. Aim at ~16 units per compute unit for the longest sequences, so
+    // that ragged batches still fill the device; keep a partition between 64 and 512 tokens.
+    const long long group = static_cast<long long>(in.num_heads / in.num_kv_heads);
+    const long long streams = static_cast<long long>(in.num_seqs)
+                            * (plan.tiled ? in.num_kv_heads * ((group + kHeadsPerWave - 1) / kHeadsPerWave) : in.num_heads);
+    long long want = streams * max_tokens / (16LL * dev.compute_units);
+    int p = floorPow2(want < 1 ? 1 : want);
+    p = p < 64 ? 64 : (p > 512 ? 512 : p);
+    if (const char *env = std::getenv("INFINIOP_AMD_PA_PARTITION")) {
+        const int forced = std::atoi(env);
+        if (forced >= 16) {
+            p = (forced + 15) / 16 * 16;
+        }
+    }
+    // Bound the workspace: at most 128 partitions, unless that would exceed what one wavefront can
+    // address through its single page-id load (64 table entries).
+    const long long cap = plan.tiled ? 64 * bs : (1LL << 30);
+    if (max_tokens > 128LL * p) {
+        long long grown = (max_tokens + 127) / 128;
+        grown = (grown + 15) / 16 * 16;
+        p = static_cast<int>(grown);
+    }
+    if (p > cap) {
+        p = static_cast<int>(cap);
+    }
+    plan.partition_tokens = p;
+    plan.max_partitions = static_cast<int>(max_tokens > 0 ? (max_tokens + p - 1) / p : 1);
+    const size_t widest = in.head_size > in.value_size ? in.head_size : in.value_size;
+    plan.dims_per_lane = static_cast<int>((widest + 63) / 64);
+
+    if (plan.max_partitions > 1) {
+        const size_t slots = in.num_seqs * in.num_heads * static_cast<size_t>(plan.max_partitions);
+        plan.acc_bytes = alignUp(slots * in.value_size * sizeof(float), 256);
+        plan.ml_bytes = alignUp(slots * sizeof(float), 256);
+    }
+    return plan;
+}
+
+template <typename T, typename Tindex>
+void launchGeneric(const DecodeArgs &a, const Plan &plan, hipStream_t stream) {
+    const dim3 grid(plan.max_partitions, a.num_heads, a.num_seqs);
+    switch (plan.dims_per_lane) {
+    case 1: decodeGenericKernel<T, Tindex, 1><<<grid, 64, 0, stream>>>(a); break;
+    case 2: decodeGenericKernel<T, Tindex, 2><<<grid, 64, 0, stream>>>(a); break;
+    case 3: decodeGenericKernel<T, Tindex, 3><<<grid, 64, 0, stream>>>(a); break;
+    case 4: decodeGenericKernel<T, Tindex, 4><<<grid, 64, 0, stream>>>(a); break;
+    default: decodeGenericKernel<T, Tindex, 9><<<grid, 64, 0, stream>>>(a); break;
+    }
+}
+
+template <typename T, typename Tindex>
+void launchReduce(const DecodeArgs &a, const Plan &plan, hipStream_t stream) {
+    const dim3 grid(a.num_heads, a.num_seqs);
+    switch (plan.dims_per_lane) {
+    case 1: decodeReduceKernel<T, Tindex, 1><<<grid, 64, 0, stream>>>(a); break;
+    case 2: decodeReduceKernel<T, Tindex, 2><<<grid, 64, 0, stream>>>(a); break;
+    case 3: decodeReduceKernel<T, Tindex, 3><<<grid, 64, 0, stream>>>(a); break;
+    case 4: decodeReduceKernel<T, Tindex, 4><<<grid, 64, 0, stream>>>(a); break;
+    default: decodeReduceKernel<T, Tindex, 9><<<grid, 64, 0, stream>>>(a); break;
+    }
+}
+
+template <typename T, typename Tindex>
+void launchAll(const DecodeArgs &a, const Plan &plan, bool tiled, hipStream_t stream) {
+    if (tiled) {
+        const int head_chunks = (a.group + kHeadsPerWave - 1) / kHeadsPerWave;
+        const dim3 grid(plan.max_partitions, a.num_kv_heads * head_chunks, a.num_seqs);
+        decodeTiledKernel<T, Tindex><<<grid, 64, 0, stream>>>(a);
+    } else {
+        launchGeneric<typename T::Base, Tindex>(a, plan, stream);
+    }
+    if (plan.max_partitions > 1) {
+        launchReduce<typename T::Base, Tindex>(a, plan, stream);
+    }
+}
+
+template <typename T>
+infiniStatus_t launchByIndex(infiniDtype_t index_dtype, const DecodeArgs &a, const Plan &plan, bool tiled,
+                             hipStream_t stream) {
+    switch (index_dtype) {
+    case INFINI_DTYPE_I64: launchAll<T, IndexI64>(a, plan, tiled, stream); break;
+    case INFINI_DTYPE_I32: launchAll<T, IndexI32>(a, plan, tiled, stream); break;
+    case INFINI_DTYPE_U32: launchAll<T, IndexU32>(a, plan, tiled, stream); break;
+    default: return INFINI_STATUS_BAD_TENSOR_DTYPE;
+    }
+    return INFINI_STATUS_SUCCESS;
+}
+
+bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+} // namespace
+
+struct Descriptor::Opaque {
+    Plan plan;
+};
+
+Descriptor::~Descriptor() { delete _opaque; }
+
+infiniStatus_t Descriptor::create(infiniopHandle_t handle, Descriptor **desc_ptr, infiniopTensorDescriptor_t out_desc,
+                                  infiniopTensorDescriptor_t q_desc, infiniopTensorDescriptor_t k_cache_desc,
+                                  infiniopTensorDescriptor_t v_cache_desc, infiniopTensorDescriptor_t block_tables_desc,
+                                  infiniopTensorDescriptor_t seq_lens_desc, infiniopTensorDescriptor_t alibi_slopes_desc,
+                                  float scale) {
+    auto info = PagedAttentionInfo::create(out_desc, q_desc, k_cache_desc, v_cache_desc, block_tables_desc,
+                                           seq_lens_desc, alibi_slopes_desc, scale);
+    CHECK_RESULT(info);
+    const PagedAttentionInfo in = info.take();
+    const Plan plan = makePlan(in, device::amd::deviceInfo(handle->device_id));
+    const size_t workspace_bytes = plan.acc_bytes + 2 * plan.ml_bytes;
+    *desc_ptr = new Descriptor(new Opaque{plan}, in, workspace_bytes, handle->device, handle->device_id);
+    return INFINI_STATUS_SUCCESS;
+}
+
+infiniStatus_t Descriptor::calculate(void *workspace, size_t workspace_size, void *out, const void *q,
+                                     const void *k_cache, const void *v_cache, const void *block_tables,
+                                     const void *seq_lens, const void *alibi_slopes, void *stream_) const {
+    const PagedAttentionInfo &in = _info;
+    const Plan &plan = _opaque->plan;
+    if (workspace_size < _workspace_size || (_workspace_size > 0 && workspace == nullptr)) {
+        return INFINI_STATUS_INSUFFICIENT_WORKSPACE;
+    }
+    if (in.num_seqs == 0 || in.num_heads == 0) {
+        return INFINI_STATUS_SUCCESS;
+    }
+    if (out == nullptr || q == nullptr || k_cache == nullptr || v_cache == nullptr || block_tables == nullptr
+        || seq_lens == nullptr) {
+        return INFINI_STATUS_NULL_POINTER;
+    }
+    if (in.has_alibi && alibi_slopes == nullptr) {
+        return INFINI_STATUS_NULL_POINTER;
+    }
+    if (in.max_num_blocks_per_seq == 0 || in.num_blocks == 0) {
+        return INFINI_STATUS_SUCCESS; // no sequence can hold a token
+    }
+
+    DecodeArgs a{};
+    a.out = out;
+    a.q = q;
+    a.k_cache = k_cache;
+    a.v_cache = v_cache;
+    a.block_tables = block_tables;
+    a.seq_lens = seq_lens;
+    a.alibi_slopes = static_cast<const float *>(alibi_slopes);
+    if (plan.max_partitions > 1) {
+        char *ws = static_cast<char *>(workspace);
+        a.part_acc = reinterpret_cast<float *>(ws);
+        a.part_m = reinterpret_cast<float *>(ws + plan.acc_bytes);
+        a.part_l = reinterpret_cast<float *>(ws + plan.acc_bytes + plan.ml_bytes);
+    }
+    a.scale_log2 = in.scale * kLog2e;
+    a.num_seqs = static_cast<int32_t>(in.num_seqs);
+    a.num_heads = static_cast<int32_t>(in.num_heads);
+    a.num_kv_heads = static_cast<int32_t>(in.num_kv_heads);
+    a.group = static_cast<int32_t>(in.num_heads / in.num_kv_heads);
+    a.head_size = static_cast<int32_t>(in.head_size);
+    a.value_size = static_cast<int32_t>(in.value_size);
+    a.block_size = static_cast<int32_t>(in.page_block_size);
+    a.block_shift = -1;
+    if (in.page_block_size > 0 && (in.page_block_size & (in.page_block_size - 1)) == 0) {
+        a.block_shift = __builtin_ctzll(in.page_block_size);
+    }
+    a.num_blocks = static_cast<int32_t>(in.num_blocks > 0x7fffffff ? 0x7fffffff : in.num_blocks);
+    a.max_blocks_per_seq = static_cast<int32_t>(in.max_num_blocks_per_seq);
+    a.partition_tokens = plan.partition_tokens;
+    a.max_partitions = plan.max_partitions;
+    a.q_stride = in.q_stride;
+    a.q_head_stride = in.q_head_stride;
+    a.o_stride = in.o_stride;
+    a.o_head_stride = in.o_head_stride;
+    a.k_batch_stride = in.k_batch_stride;
+    a.k_head_stride = in.k_head_stride;
+    a.k_row_stride = in.k_row_stride;
+    a.v_batch_stride = in.v_batch_stride;
+    a.v_head_stride = in.v_head_stride;
+    a.v_row_stride = in.v_row_stride;
+    a.block_table_batch_stride = in.block_table_batch_stride;
+
+    // The tiled kernel moves 16 bytes per lane; base addresses that are not 16-byte aligned take
+    // the element-wise kernel instead.
+    const bool tiled = plan.tiled && aligned16(out) && aligned16(q) && aligned16(k_cache) && aligned16(v_cache)
+                    && (plan.max_partitions == 1 || aligned16(workspace));
+    auto stream = static_cast<hipStream_t>(stream_);
+
+    infiniStatus_t status;
+    if (in.dtype == INFINI_DTYPE_F16) {
+        status = launchByIndex<TileF16>(in.index_dtype, a, plan, tiled, stream);
+    } else {
+        status = launchByIndex<TileBF16>(in.index_dtype, a, plan, tiled, stream);
+    }
+    if (status != INFINI_STATUS_SUCCESS) {
+        return status;
+    }
+    return hipGetLastError() == hipSuccess ? INFINI_STATUS_SUCCESS : INFINI_STATUS_INTERNAL_ERROR;
+}
+
+} // namespace op::paged_attention::amd

@@ -1,0 +1,191 @@
+// paged_caching on AMD Instinct (gfx950): scatter the K and V vectors of a chunk of tokens into
+// their slots of the paged pool.
+//
+// The operation is a pure byte copy, so the kernel is written for memory transactions, not for
+// elements: a token's (head, vector) rows are moved in the widest power-of-two unit (up to 16
+// bytes) that divides every row length, stride and base address involved. A workgroup is a
+// (chunk lanes) x (heads) x (tokens) box of 256 threads; adjacent lanes move adjacent units of one
+// row, so every wavefront load/store instruction covers whole contiguous rows.
+// Semantics follow the reference kernel src/infiniop/ops/paged_caching/cuda/kernel.cuh:22-89
+// (negative slot = padding, page = slot / block_size, row = slot % block_size, source heads packed).
+#include "paged_caching_amd.h"
+#include "../../../handle.h"
+#include "../../../../utils/check.h"
+#include <cstdint>
+#include <hip/hip_runtime.h>
+
+namespace op::paged_caching::amd {
+
+namespace {
+
+// Everything below is in units of the copy vector (`Unit`), not of elements.
+struct ScatterArgs {
+    void *k_cache;
+    void *v_cache;
+    const void *k;
+    const void *v;
+    const int64_t *slot_mapping;
+    int64_t num_tokens;
+    int64_t num_slots;        // num_blocks * block_size; slots at or beyond it are ignored
+    int32_t num_kv_heads;
+    int32_t block_size;
+    int32_t block_shift;      // log2(block_size) when it is a power of two, else -1
+    int32_t k_units_per_row;  // head_size * element_size / sizeof(Unit)
+    int32_t v_units_per_row;
+    int64_t k_src_token_stride, v_src_token_stride;
+    int64_t k_block_stride, k_head_stride, k_slot_stride;
+    int64_t v_block_stride, v_head_stride, v_slot_stride;
+};
+
+template <typename Unit>
+__global__ void __launch_bounds__(256) pagedCachingScatterKernel(ScatterArgs a) {
+    const int64_t token = static_cast<int64_t>(blockIdx.x) * blockDim.z + threadIdx.z;
+    if (token >= a.num_tokens) {
+        return;
+    }
+    const int64_t slot = a.slot_mapping[token];
+    // Negative = padding (kernel.cuh:61-63). Slots past the pool would be an out-of-bounds write
+    // in the reference; here they are dropped.
+    if (slot < 0 || slot >= a.num_slots) {
+        return;
+    }
+    int64_t page, row;
+    if (a.block_shift >= 0) {
+        page = slot >> a.block_shift;
+        row = slot & (a.block_size - 1);
+    } else if (a.num_slots <= 0x7fffffff) {
+        const uint32_t s = static_cast<uint32_t>(slot), bs = static_cast<uint32_t>(a.block_size);
+        page = s / bs;
+        row = s % bs;
+    } else {
+        page = slot / a.block_size;
+        row = slot % a.block_size;
+    }
+
+    const Unit *k_src = static_cast<const Unit *>(a.k) + token * a.k_src_token_stride;
+    const Unit *v_src = static_cast<const Unit *>(a.v) + token * a.v_src_token_stride;
+    Unit *k_dst = static_cast<Unit *>(a.k_cache) + page * a.k_block_stride + row * a.k_slot_stride;
+    Unit *v_dst = static_cast<Unit *>(a.v_cache) + page * a.v_block_stride + row * a.v_slot_stride;
+
+    for (int head = threadIdx.y; head < a.num_kv_heads; head += blockDim.y) {
+        const Unit *ks = k_src + static_cast<int64_t>(head) * a.k_units_per_row;
+        const Unit *vs = v_src + static_cast<int64_t>(head) * a.v_units_per_row;
+        Unit *kd = k_dst + head * a.k_head_stride;
+        Unit *vd = v_dst + head * a.v_head_stride;
+        for (int c = threadIdx.x; c < a.k_units_per_row; c += blockDim.x) {
+            kd[c] = ks[c];
+        }
+        for (int c = threadIdx.x; c < a.v_units_per_row; c += blockDim.x) {
+            vd[c] = vs[c];
+        }
+    }
+}
+
+int ceilPow2(int x) {
+    int p = 1;
+    while (p < x) {
+        p <<= 1;
+    }
+    return p;
+}
+
+// Largest power of two <= 16 that divides every byte quantity in the list.
+size_t commonUnitBytes(std::initializer_list<uint64_t> byte_quantities) {
+    uint64_t bits = 16;
+    for (uint64_t q : byte_quantities) {
+        bits |= q;
+    }
+    return static_cast<size_t>(bits & (~bits + 1)); // lowest set bit
+}
+
+} // namespace
+
+struct Descriptor::Opaque {};
+
+Descriptor::~Descriptor() { delete _opaque; }
+
+infiniStatus_t Descriptor::create(infiniopHandle_t handle, Descriptor **desc_ptr,
+                                  infiniopTensorDescriptor_t k_cache_desc, infiniopTensorDescriptor_t v_cache_desc,
+                                  infiniopTensorDescriptor_t k_desc, infiniopTensorDescriptor_t v_desc,
+                                  infiniopTensorDescriptor_t slot_mapping_desc) {
+    auto info = PagedCachingInfo::create(k_cache_desc, v_cache_desc, k_desc, v_desc, slot_mapping_desc);
+    CHECK_RESULT(info);
+    // The scatter needs no scratch (reference: nvidia/paged_caching_nvidia.cu:47-49 reports 0 too).
+    *desc_ptr = new Descriptor(new Opaque{}, info.take(), 0, handle->device, handle->device_id);
+    return INFINI_STATUS_SUCCESS;
+}
+
+infiniStatus_t Descriptor::calculate(void *workspace, size_t workspace_size, void *k_cache, void *v_cache,
+                                     const void *k, const void *v, const void *slot_mapping, void *stream_) const {
+    (void)workspace;
+    (void)workspace_size;
+    const PagedCachingInfo &in = _info;
+    if (in.num_tokens == 0 || in.num_kv_heads == 0 || (in.head_size == 0 && in.v_head_size == 0)) {
+        return INFINI_STATUS_SUCCESS;
+    }
+    if (k_cache == nullptr || v_cache == nullptr || k == nullptr || v == nullptr || slot_mapping == nullptr) {
+        return INFINI_STATUS_NULL_POINTER;
+    }
+
+    const uint64_t es = infiniSizeOf(in.dtype);
+    auto bytes = [es](ptrdiff_t elements) { return static_cast<uint64_t>(elements) * es; };
+    const size_t unit = commonUnitBytes({
+        in.head_size * es, in.v_head_size * es,
+        bytes(in.k_src_stride), bytes(in.v_src_stride),
+        bytes(in.k_cache_block_stride), bytes(in.k_cache_head_stride), bytes(in.k_cache_slot_stride),
+        bytes(in.v_cache_block_stride), bytes(in.v_cache_head_stride), bytes(in.v_cache_slot_stride),
+        reinterpret_cast<uint64_t>(k_cache), reinterpret_cast<uint64_t>(v_cache),
+        reinterpret_cast<uint64_t>(k), reinterpret_cast<uint64_t>(v)});
+    if (unit < es) {
+        return INFINI_STATUS_BAD_PARAM; // a base address that is not aligned to the element size
+    }
+    const int64_t per = static_cast<int64_t>(unit / es); // elements per copy unit
+    auto units = [per](ptrdiff_t elements) { return static_cast<int64_t>(elements) / per; };
+
+    ScatterArgs a{};
+    a.k_cache = k_cache;
+    a.v_cache = v_cache;
+    a.k = k;
+    a.v = v;
+    a.slot_mapping = static_cast<const int64_t *>(slot_mapping);
+    a.num_tokens = static_cast<int64_t>(in.num_tokens);
+    a.num_slots = static_cast<int64_t>(in.num_blocks) * static_cast<int64_t>(in.block_size);
+    a.num_kv_heads = static_cast<int32_t>(in.num_kv_heads);
+    a.block_size = static_cast<int32_t>(in.block_size);
+    a.block_shift = -1;
+    if (in.block_size > 0 && (in.block_size & (in.block_size - 1)) == 0) {
+        a.block_shift = __builtin_ctzll(in.block_size);
+    }
+    a.k_units_per_row = static_cast<int32_t>(units(in.head_size));
+    a.v_units_per_row = static_cast<int32_t>(units(in.v_head_size));
+    a.k_src_token_stride = units(in.k_src_stride);
+    a.v_src_token_stride = units(in.v_src_stride);
+    a.k_block_stride = units(in.k_cache_block_stride);
+    a.k_head_stride = units(in.k_cache_head_stride);
+    a.k_slot_stride = units(in.k_cache_slot_stride);
+    a.v_block_stride = units(in.v_cache_block_stride);
+    a.v_head_stride = units(in.v_cache_head_stride);
+    a.v_slot_stride = units(in.v_cache_slot_stride);
+
+    // 256-thread box: x = units along a row, y = heads, z = tokens.
+    const int row_units = a.k_units_per_row > a.v_units_per_row ? a.k_units_per_row : a.v_units_per_row;
+    int bx = ceilPow2(row_units);
+    bx = bx > 64 ? 64 : bx;
+    int by = ceilPow2(a.num_kv_heads);
+    by = by > 256 / bx ? 256 / bx : by;
+    const int bz = 256 / (bx * by);
+    const dim3 block(bx, by, bz);
+    const dim3 grid(static_cast<unsigned>((in.num_tokens + bz - 1) / bz));
+    auto stream = static_cast<hipStream_t>(stream_);
+
+    switch (unit) {
+    case 16: pagedCachingScatterKernel<uint4><<<grid, block, 0, stream>>>(a); break;
+    case 8: pagedCachingScatterKernel<uint2><<<grid, block, 0, stream>>>(a); break;
+    case 4: pagedCachingScatterKernel<uint32_t><<<grid, block, 0, stream>>>(a); break;
+    case 2: pagedCachingScatterKernel<uint16_t><<<grid, block, 0, stream>>>(a); break;
+    default: return INFINI_STATUS_BAD_TENSOR_STRIDES;
+    }
+    return hipGetLastError() == hipSuccess ? INFINI_STATUS_SUCCESS : INFINI_STATUS_INTERNAL_ERROR;
+}
+
+} // namespace op::paged_caching::amd

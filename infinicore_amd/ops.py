@@ -1,0 +1,174 @@
+"""``paged_attention`` / ``paged_caching`` on torch CUDA tensors, executed by ``libinfiniop.so``.
+
+Argument order and meaning are those of the reference's Python operators
+(``python/infinicore/ops/paged_attention.py:5-40``, ``python/infinicore/ops/paged_caching.py:5-21``).
+What the reference's C++ adaptor does between that call and the C API
+(``src/infinicore/ops/paged_attention/paged_attention_infiniop.cc:16-58``: build tensor descriptors,
+fetch or create a cached operator descriptor keyed by the tensors' metadata, allocate a byte
+workspace of the size the descriptor asks for, call the operator on the current stream) is done here
+with torch providing device memory and the stream.
+"""
+from __future__ import annotations
+
+import ctypes
+from collections import OrderedDict
+from ctypes import c_size_t, c_void_p
+
+import torch
+
+from . import libinfiniop as lib
+from .libinfiniop import LIBINFINIOP, InfiniDevice, InfiniDtype, check_error
+
+_TORCH_TO_INFINI = {
+    torch.float16: InfiniDtype.F16,
+    torch.bfloat16: InfiniDtype.BF16,
+    torch.float32: InfiniDtype.F32,
+    torch.int64: InfiniDtype.I64,
+    torch.int32: InfiniDtype.I32,
+    torch.uint32: InfiniDtype.U32,
+    torch.uint8: InfiniDtype.U8,
+}
+
+_PLAN_CACHE_CAPACITY = 100  # the reference keeps a thread-local LRU of 100 descriptors per operator
+_handles: dict[int, object] = {}
+_plans: "OrderedDict[tuple, _Plan]" = OrderedDict()
+
+
+def _device_index(t: torch.Tensor) -> int:
+    if not t.is_cuda:
+        raise ValueError("infinicore_amd.ops works on CUDA (HIP) tensors only; there is no host fallback")
+    return t.device.index if t.device.index is not None else torch.cuda.current_device()
+
+
+def _handle_for(index: int):
+    lib.set_device(InfiniDevice.AMD, index)
+    if index not in _handles:
+        _handles[index] = lib.create_handle()
+    return _handles[index]
+
+
+def _meta(t: torch.Tensor | None):
+    return None if t is None else (t.dtype, tuple(t.shape), tuple(t.stride()))
+
+
+def _describe(t: torch.Tensor):
+    return lib.create_tensor_descriptor(tuple(t.shape), tuple(t.stride()), _TORCH_TO_INFINI[t.dtype])
+
+
+def _ptr(t: torch.Tensor | None):
+    return c_void_p(0) if t is None else c_void_p(t.data_ptr())
+
+
+class _Plan:
+    """An operator descriptor plus its workspace; owns both until evicted from the cache."""
+
+    def __init__(self, descriptor, destroy, workspace_bytes: int, device: torch.device):
+        self.descriptor = descriptor
+        self._destroy = destroy
+        self.workspace_bytes = workspace_bytes
+        self.workspace = torch.empty(workspace_bytes, dtype=torch.uint8, device=device) if workspace_bytes else None
+
+    def close(self):
+        if self.descriptor is not None:
+            check_error(self._destroy(self.descriptor))
+            self.descriptor = None
+
+
+def _cached_plan(key, make):
+    plan = _plans.get(key)
+    if plan is not None:
+        _plans.move_to_end(key)
+        return plan
+    plan = make()
+    _plans[key] = plan
+    if len(_plans) > _PLAN_CACHE_CAPACITY:
+        _, old = _plans.popitem(last=False)
+        old.close()
+    return plan
+
+
+def clear_plan_cache() -> None:
+    while _plans:
+        _, plan = _plans.popitem()
+        plan.close()
+
+
+def _stream_ptr(device_index: int):
+    return c_void_p(torch.cuda.current_stream(device_index).cuda_stream)
+
+
+def paged_attention(q, k_cache, v_cache, block_tables, cache_lens, alibi_slopes=None, scale: float = 1.0, *, out=None):
+    """Decode attention of one query token per sequence over a paged KV pool; returns ``out``.
+
+    q [num_seqs, num_heads, head_size]; k_cache / v_cache [num_blocks, num_kv_heads, block_size, d];
+    block_tables [num_seqs, max_blocks] and cache_lens [num_seqs] int64/int32/uint32.
+    """
+    index = _device_index(q)
+    if out is None:
+        out = torch.empty((*q.shape[:-1], v_cache.shape[-1]), dtype=q.dtype, device=q.device)
+    tensors = (out, q, k_cache, v_cache, block_tables, cache_lens)
+    key = ("paged_attention", index, float(scale), *(_meta(t) for t in tensors), _meta(alibi_slopes))
+
+    def make():
+        handle = _handle_for(index)
+        descs = [_describe(t) for t in tensors]
+        alibi_desc = _describe(alibi_slopes) if alibi_slopes is not None else lib.infiniopTensorDescriptor_t()
+        op = lib.infiniopOperatorDescriptor_t()
+        try:
+            check_error(
+                LIBINFINIOP.infiniopCreatePagedAttentionDescriptor(handle, ctypes.byref(op), *descs, alibi_desc, scale),
+                "infiniopCreatePagedAttentionDescriptor",
+            )
+        finally:
+            for d in descs:
+                lib.destroy_tensor_descriptor(d)
+            if alibi_slopes is not None:
+                lib.destroy_tensor_descriptor(alibi_desc)
+        size = c_size_t(0)
+        check_error(LIBINFINIOP.infiniopGetPagedAttentionWorkspaceSize(op, ctypes.byref(size)))
+        return _Plan(op, LIBINFINIOP.infiniopDestroyPagedAttentionDescriptor, size.value, q.device)
+
+    plan = _cached_plan(key, make)
+    lib.set_device(InfiniDevice.AMD, index)
+    check_error(
+        LIBINFINIOP.infiniopPagedAttention(
+            plan.descriptor, _ptr(plan.workspace), plan.workspace_bytes, _ptr(out), _ptr(q), _ptr(k_cache),
+            _ptr(v_cache), _ptr(block_tables), _ptr(cache_lens), _ptr(alibi_slopes), _stream_ptr(index),
+        ),
+        "infiniopPagedAttention",
+    )
+    return out
+
+
+def paged_caching(k_cache, v_cache, k, v, slot_mapping):
+    """Scatter ``k`` / ``v`` [num_tokens, num_kv_heads, d] into the pools in place; returns the pools."""
+    index = _device_index(k)
+    tensors = (k_cache, v_cache, k, v, slot_mapping)
+    key = ("paged_caching", index, *(_meta(t) for t in tensors))
+
+    def make():
+        handle = _handle_for(index)
+        descs = [_describe(t) for t in tensors]
+        op = lib.infiniopOperatorDescriptor_t()
+        try:
+            check_error(
+                LIBINFINIOP.infiniopCreatePagedCachingDescriptor(handle, ctypes.byref(op), *descs),
+                "infiniopCreatePagedCachingDescriptor",
+            )
+        finally:
+            for d in descs:
+                lib.destroy_tensor_descriptor(d)
+        size = c_size_t(0)
+        check_error(LIBINFINIOP.infiniopGetPagedCachingWorkspaceSize(op, ctypes.byref(size)))
+        return _Plan(op, LIBINFINIOP.infiniopDestroyPagedCachingDescriptor, size.value, k.device)
+
+    plan = _cached_plan(key, make)
+    lib.set_device(InfiniDevice.AMD, index)
+    check_error(
+        LIBINFINIOP.infiniopPagedCaching(
+            plan.descriptor, _ptr(plan.workspace), plan.workspace_bytes, _ptr(k_cache), _ptr(v_cache), _ptr(k),
+            _ptr(v), _ptr(slot_mapping), _stream_ptr(index),
+        ),
+        "infiniopPagedCaching",
+    )
+    return k_cache, v_cache

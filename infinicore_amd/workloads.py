@@ -1,0 +1,152 @@
+"""Seeded synthetic inputs for the paged-KV benchmark configurations (host tensors, torch CPU).
+
+Every generator is a pure function of its seed (numpy PCG64), so the CPU container and the GPU box
+build bit-identical inputs. Shapes follow the five benchmark configurations: a small MHA plumbing
+case, the Llama-3-8B GQA batch-32 decode shape, a long-context peaked-softmax case, a 70B-class
+one-GPU share, and a paged_caching scatter of a prefill chunk.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+
+import numpy as np
+import torch
+
+
+@dataclass
+class DecodeConfig:
+    name: str
+    dtype: torch.dtype
+    num_seqs: int
+    num_heads: int
+    num_kv_heads: int
+    head_size: int
+    block_size: int
+    min_len: int
+    max_len: int
+    spare_block_fraction: float = 0.0  # extra unused pages in the pool
+    peaked_fraction: float = 0.0       # fraction of token positions whose K row is scaled
+    peaked_scale: float = 8.0
+    seed: int = 0
+
+    @property
+    def scale(self) -> float:
+        return 1.0 / float(self.head_size) ** 0.5
+
+
+@dataclass
+class CachingConfig:
+    name: str
+    dtype: torch.dtype
+    num_tokens: int
+    num_kv_heads: int
+    head_size: int
+    block_size: int
+    num_slots: int
+    padding_fraction: float
+    seed: int = 0
+
+
+DECODE_CONFIGS = {
+    "c1_plumbing_mha": DecodeConfig("c1_plumbing_mha", torch.float16, 4, 8, 8, 128, 16, 1, 256, seed=101),
+    "c2_llama3_8b_b32": DecodeConfig("c2_llama3_8b_b32", torch.bfloat16, 32, 32, 8, 128, 16, 512, 4096,
+                                     spare_block_fraction=0.10, seed=102),
+    "c3_long_context": DecodeConfig("c3_long_context", torch.bfloat16, 8, 32, 8, 128, 16, 16384, 32768,
+                                    peaked_fraction=0.01, seed=103),
+    "c4_70b_share_b128": DecodeConfig("c4_70b_share_b128", torch.float16, 128, 64, 8, 128, 16, 1024, 8192, seed=104),
+}
+CACHING_CONFIGS = {
+    "c5_prefill_scatter": CachingConfig("c5_prefill_scatter", torch.bfloat16, 4096, 8, 128, 16, 65536, 0.05, seed=105),
+}
+
+
+@dataclass
+class DecodeInputs:
+    config: DecodeConfig
+    q: torch.Tensor             # [B, H, D]
+    k_cache: torch.Tensor       # [NB, Hkv, bs, D]
+    v_cache: torch.Tensor
+    block_tables: torch.Tensor  # [B, max_blocks] int64, unused entries 0
+    seq_lens: torch.Tensor      # [B] int64
+    scale: float
+    extra: dict = field(default_factory=dict)
+
+
+def _normal(rng: np.random.Generator, shape, dtype: torch.dtype) -> torch.Tensor:
+    return torch.from_numpy(rng.standard_normal(shape, dtype=np.float32)).to(dtype)
+
+
+def draw_seq_lens(cfg: DecodeConfig) -> np.ndarray:
+    rng = np.random.default_rng(cfg.seed)
+    return rng.integers(cfg.min_len, cfg.max_len + 1, size=cfg.num_seqs, dtype=np.int64)
+
+
+def decode_algorithmic_bytes(cfg: DecodeConfig, seq_lens) -> int:
+    """HBM bytes one decode call has to move: K and V once per KV head, Q in, O out, the table
+    entries actually needed (int64) and the lengths."""
+    e = 2
+    lens = np.asarray(seq_lens, dtype=np.int64)
+    kv = int(lens.sum()) * cfg.num_kv_heads * 2 * cfg.head_size * e
+    qo = 2 * cfg.num_seqs * cfg.num_heads * cfg.head_size * e
+    idx = int(((lens + cfg.block_size - 1) // cfg.block_size).sum()) * 8 + cfg.num_seqs * 8
+    return kv + qo + idx
+
+
+def make_decode_inputs(cfg: DecodeConfig, seed_offset: int = 0) -> DecodeInputs:
+    """Pool of exactly the needed pages (plus the spare fraction), pages dealt to sequences by a
+    seeded random permutation, Q/K/V ~ N(0,1) rounded to the storage dtype."""
+    lens = draw_seq_lens(cfg)
+    rng = np.random.default_rng([cfg.seed, 7, seed_offset])
+    blocks_per_seq = (lens + cfg.block_size - 1) // cfg.block_size
+    needed = int(blocks_per_seq.sum())
+    num_blocks = int(np.ceil(needed * (1.0 + cfg.spare_block_fraction)))
+    perm = rng.permutation(num_blocks)[:needed]
+    max_blocks = int(blocks_per_seq.max())
+    table = np.zeros((cfg.num_seqs, max_blocks), dtype=np.int64)
+    cursor = 0
+    for s, nb in enumerate(blocks_per_seq):
+        table[s, :nb] = perm[cursor:cursor + nb]
+        cursor += nb
+
+    q = _normal(rng, (cfg.num_seqs, cfg.num_heads, cfg.head_size), cfg.dtype)
+    cache_shape = (num_blocks, cfg.num_kv_heads, cfg.block_size, cfg.head_size)
+    k_cache = _normal(rng, cache_shape, torch.float32)
+    if cfg.peaked_fraction > 0.0:
+        # scale whole token rows (all KV heads of a position) so the softmax is sharply peaked
+        hot = rng.random((num_blocks, 1, cfg.block_size, 1)) < cfg.peaked_fraction
+        k_cache = k_cache * torch.from_numpy(np.where(hot, cfg.peaked_scale, 1.0).astype(np.float32))
+    k_cache = k_cache.to(cfg.dtype)
+    v_cache = _normal(rng, cache_shape, cfg.dtype)
+    return DecodeInputs(cfg, q, k_cache, v_cache, torch.from_numpy(table), torch.from_numpy(lens), cfg.scale)
+
+
+@dataclass
+class CachingInputs:
+    config: CachingConfig
+    k: torch.Tensor             # [ntok, Hkv, D]
+    v: torch.Tensor
+    k_cache: torch.Tensor       # [NB, Hkv, bs, D], pre-filled with a sentinel pattern
+    v_cache: torch.Tensor
+    slot_mapping: torch.Tensor  # [ntok] int64, -1 = padding
+
+
+def caching_algorithmic_bytes(cfg: CachingConfig, slot_mapping) -> int:
+    e = 2 if cfg.dtype in (torch.float16, torch.bfloat16) else 4
+    valid = int((np.asarray(slot_mapping) >= 0).sum())
+    moved = valid * cfg.num_kv_heads * cfg.head_size * e * 2  # K and V
+    return 2 * moved + cfg.num_tokens * 8  # read + write + slot ids
+
+
+def make_caching_inputs(cfg: CachingConfig) -> CachingInputs:
+    rng = np.random.default_rng([cfg.seed, 11])
+    slots = rng.permutation(cfg.num_slots)[:cfg.num_tokens].astype(np.int64)
+    padding = rng.random(cfg.num_tokens) < cfg.padding_fraction
+    slots[padding] = -1
+    k = _normal(rng, (cfg.num_tokens, cfg.num_kv_heads, cfg.head_size), cfg.dtype)
+    v = _normal(rng, (cfg.num_tokens, cfg.num_kv_heads, cfg.head_size), cfg.dtype)
+    num_blocks = cfg.num_slots // cfg.block_size
+    shape = (num_blocks, cfg.num_kv_heads, cfg.block_size, cfg.head_size)
+    # sentinel: a value no N(0,1) draw rounds to, so untouched bytes are recognisable
+    k_cache = torch.full(shape, -777.0, dtype=cfg.dtype)
+    v_cache = torch.full(shape, 555.0, dtype=cfg.dtype)
+    return CachingInputs(cfg, k, v, k_cache, v_cache, torch.from_numpy(slots))

@@ -1,0 +1,330 @@
+/*
+ * CPU oracle for InfiniOP paged_attention (decode) and paged_caching.
+ *
+ * TEST INFRASTRUCTURE ONLY. This file restates, in plain C, the algorithm of the reference's device
+ * kernels so that the HIP kernels of this repository can be checked against it. Only tests/,
+ * __graft_entry__.smoke() and the cpu_baseline leg of bench.py may load it; the product
+ * (libinfiniop.so) never does and has no CPU path of its own.
+ *
+ * The reference ships no CPU implementation and no golden vectors for these two operators, and its
+ * CUDA sources cannot be compiled here, so the oracle is pinned by mathematics instead (see
+ * tests/test_oracle_pinning.py): an independent fp64 two-pass softmax on gathered K/V, torch's
+ * scaled_dot_product_attention on the gathered sequence, closed forms (length 1, equal V rows,
+ * zero query, one dominant key), invariance under page permutation, GQA == MHA on repeated heads,
+ * split == unsplit, and a byte-exact scatter model for paged_caching.
+ *
+ * Functions and the reference code each one follows:
+ *   oracle_paged_attention         src/infiniop/ops/paged_attention/cuda/kernel_v2.cuh:134-336
+ *                                  (one query head at a time: fp32 dot product, score in the log2
+ *                                  domain, online max/sum softmax with exp2f, out = acc / (l + 1e-6),
+ *                                  round-to-nearest-even to fp16 / bf16; seq_len <= 0 leaves out untouched)
+ *   oracle_paged_attention_splitkv kernel_v2.cuh:340-554 (token shards of ceil(len / splits), partial
+ *                                  (m, l, acc) per shard, empty shard = (-inf, 0, 0)) and :556-616 (combine)
+ *   oracle_paged_caching           src/infiniop/ops/paged_caching/cuda/kernel.cuh:22-89
+ *                                  (slot < 0 skipped, page = slot / block_size, row = slot % block_size,
+ *                                  source heads packed, element-wise copy)
+ *
+ * Build: make -C oracle   (gcc -O2 -fopenmp -shared)
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+#define ORACLE_DTYPE_F16 0
+#define ORACLE_DTYPE_BF16 1
+
+/* ---- storage formats <-> float, round-to-nearest-even ---- */
+
+static float bf16_to_float(uint16_t h) {
+    uint32_t u = (uint32_t)h << 16;
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+}
+
+static uint16_t float_to_bf16(float f) {
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    if ((u & 0x7fffffffu) > 0x7f800000u) {
+        return (uint16_t)((u >> 16) | 0x0040u); /* quiet NaN */
+    }
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+
+static float f16_to_float(uint16_t h) {
+    const uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+    uint32_t exp = (h >> 10) & 0x1fu;
+    uint32_t man = h & 0x3ffu;
+    uint32_t u;
+    if (exp == 0) {
+        if (man == 0) {
+            u = sign;
+        } else { /* subnormal: normalise */
+            int shift = 0;
+            while ((man & 0x400u) == 0) {
+                man <<= 1;
+                ++shift;
+            }
+            man &= 0x3ffu;
+            u = sign | ((uint32_t)(127 - 15 - shift + 1) << 23) | (man << 13);
+        }
+    } else if (exp == 31) {
+        u = sign | 0x7f800000u | (man << 13);
+    } else {
+        u = sign | ((exp + 127 - 15) << 23) | (man << 13);
+    }
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+}
+
+static uint16_t float_to_f16(float f) {
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    const uint16_t sign = (uint16_t)((u >> 16) & 0x8000u);
+    const uint32_t abs = u & 0x7fffffffu;
+    if (abs > 0x7f800000u) {
+        return (uint16_t)(sign | 0x7e00u); /* NaN */
+    }
+    if (abs >= 0x477ff000u) { /* >= 65520 rounds to inf */
+        return (uint16_t)(sign | 0x7c00u);
+    }
+    if (abs < 0x33000001u) { /* <= 2^-25 rounds to zero */
+        return sign;
+    }
+    int32_t exp = (int32_t)(abs >> 23) - 127;
+    uint32_t man = (abs & 0x7fffffu) | 0x800000u; /* 24-bit significand */
+    int shift; /* bits to drop from the 24-bit significand */
+    uint32_t base;
+    if (exp < -14) { /* subnormal half */
+        shift = 13 + (-14 - exp);
+        base = 0;
+    } else {
+        shift = 13;
+        base = ((uint32_t)(exp + 15) << 10) - 0x400u; /* the implicit bit adds the 0x400 back */
+    }
+    uint32_t kept = man >> shift;
+    const uint32_t rem = man & ((1u << shift) - 1u);
+    const uint32_t half = 1u << (shift - 1);
+    if (rem > half || (rem == half && (kept & 1u))) {
+        ++kept;
+    }
+    return (uint16_t)(sign | (base + kept));
+}
+
+static float load_elem(const uint16_t *p, int dtype) {
+    return dtype == ORACLE_DTYPE_F16 ? f16_to_float(*p) : bf16_to_float(*p);
+}
+
+static uint16_t store_elem(float f, int dtype) {
+    return dtype == ORACLE_DTYPE_F16 ? float_to_f16(f) : float_to_bf16(f);
+}
+
+/* exposed so the conversion helpers themselves can be checked against numpy / torch */
+float oracle_to_float(uint16_t bits, int dtype) { return load_elem(&bits, dtype); }
+uint16_t oracle_from_float(float f, int dtype) { return store_elem(f, dtype); }
+
+typedef struct {
+    int dtype; /* ORACLE_DTYPE_* of q, out and both caches */
+    int64_t num_seqs, num_heads, num_kv_heads, head_size, value_size, block_size, max_blocks_per_seq;
+    /* element strides */
+    int64_t q_stride, q_head_stride, o_stride, o_head_stride;
+    int64_t k_batch_stride, k_head_stride, k_row_stride;
+    int64_t v_batch_stride, v_head_stride, v_row_stride;
+    int64_t block_table_stride;
+    float scale;
+} oracle_attention_shape;
+
+static const float kLog2e = 1.4426950408889634f;
+
+/* One query head of one sequence over tokens [t_begin, t_end): the recurrence of
+ * kernel_v2.cuh:223-315. Leaves the un-normalised accumulator in acc[value_size] and returns m, l. */
+static void attend_range(const oracle_attention_shape *s, const uint16_t *q_row, const uint16_t *k_cache,
+                         const uint16_t *v_cache, const int64_t *block_table, int64_t kv_head, float alibi_slope,
+                         int64_t seq_len, int64_t t_begin, int64_t t_end, float *acc, float *m_out, float *l_out) {
+    const float scale_log2 = s->scale * kLog2e;
+    float m = -INFINITY, l = 0.0f;
+    for (int64_t d = 0; d < s->value_size; ++d) {
+        acc[d] = 0.0f;
+    }
+    for (int64_t t = t_begin; t < t_end; ++t) {
+        const int64_t page = block_table[t / s->block_size];
+        const int64_t row = t % s->block_size;
+        const uint16_t *k_row = k_cache + page * s->k_batch_stride + kv_head * s->k_head_stride + row * s->k_row_stride;
+        const uint16_t *v_row = v_cache + page * s->v_batch_stride + kv_head * s->v_head_stride + row * s->v_row_stride;
+
+        float qk = 0.0f;
+        for (int64_t d = 0; d < s->head_size; ++d) {
+            qk += load_elem(q_row + d, s->dtype) * load_elem(k_row + d, s->dtype);
+        }
+        float score = qk * scale_log2;
+        if (alibi_slope != 0.0f) {
+            score += (alibi_slope * (float)(t - (seq_len - 1))) * kLog2e;
+        }
+        const float m_new = fmaxf(m, score);
+        const float alpha = exp2f(m - m_new);
+        const float beta = exp2f(score - m_new);
+        l = l * alpha + beta;
+        m = m_new;
+        for (int64_t d = 0; d < s->value_size; ++d) {
+            acc[d] = acc[d] * alpha + beta * load_elem(v_row + d, s->dtype);
+        }
+    }
+    *m_out = m;
+    *l_out = l;
+}
+
+/* Unsplit decode, kernel_v2.cuh:134-336. Returns 0, or -1 on a bad argument. */
+int oracle_paged_attention(void *out_, const void *q_, const void *k_cache_, const void *v_cache_,
+                           const int64_t *block_tables, const int64_t *seq_lens, const float *alibi_slopes,
+                           const oracle_attention_shape *s, int num_threads) {
+    if (s->num_kv_heads <= 0 || s->num_heads % s->num_kv_heads != 0 || s->block_size <= 0) {
+        return -1;
+    }
+    uint16_t *out = (uint16_t *)out_;
+    const uint16_t *q = (const uint16_t *)q_;
+    const int64_t group = s->num_heads / s->num_kv_heads;
+    const int64_t work = s->num_seqs * s->num_heads;
+    if (num_threads < 1) {
+        num_threads = 1;
+    }
+#pragma omp parallel num_threads(num_threads)
+    {
+        float *acc = (float *)malloc(sizeof(float) * (size_t)(s->value_size > 0 ? s->value_size : 1));
+#pragma omp for schedule(dynamic, 1)
+        for (int64_t w = 0; w < work; ++w) {
+            const int64_t seq = w / s->num_heads, head = w % s->num_heads;
+            const int64_t seq_len = seq_lens[seq];
+            if (seq_len <= 0) {
+                continue; /* :164-167, nothing is written */
+            }
+            float m, l;
+            attend_range(s, q + seq * s->q_stride + head * s->q_head_stride, (const uint16_t *)k_cache_,
+                         (const uint16_t *)v_cache_, block_tables + seq * s->block_table_stride, head / group,
+                         alibi_slopes ? alibi_slopes[head] : 0.0f, seq_len, 0, seq_len, acc, &m, &l);
+            const float inv_l = 1.0f / (l + 1e-6f);
+            uint16_t *o_row = out + seq * s->o_stride + head * s->o_head_stride;
+            for (int64_t d = 0; d < s->value_size; ++d) {
+                o_row[d] = store_elem(acc[d] * inv_l, s->dtype);
+            }
+        }
+        free(acc);
+    }
+    return 0;
+}
+
+/* Split-KV decode and combine, kernel_v2.cuh:340-616: shard i covers tokens
+ * [i * ceil(len / splits), min(len, (i + 1) * ceil(len / splits))). */
+int oracle_paged_attention_splitkv(void *out_, const void *q_, const void *k_cache_, const void *v_cache_,
+                                   const int64_t *block_tables, const int64_t *seq_lens, const float *alibi_slopes,
+                                   const oracle_attention_shape *s, int num_splits, int num_threads) {
+    if (s->num_kv_heads <= 0 || s->num_heads % s->num_kv_heads != 0 || s->block_size <= 0 || num_splits < 1) {
+        return -1;
+    }
+    uint16_t *out = (uint16_t *)out_;
+    const uint16_t *q = (const uint16_t *)q_;
+    const int64_t group = s->num_heads / s->num_kv_heads;
+    const int64_t work = s->num_seqs * s->num_heads;
+    const size_t vs = (size_t)(s->value_size > 0 ? s->value_size : 1);
+    if (num_threads < 1) {
+        num_threads = 1;
+    }
+#pragma omp parallel num_threads(num_threads)
+    {
+        float *part_acc = (float *)malloc(sizeof(float) * vs * (size_t)num_splits);
+        float *part_m = (float *)malloc(sizeof(float) * (size_t)num_splits);
+        float *part_l = (float *)malloc(sizeof(float) * (size_t)num_splits);
+#pragma omp for schedule(dynamic, 1)
+        for (int64_t w = 0; w < work; ++w) {
+            const int64_t seq = w / s->num_heads, head = w % s->num_heads;
+            const int64_t seq_len = seq_lens[seq];
+            if (seq_len <= 0) {
+                continue;
+            }
+            const int64_t shard = (seq_len + num_splits - 1) / num_splits;
+            for (int i = 0; i < num_splits; ++i) {
+                const int64_t t0 = (int64_t)i * shard;
+                const int64_t t1 = t0 + shard < seq_len ? t0 + shard : seq_len;
+                if (t0 >= t1) { /* empty shard, :676-693 */
+                    part_m[i] = -INFINITY;
+                    part_l[i] = 0.0f;
+                    for (size_t d = 0; d < vs; ++d) {
+                        part_acc[(size_t)i * vs + d] = 0.0f;
+                    }
+                    continue;
+                }
+                attend_range(s, q + seq * s->q_stride + head * s->q_head_stride, (const uint16_t *)k_cache_,
+                             (const uint16_t *)v_cache_, block_tables + seq * s->block_table_stride, head / group,
+                             alibi_slopes ? alibi_slopes[head] : 0.0f, seq_len, t0, t1, part_acc + (size_t)i * vs,
+                             &part_m[i], &part_l[i]);
+            }
+            /* combine, :574-614 */
+            float m = -INFINITY;
+            for (int i = 0; i < num_splits; ++i) {
+                m = fmaxf(m, part_m[i]);
+            }
+            float l = 0.0f;
+            for (int i = 0; i < num_splits; ++i) {
+                if (part_l[i] > 0.0f) {
+                    l += part_l[i] * exp2f(part_m[i] - m);
+                }
+            }
+            const float inv_l = 1.0f / (l + 1e-6f);
+            uint16_t *o_row = out + seq * s->o_stride + head * s->o_head_stride;
+            for (int64_t d = 0; d < s->value_size; ++d) {
+                float acc = 0.0f;
+                for (int i = 0; i < num_splits; ++i) {
+                    acc += part_acc[(size_t)i * vs + (size_t)d] * exp2f(part_m[i] - m);
+                }
+                o_row[d] = store_elem(acc * inv_l, s->dtype);
+            }
+        }
+        free(part_acc);
+        free(part_m);
+        free(part_l);
+    }
+    return 0;
+}
+
+typedef struct {
+    int64_t elem_size; /* bytes per element: 2 (fp16 / bf16) or 4 (fp32) */
+    int64_t num_tokens, num_kv_heads, head_size, v_head_size, block_size;
+    /* element strides */
+    int64_t k_src_stride, v_src_stride;
+    int64_t k_cache_block_stride, v_cache_block_stride;
+    int64_t k_cache_head_stride, v_cache_head_stride;
+    int64_t k_cache_slot_stride, v_cache_slot_stride;
+} oracle_caching_shape;
+
+/* Slot scatter, paged_caching/cuda/kernel.cuh:52-88. */
+int oracle_paged_caching(void *k_cache_, void *v_cache_, const void *k_, const void *v_, const int64_t *slot_mapping,
+                         const oracle_caching_shape *s) {
+    if (s->block_size <= 0 || (s->elem_size != 2 && s->elem_size != 4)) {
+        return -1;
+    }
+    char *k_cache = (char *)k_cache_, *v_cache = (char *)v_cache_;
+    const char *k = (const char *)k_, *v = (const char *)v_;
+    const int64_t es = s->elem_size;
+    for (int64_t tok = 0; tok < s->num_tokens; ++tok) {
+        const int64_t slot = slot_mapping[tok];
+        if (slot < 0) {
+            continue; /* padding, :61-63 */
+        }
+        const int64_t page = slot / s->block_size, row = slot % s->block_size;
+        for (int64_t head = 0; head < s->num_kv_heads; ++head) {
+            const char *k_src = k + (tok * s->k_src_stride + head * s->head_size) * es;
+            const char *v_src = v + (tok * s->v_src_stride + head * s->v_head_size) * es;
+            char *k_dst = k_cache + (page * s->k_cache_block_stride + head * s->k_cache_head_stride + row * s->k_cache_slot_stride) * es;
+            char *v_dst = v_cache + (page * s->v_cache_block_stride + head * s->v_cache_head_stride + row * s->v_cache_slot_stride) * es;
+            for (int64_t i = 0; i < s->head_size; ++i) {
+                memcpy(k_dst + i * es, k_src + i * es, (size_t)es);
+            }
+            for (int64_t i = 0; i < s->v_head_size; ++i) {
+                memcpy(v_dst + i * es, v_src + i * es, (size_t)es);
+            }
+        }
+    }
+    return 0;
+}

@@ -1,0 +1,96 @@
+"""Helpers that drive the operators through the raw C ABI the way the reference's ctypes tests do
+(test/infiniop/paged_attention.py:185-263, test/infiniop/paged_caching.py:160-232): build tensor
+descriptors, create the operator descriptor, query the workspace, destroy the tensor descriptors
+BEFORE running (the operator must own its metadata), run on the NULL stream, synchronise."""
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_size_t, c_void_p
+
+import torch
+
+from infinicore_amd import libinfiniop as L
+
+TORCH_TO_INFINI = {
+    torch.float16: L.InfiniDtype.F16,
+    torch.bfloat16: L.InfiniDtype.BF16,
+    torch.float32: L.InfiniDtype.F32,
+    torch.int64: L.InfiniDtype.I64,
+    torch.int32: L.InfiniDtype.I32,
+    torch.uint32: L.InfiniDtype.U32,
+}
+
+
+def describe(t: torch.Tensor, dtype=None):
+    return L.create_tensor_descriptor(tuple(t.shape), tuple(t.stride()), dtype or TORCH_TO_INFINI[t.dtype])
+
+
+def ptr(t):
+    return c_void_p(0) if t is None else c_void_p(t.data_ptr())
+
+
+def create_paged_attention(handle, out, q, k_cache, v_cache, block_tables, seq_lens, alibi, scale):
+    """Returns (status, descriptor). Tensor descriptors are destroyed before returning."""
+    descs = [describe(t) for t in (out, q, k_cache, v_cache, block_tables, seq_lens)]
+    alibi_desc = describe(alibi) if alibi is not None else L.infiniopTensorDescriptor_t()
+    op = L.infiniopOperatorDescriptor_t()
+    status = L.LIBINFINIOP.infiniopCreatePagedAttentionDescriptor(handle, ctypes.byref(op), *descs, alibi_desc, scale)
+    for d in descs:
+        L.destroy_tensor_descriptor(d)
+    if alibi is not None:
+        L.destroy_tensor_descriptor(alibi_desc)
+    return status, op
+
+
+def workspace_size_attention(op) -> int:
+    size = c_size_t(0)
+    L.check_error(L.LIBINFINIOP.infiniopGetPagedAttentionWorkspaceSize(op, ctypes.byref(size)))
+    return size.value
+
+
+def run_paged_attention(handle, q, k_cache, v_cache, block_tables, seq_lens, scale, alibi=None, out=None,
+                        stream=None, workspace_fill=1):
+    """Full create / query / run / destroy cycle on device tensors; returns ``out``."""
+    if out is None:
+        out = torch.zeros((*q.shape[:-1], v_cache.shape[-1]), dtype=q.dtype, device=q.device)
+    status, op = create_paged_attention(handle, out, q, k_cache, v_cache, block_tables, seq_lens, alibi, scale)
+    L.check_error(status, "infiniopCreatePagedAttentionDescriptor")
+    size = workspace_size_attention(op)
+    # the reference harness hands over a workspace of ones (TestWorkspace); content must not matter
+    workspace = torch.full((max(size, 1),), workspace_fill, dtype=torch.uint8, device=q.device)
+    torch.cuda.synchronize()
+    L.check_error(
+        L.LIBINFINIOP.infiniopPagedAttention(op, ptr(workspace), size, ptr(out), ptr(q), ptr(k_cache), ptr(v_cache),
+                                             ptr(block_tables), ptr(seq_lens), ptr(alibi), c_void_p(stream or 0)),
+        "infiniopPagedAttention",
+    )
+    torch.cuda.synchronize()
+    L.check_error(L.LIBINFINIOP.infiniopDestroyPagedAttentionDescriptor(op))
+    return out
+
+
+def create_paged_caching(handle, k_cache, v_cache, k, v, slot_mapping):
+    descs = [describe(t) for t in (k_cache, v_cache, k, v, slot_mapping)]
+    op = L.infiniopOperatorDescriptor_t()
+    status = L.LIBINFINIOP.infiniopCreatePagedCachingDescriptor(handle, ctypes.byref(op), *descs)
+    for d in descs:
+        L.destroy_tensor_descriptor(d)
+    return status, op
+
+
+def run_paged_caching(handle, k_cache, v_cache, k, v, slot_mapping, stream=None):
+    """In place on the device pools; returns them."""
+    status, op = create_paged_caching(handle, k_cache, v_cache, k, v, slot_mapping)
+    L.check_error(status, "infiniopCreatePagedCachingDescriptor")
+    size = c_size_t(123)
+    L.check_error(L.LIBINFINIOP.infiniopGetPagedCachingWorkspaceSize(op, ctypes.byref(size)))
+    assert size.value == 0
+    torch.cuda.synchronize()
+    L.check_error(
+        L.LIBINFINIOP.infiniopPagedCaching(op, c_void_p(0), 0, ptr(k_cache), ptr(v_cache), ptr(k), ptr(v),
+                                           ptr(slot_mapping), c_void_p(stream or 0)),
+        "infiniopPagedCaching",
+    )
+    torch.cuda.synchronize()
+    L.check_error(L.LIBINFINIOP.infiniopDestroyPagedCachingDescriptor(op))
+    return k_cache, v_cache
