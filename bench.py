@@ -1,0 +1,218 @@
+#!/usr/bin/env python3
+"""Paged-attention decode benchmark on one MI355X.
+
+A step is one ``infiniopPagedAttention`` call (decode kernel + partition merge) through the C ABI on
+the Llama-3-8B GQA batch-32 decode shape (bf16, 32 query / 8 KV heads, head 128, pages of 16
+tokens, ragged lengths 512..4096 through a shuffled block table). Inputs are resident in HBM before
+the timed region. Consecutive steps read different KV pools (same content, different addresses,
+together far larger than the 256 MiB last-level cache), so every step streams its K/V from HBM as a
+real model does when it moves from layer to layer.
+
+Prints one JSON line: throughput in algorithmic GB/s (K and V once per KV head + Q + O + the
+needed table entries + lengths), the time per call, the HBM roofline of the step measured with
+device events on the stream the kernels run on, and a CPU baseline (the CPU oracle, a C restatement
+of the reference kernel's arithmetic, timed on this machine's host cores).
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+from ctypes import c_float, c_size_t, c_void_p
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+
+HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=400)
+    ap.add_argument("--warmup", type=int, default=40)
+    ap.add_argument("--workload", default="c2_llama3_8b_b32")
+    ap.add_argument("--pools", type=int, default=4, help="distinct KV pools the steps rotate over")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-check", action="store_true", help="skip the oracle check of the output")
+    return ap.parse_args()
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py: this path runs on ONE GPU (no collective on it); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from infinicore_amd import libinfiniop as L
+    from infinicore_amd import workloads
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the HIP path has no CPU fallback", file=sys.stderr)
+        sys.exit(3)
+    dev = torch.device("cuda:0")
+    cfg = workloads.DECODE_CONFIGS[args.workload]
+    inp = workloads.make_decode_inputs(cfg)
+    algo_bytes = workloads.decode_algorithmic_bytes(cfg, inp.seq_lens.numpy())
+
+    L.set_device(L.InfiniDevice.AMD, 0)
+    handle = L.create_handle()
+
+    q = inp.q.to(dev)
+    bt = inp.block_tables.to(dev)
+    sl = inp.seq_lens.to(dev)
+    k_pools = [inp.k_cache.to(dev)]
+    v_pools = [inp.v_cache.to(dev)]
+    for _ in range(1, max(1, args.pools)):
+        k_pools.append(k_pools[0].clone())
+        v_pools.append(v_pools[0].clone())
+    out = torch.zeros_like(q)
+
+    # descriptor + workspace, exactly as a caller of the C API does it
+    def describe(t):
+        return L.create_tensor_descriptor(tuple(t.shape), tuple(t.stride()), DTYPES[t.dtype])
+
+    DTYPES = {torch.float16: L.InfiniDtype.F16, torch.bfloat16: L.InfiniDtype.BF16, torch.int64: L.InfiniDtype.I64}
+    descs = [describe(t) for t in (out, q, k_pools[0], v_pools[0], bt, sl)]
+    op = L.infiniopOperatorDescriptor_t()
+    L.check_error(L.LIBINFINIOP.infiniopCreatePagedAttentionDescriptor(
+        handle, ctypes.byref(op), *descs, L.infiniopTensorDescriptor_t(), inp.scale))
+    for d in descs:
+        L.destroy_tensor_descriptor(d)
+    ws_size = c_size_t(0)
+    L.check_error(L.LIBINFINIOP.infiniopGetPagedAttentionWorkspaceSize(op, ctypes.byref(ws_size)))
+    workspace = torch.empty(max(ws_size.value, 1), dtype=torch.uint8, device=dev)
+
+    stream = c_void_p()
+    L.check_error(L.LIBINFINIRT.infinirtStreamCreate(ctypes.byref(stream)))
+    ev0, ev1 = c_void_p(), c_void_p()
+    L.check_error(L.LIBINFINIRT.infinirtEventCreate(ctypes.byref(ev0)))
+    L.check_error(L.LIBINFINIRT.infinirtEventCreate(ctypes.byref(ev1)))
+
+    def step(i):
+        p = i % len(k_pools)
+        L.check_error(L.LIBINFINIOP.infiniopPagedAttention(
+            op, c_void_p(workspace.data_ptr()), ws_size.value, c_void_p(out.data_ptr()), c_void_p(q.data_ptr()),
+            c_void_p(k_pools[p].data_ptr()), c_void_p(v_pools[p].data_ptr()), c_void_p(bt.data_ptr()),
+            c_void_p(sl.data_ptr()), c_void_p(0), stream))
+
+    torch.cuda.synchronize()
+    for i in range(args.warmup):
+        step(i)
+    L.check_error(L.LIBINFINIRT.infinirtStreamSynchronize(stream))
+    torch.cuda.synchronize()
+
+    t0 = time.perf_counter()
+    L.check_error(L.LIBINFINIRT.infinirtEventRecord(ev0, stream))
+    for i in range(args.steps):
+        step(i)
+    L.check_error(L.LIBINFINIRT.infinirtEventRecord(ev1, stream))
+    L.check_error(L.LIBINFINIRT.infinirtStreamSynchronize(stream))
+    torch.cuda.synchronize()
+    wall_s = time.perf_counter() - t0
+    ms = c_float(0)
+    L.check_error(L.LIBINFINIRT.infinirtEventElapsedTime(ctypes.byref(ms), ev0, ev1))
+
+    us_wall = wall_s / args.steps * 1e6
+    us_dev = ms.value / args.steps * 1e3           # device time per call on the kernels' stream
+    gbps_wall = algo_bytes / (us_wall * 1e-6) / 1e9
+    gbps_dev = algo_bytes / (us_dev * 1e-6) / 1e9
+
+    result = {
+        "metric": "PagedAttn decode achieved HBM GB/s (algorithmic bytes / time per call), 8B-GQA b=32, 1 GPU",
+        "value": round(gbps_wall, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(us_wall / 1e3, 6),
+        "us_per_call": round(us_wall, 2),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16" if cfg.dtype == torch.bfloat16 else "f16",
+        "data": "synthetic",
+        "config": {
+            "workload": cfg.name,
+            "num_seqs": cfg.num_seqs, "num_heads": cfg.num_heads, "num_kv_heads": cfg.num_kv_heads,
+            "head_size": cfg.head_size, "block_size": cfg.block_size,
+            "seq_lens": f"uniform[{cfg.min_len},{cfg.max_len}] sum={int(inp.seq_lens.sum())}",
+            "kv_pools_rotated": len(k_pools),
+            "algorithmic_bytes_per_call": algo_bytes,
+        },
+        "roofline": {
+            "bound": "hbm",
+            "achieved": round(gbps_dev, 1),
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": round(gbps_dev / HBM_PEAK_GBPS, 4),
+            "traffic": None,
+            "us_per_call_device": round(us_dev, 2),
+            "note": "device events bracket the whole call: decode kernel + partition-merge kernel",
+        },
+    }
+
+    if not args.no_check:
+        # not timed: one more call on pool 0, compared with the CPU oracle
+        from oracle import paged_oracle
+
+        step(0)
+        L.check_error(L.LIBINFINIRT.infinirtStreamSynchronize(stream))
+        want = paged_oracle.paged_attention(inp.q, inp.k_cache, inp.v_cache, inp.block_tables, inp.seq_lens,
+                                            inp.scale, num_threads=min(16, os.cpu_count() or 1))
+        err = (out.float().cpu() - want.float()).abs()
+        ok = bool((err <= 1e-2 + 2e-3 * want.float().abs()).all())
+        result["parity"] = {"max_abs_err": float(err.max()), "within_atol1e-2_rtol2e-3": ok}
+        if not ok:
+            print(json.dumps(result))
+            print("bench.py: output does not match the oracle", file=sys.stderr)
+            sys.exit(4)
+
+    if not args.no_cpu_baseline:
+        from oracle import paged_oracle
+
+        threads = min(16, os.cpu_count() or 1)
+        paged_oracle.paged_attention(inp.q, inp.k_cache, inp.v_cache, inp.block_tables, inp.seq_lens, inp.scale,
+                                     num_threads=threads)
+        reps, t0 = 0, time.perf_counter()
+        while reps < 50 and time.perf_counter() - t0 < 12.0:
+            paged_oracle.paged_attention(inp.q, inp.k_cache, inp.v_cache, inp.block_tables, inp.seq_lens, inp.scale,
+                                         num_threads=threads)
+            reps += 1
+        cpu_s = (time.perf_counter() - t0) / reps
+        result["cpu_baseline"] = {
+            "value": round(algo_bytes / cpu_s / 1e9, 3),
+            "unit": "GB/s",
+            "cores": threads,
+            "kind": "port",
+            "sample": f"{reps} full calls of the same workload through the C oracle (OpenMP over sequence x head), "
+                      f"{cpu_s * 1e3:.1f} ms per call",
+            "us_per_call": round(cpu_s * 1e6, 1),
+        }
+        # the torch statement the reference's own test uses as expected value (vectorised gather), one call
+        torch.set_num_threads(threads)
+        t0 = time.perf_counter()
+        paged_oracle.torch_reference_attention(inp.q, inp.k_cache, inp.v_cache, inp.block_tables, inp.seq_lens, inp.scale)
+        torch_s = time.perf_counter() - t0
+        result["cpu_baseline_torch"] = {
+            "value": round(algo_bytes / torch_s / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+            "sample": "1 full call of the reference test's torch formulation (vectorised gather) on CPU",
+            "us_per_call": round(torch_s * 1e6, 1),
+        }
+
+    print(json.dumps(result))
+    L.check_error(L.LIBINFINIOP.infiniopDestroyPagedAttentionDescriptor(op))
+    L.check_error(L.LIBINFINIRT.infinirtEventDestroy(ev0))
+    L.check_error(L.LIBINFINIRT.infinirtEventDestroy(ev1))
+    L.check_error(L.LIBINFINIRT.infinirtStreamDestroy(stream))
+    L.destroy_handle(handle)
+
+
+if __name__ == "__main__":
+    main()

@@ -12,7 +12,7 @@
 //   * V needs no LDS: the lane that loads rows 4g..4g+3 of one 8-column strip is the lane that feeds
 //     those four tokens to the matrix instruction; four rows are interleaved per column with byte
 //     permutes.
-//   * the loads of tile t+1 are issued before tile t is computed; page ids of the whole partition
+//   * the loads of tiles t+1 and t+2 are in flight while tile t is computed; page ids of the whole partition
 //     are fetched with one coalesced load up front, so no load address depends on a load in the loop.
 //
 // Arithmetic per tile, with lane = 16*g + c (g = 0..3, c = 0..15):
@@ -82,10 +82,121 @@ constexpr int kTileTokens = 16;     // tokens per tile = rows of one matrix inst
 constexpr int kTiledHead = 128;     // head_size = value_size handled by this kernel
 constexpr int kHeadsPerWave = 16;   // query heads of one KV head packed into one wavefront
 
+// K and V rows of one 16-token tile as they come out of the global loads; kept in registers.
 struct TileRegs {
-    uint4 k[4]; // k[j]: token row 4j+g, columns 8c..8c+7
-    uint4 v[4]; // v[j]: token row 4g+j, columns 8c..8c+7
+    uint4 k0, k1, k2, k3; // k<j>: token row 4j+g, columns 8c..8c+7
+    uint4 v0, v1, v2, v3; // v<j>: token row 4g+j, columns 8c..8c+7
 };
+
+// 16-byte load from (wave-uniform base) + (32-bit per-lane byte offset). The empty asm keeps the
+// offset a value defined where it is used, so that instruction selection sees "scalar base +
+// zero-extended lane offset" and emits the scalar-base form of the load, which needs no vector
+// registers for addresses.
+__device__ __forceinline__ uint4 loadLane16(const char *uniform_base, uint32_t lane_offset) {
+    asm volatile("" : "+v"(lane_offset));
+    return *reinterpret_cast<const uint4 *>(uniform_base + lane_offset);
+}
+
+// max over the four lanes {c, c+16, c+32, c+48}; every one of them gets the result (two lane swaps,
+// no LDS traffic)
+__device__ __forceinline__ float maxAcrossTokenGroups(float x) {
+    typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+    u32x2 r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    x = fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+    r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float sumAcrossTokenGroups(float x) {
+    typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+    u32x2 r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    x = __uint_as_float(r[0]) + __uint_as_float(r[1]);
+    r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
+// Softmax state of one wavefront. o[e][r] = O[head 4g+r of the chunk][column 8c+e].
+struct TileState {
+    f32x4 o[8];
+    float m; // running maximum of head c (same value in the four lanes g = 0..3)
+    float l; // sum of rounded probabilities of head c over this lane's tokens only
+};
+
+// One tile: scores, online softmax, accumulate. `valid` = tokens of the tile that belong to the
+// sequence (16 except possibly in the last tile).
+template <typename T>
+__device__ __forceinline__ void computeTile(TileState &st, const TileRegs r, const uint4 (&q_reg)[4], uint4 *k_lds,
+                                            int c, int g, float scale_log2, float slope, int rel_pos0, int valid) {
+    // K: registers -> swizzled LDS -> matrix-operand layout (token c, columns 32*kk + 8g .. +7)
+    k_lds[(g) * 16 + (c ^ (g))] = r.k0;
+    k_lds[(4 + g) * 16 + (c ^ (4 + g))] = r.k1;
+    k_lds[(8 + g) * 16 + (c ^ (8 + g))] = r.k2;
+    k_lds[(12 + g) * 16 + (c ^ (12 + g))] = r.k3;
+    __builtin_amdgcn_wave_barrier();
+    f32x4 s = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+        s = T::mfmaK32(k_lds[c * 16 + ((4 * kk + g) ^ c)], q_reg[kk], s);
+    }
+    __builtin_amdgcn_wave_barrier();
+
+    // scores of head c for tokens 4g + rr of the tile, log2 domain; rel_pos0 = position of the
+    // tile's first token relative to the last token of the sequence (ALiBi distance)
+    const bool tail = valid < kTileTokens;
+    float sc[4];
+#pragma unroll
+    for (int rr = 0; rr < 4; ++rr) {
+        sc[rr] = s[rr] * scale_log2 + slope * static_cast<float>(rel_pos0 + 4 * g + rr);
+        sc[rr] = (tail && 4 * g + rr >= valid) ? -INFINITY : sc[rr];
+    }
+    const float mx = maxAcrossTokenGroups(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])));
+    const float m_new = fmaxf(st.m, mx);
+
+    if (__builtin_amdgcn_ballot_w64(m_new > st.m) != 0) {
+        // some head's maximum moved: rescale. Lane holds accumulators of heads 4g..4g+3, whose
+        // factors live in lanes 4g..4g+3.
+        const float alpha = fastExp2(st.m - m_new);
+        st.l *= alpha;
+        st.m = m_new;
+#pragma unroll
+        for (int rr = 0; rr < 4; ++rr) {
+            const float alpha_r = __shfl(alpha, 4 * g + rr, 64);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                st.o[e][rr] *= alpha_r;
+            }
+        }
+    }
+
+    // probabilities, rounded to the storage dtype: A operand of P.V
+    uint2 p_op;
+    p_op.x = T::pack2(fastExp2(sc[0] - st.m), fastExp2(sc[1] - st.m));
+    p_op.y = T::pack2(fastExp2(sc[2] - st.m), fastExp2(sc[3] - st.m));
+    st.l += (T::unpackLo(p_op.x) + T::unpackHi(p_op.x)) + (T::unpackLo(p_op.y) + T::unpackHi(p_op.y));
+
+    // V rows beyond the sequence may hold anything (NaN included) and 0 * NaN is NaN: zero them.
+    typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+    u32x4 v0 = __builtin_bit_cast(u32x4, r.v0), v1 = __builtin_bit_cast(u32x4, r.v1);
+    u32x4 v2 = __builtin_bit_cast(u32x4, r.v2), v3 = __builtin_bit_cast(u32x4, r.v3);
+    if (tail) {
+        const u32x4 zero = {0u, 0u, 0u, 0u};
+        v0 = (4 * g + 0 >= valid) ? zero : v0;
+        v1 = (4 * g + 1 >= valid) ? zero : v1;
+        v2 = (4 * g + 2 >= valid) ? zero : v2;
+        v3 = (4 * g + 3 >= valid) ? zero : v3;
+    }
+
+    // O += P . V, one 16-column output tile per e: column 8c+e of rows 4g..4g+3
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+        uint2 even, odd;
+        even.x = __builtin_amdgcn_perm(v1[w], v0[w], 0x05040100u);
+        even.y = __builtin_amdgcn_perm(v3[w], v2[w], 0x05040100u);
+        odd.x = __builtin_amdgcn_perm(v1[w], v0[w], 0x07060302u);
+        odd.y = __builtin_amdgcn_perm(v3[w], v2[w], 0x07060302u);
+        st.o[2 * w] = T::mfmaK16(p_op, even, st.o[2 * w]);
+        st.o[2 * w + 1] = T::mfmaK16(p_op, odd, st.o[2 * w + 1]);
+    }
+}
 
 template <typename T, typename Tindex>
 __global__ void __launch_bounds__(64) decodeTiledKernel(DecodeArgs a) {
@@ -137,145 +248,84 @@ __global__ void __launch_bounds__(64) decodeTiledKernel(DecodeArgs a) {
     }
     const float slope = (a.alibi_slopes != nullptr && head_valid) ? a.alibi_slopes[head] * kLog2e : 0.0f;
 
-    const S *k_head = static_cast<const S *>(a.k_cache) + kv_head * a.k_head_stride;
-    const S *v_head = static_cast<const S *>(a.v_cache) + kv_head * a.v_head_stride;
+    const char *k_head = reinterpret_cast<const char *>(static_cast<const S *>(a.k_cache) + kv_head * a.k_head_stride);
+    const char *v_head = reinterpret_cast<const char *>(static_cast<const S *>(a.v_cache) + kv_head * a.v_head_stride);
     const int block_mask = a.block_size - 1;
+    // Byte offsets of this lane's eight 16-byte pieces inside a tile. They do not change from tile
+    // to tile, so a tile's loads are "wave-uniform tile address + constant lane offset" and need no
+    // per-tile vector address arithmetic.
+    const uint32_t k_row_bytes = static_cast<uint32_t>(a.k_row_stride) * sizeof(S);
+    const uint32_t v_row_bytes = static_cast<uint32_t>(a.v_row_stride) * sizeof(S);
+    uint32_t k_off[4], v_off[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        k_off[j] = (4 * j + g) * k_row_bytes + 16 * c;
+        v_off[j] = (4 * g + j) * v_row_bytes + 16 * c;
+    }
 
-    auto loadTile = [&](int t, TileRegs &r) {
-        const int tok0 = start + t * kTileTokens;
+    // Tile indices past the end of the partition are clamped to the last tile: the loop body stays
+    // branch-free with a fixed number of loads in flight, and the repeated loads hit in cache.
+    auto loadTile = [&](int t) -> TileRegs {
+        const int tok0 = start + min(t, n_tiles - 1) * kTileTokens;
         const int page = __builtin_amdgcn_readlane(page_ids, (tok0 >> a.block_shift) - first_entry);
         const int row0 = tok0 & block_mask;
-        const S *k_tile = k_head + page * a.k_batch_stride + row0 * a.k_row_stride;
-        const S *v_tile = v_head + page * a.v_batch_stride + row0 * a.v_row_stride;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            r.k[j] = *reinterpret_cast<const uint4 *>(k_tile + (4 * j + g) * a.k_row_stride + 8 * c);
-        }
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            r.v[j] = *reinterpret_cast<const uint4 *>(v_tile + (4 * g + j) * a.v_row_stride + 8 * c);
-        }
+        const char *k_tile = k_head + (page * a.k_batch_stride + row0 * a.k_row_stride) * static_cast<int64_t>(sizeof(S));
+        const char *v_tile = v_head + (page * a.v_batch_stride + row0 * a.v_row_stride) * static_cast<int64_t>(sizeof(S));
+        TileRegs r;
+        r.k0 = loadLane16(k_tile, k_off[0]);
+        r.k1 = loadLane16(k_tile, k_off[1]);
+        r.k2 = loadLane16(k_tile, k_off[2]);
+        r.k3 = loadLane16(k_tile, k_off[3]);
+        r.v0 = loadLane16(v_tile, v_off[0]);
+        r.v1 = loadLane16(v_tile, v_off[1]);
+        r.v2 = loadLane16(v_tile, v_off[2]);
+        r.v3 = loadLane16(v_tile, v_off[3]);
+        return r;
     };
 
-    f32x4 o_acc[8]; // o_acc[e][r] = O[head 4g+r of the chunk][column 8c+e]
+    TileState st;
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-        o_acc[e] = f32x4{0.f, 0.f, 0.f, 0.f};
+        st.o[e] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
-    float m_run = -INFINITY; // running maximum of head c (same value in the four lanes g = 0..3)
-    float l_run = 0.0f;      // sum of rounded probabilities of head c over this lane's tokens only
+    st.m = -INFINITY;
+    st.l = 0.0f;
 
-    auto computeTile = [&](int t, TileRegs &r) {
+    auto compute = [&](int t, const TileRegs &r) {
         const int tok0 = start + t * kTileTokens;
-
-        // K: registers -> swizzled LDS -> matrix-operand layout (token c, columns 32*kk + 8g .. +7)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int row = 4 * j + g;
-            k_lds[row * 16 + (c ^ row)] = r.k[j];
-        }
-        __builtin_amdgcn_wave_barrier();
-        f32x4 s = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int kk = 0; kk < 4; ++kk) {
-            const uint4 k_op = k_lds[c * 16 + ((4 * kk + g) ^ c)];
-            s = T::mfmaK32(k_op, q_reg[kk], s);
-        }
-        __builtin_amdgcn_wave_barrier();
-
-        // scores of head c for tokens tok0 + 4g + r, log2 domain
-        float sc[4];
-        const bool tail = tok0 + kTileTokens > end;
-#pragma unroll
-        for (int rr = 0; rr < 4; ++rr) {
-            const int tok = tok0 + 4 * g + rr;
-            sc[rr] = s[rr] * a.scale_log2 + slope * static_cast<float>(tok - (len - 1));
-            if (tail && tok >= end) {
-                sc[rr] = -INFINITY;
-            }
-        }
-        float mx = fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3]));
-        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-        const float m_new = fmaxf(m_run, mx);
-
-        if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0) {
-            // some head's maximum moved: rescale. Lane holds accumulators of heads 4g..4g+3, whose
-            // factors live in lanes 4g..4g+3.
-            const float alpha = fastExp2(m_run - m_new);
-            l_run *= alpha;
-            m_run = m_new;
-#pragma unroll
-            for (int rr = 0; rr < 4; ++rr) {
-                const float alpha_r = __shfl(alpha, 4 * g + rr, 64);
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    o_acc[e][rr] *= alpha_r;
-                }
-            }
-        }
-
-        // probabilities, rounded to the storage dtype: A operand of P.V
-        uint2 p_op;
-        p_op.x = T::pack2(fastExp2(sc[0] - m_run), fastExp2(sc[1] - m_run));
-        p_op.y = T::pack2(fastExp2(sc[2] - m_run), fastExp2(sc[3] - m_run));
-        l_run += (T::unpackLo(p_op.x) + T::unpackHi(p_op.x)) + (T::unpackLo(p_op.y) + T::unpackHi(p_op.y));
-
-        // V rows beyond the sequence may hold anything (NaN included): zero them, 0 * NaN is NaN.
-        if (tail) {
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                if (tok0 + 4 * g + j >= end) {
-                    r.v[j] = make_uint4(0, 0, 0, 0);
-                }
-            }
-        }
-
-        // O += P . V, one 16-column output tile per e: column 8c+e of rows 4g..4g+3
-        const uint32_t v0[4] = {r.v[0].x, r.v[0].y, r.v[0].z, r.v[0].w};
-        const uint32_t v1[4] = {r.v[1].x, r.v[1].y, r.v[1].z, r.v[1].w};
-        const uint32_t v2[4] = {r.v[2].x, r.v[2].y, r.v[2].z, r.v[2].w};
-        const uint32_t v3[4] = {r.v[3].x, r.v[3].y, r.v[3].z, r.v[3].w};
-#pragma unroll
-        for (int w = 0; w < 4; ++w) {
-            uint2 even, odd;
-            even.x = __builtin_amdgcn_perm(v1[w], v0[w], 0x05040100u);
-            even.y = __builtin_amdgcn_perm(v3[w], v2[w], 0x05040100u);
-            odd.x = __builtin_amdgcn_perm(v1[w], v0[w], 0x07060302u);
-            odd.y = __builtin_amdgcn_perm(v3[w], v2[w], 0x07060302u);
-            o_acc[2 * w] = T::mfmaK16(p_op, even, o_acc[2 * w]);
-            o_acc[2 * w + 1] = T::mfmaK16(p_op, odd, o_acc[2 * w + 1]);
-        }
+        computeTile<T>(st, r, q_reg, k_lds, c, g, a.scale_log2, slope, tok0 - (len - 1), min(kTileTokens, end - tok0));
     };
 
-    // Two register sets alternate so that the loads of the next tile are in flight while the
-    // current one is computed.
-    TileRegs ra, rb;
-    loadTile(0, ra);
-    for (int t = 0; t < n_tiles; t += 2) {
+    // Three register sets rotate so that the loads of the next two tiles are in flight while the
+    // current one is computed. Invariant at the top of the loop: b0 / b1 hold (or are receiving)
+    // tiles t and t+1.
+    TileRegs b0 = loadTile(0), b1 = loadTile(1);
+    int t = 0;
+    for (; t + 3 <= n_tiles; t += 3) {
+        const TileRegs b2 = loadTile(t + 2);
+        compute(t, b0);
+        b0 = loadTile(t + 3);
+        compute(t + 1, b1);
+        b1 = loadTile(t + 4);
+        compute(t + 2, b2);
+    }
+    if (t < n_tiles) {
+        compute(t, b0);
         if (t + 1 < n_tiles) {
-            loadTile(t + 1, rb);
-        }
-        computeTile(t, ra);
-        if (t + 1 < n_tiles) {
-            if (t + 2 < n_tiles) {
-                loadTile(t + 2, ra);
-            }
-            computeTile(t + 1, rb);
+            compute(t + 1, b1);
         }
     }
 
     // Epilogue. Denominator of head c over all 16 token slots, then move per-head scalars to the
     // lanes that hold that head's accumulators.
-    float l_tot = l_run + __shfl_xor(l_run, 16, 64);
-    l_tot += __shfl_xor(l_tot, 32, 64);
+    const float l_tot = sumAcrossTokenGroups(st.l);
 
     const bool single = len <= a.partition_tokens;
 #pragma unroll
     for (int rr = 0; rr < 4; ++rr) {
         const int hl = 4 * g + rr; // head (within the chunk) of accumulator row rr
         const float l_h = __shfl(l_tot, hl, 64);
-        const float m_h = __shfl(m_run, hl, 64);
+        const float m_h = __shfl(st.m, hl, 64);
         const int hg = chunk * kHeadsPerWave + hl;
         if (hg >= a.group) {
             continue;
@@ -284,17 +334,17 @@ __global__ void __launch_bounds__(64) decodeTiledKernel(DecodeArgs a) {
         if (single) {
             const float inv_l = 1.0f / (l_h + 1e-6f);
             uint4 packed;
-            packed.x = T::pack2(o_acc[0][rr] * inv_l, o_acc[1][rr] * inv_l);
-            packed.y = T::pack2(o_acc[2][rr] * inv_l, o_acc[3][rr] * inv_l);
-            packed.z = T::pack2(o_acc[4][rr] * inv_l, o_acc[5][rr] * inv_l);
-            packed.w = T::pack2(o_acc[6][rr] * inv_l, o_acc[7][rr] * inv_l);
+            packed.x = T::pack2(st.o[0][rr] * inv_l, st.o[1][rr] * inv_l);
+            packed.y = T::pack2(st.o[2][rr] * inv_l, st.o[3][rr] * inv_l);
+            packed.z = T::pack2(st.o[4][rr] * inv_l, st.o[5][rr] * inv_l);
+            packed.w = T::pack2(st.o[6][rr] * inv_l, st.o[7][rr] * inv_l);
             S *o_ptr = static_cast<S *>(a.out) + seq * a.o_stride + out_head * a.o_head_stride;
             *reinterpret_cast<uint4 *>(o_ptr + 8 * c) = packed;
         } else {
             const int64_t slot = (static_cast<int64_t>(seq) * a.num_heads + out_head) * a.max_partitions + part;
             float4 *pa = reinterpret_cast<float4 *>(a.part_acc + slot * kTiledHead + 8 * c);
-            pa[0] = make_float4(o_acc[0][rr], o_acc[1][rr], o_acc[2][rr], o_acc[3][rr]);
-            pa[1] = make_float4(o_acc[4][rr], o_acc[5][rr], o_acc[6][rr], o_acc[7][rr]);
+            pa[0] = make_float4(st.o[0][rr], st.o[1][rr], st.o[2][rr], st.o[3][rr]);
+            pa[1] = make_float4(st.o[4][rr], st.o[5][rr], st.o[6][rr], st.o[7][rr]);
             if (c == 0) {
                 a.part_m[slot] = m_h;
                 a.part_l[slot] = l_h;

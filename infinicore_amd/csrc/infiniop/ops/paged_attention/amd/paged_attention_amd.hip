@@ -49,7 +49,9 @@ Plan makePlan(const PagedAttentionInfo &in, const device::amd::DeviceInfo &dev) 
               && multipleOf8(in.q_stride) && multipleOf8(in.q_head_stride) && multipleOf8(in.o_stride)
               && multipleOf8(in.o_head_stride) && multipleOf8(in.k_batch_stride) && multipleOf8(in.k_head_stride)
               && multipleOf8(in.k_row_stride) && multipleOf8(in.v_batch_stride) && multipleOf8(in.v_head_stride)
-              && multipleOf8(in.v_row_stride) && in.num_blocks > 0 && in.num_blocks <= 0x7fffffff;
+              && multipleOf8(in.v_row_stride) && in.num_blocks > 0 && in.num_blocks <= 0x7fffffff
+              // lane offsets inside a tile (15 rows + one row of bytes) are kept in 32 bits
+              && in.k_row_stride > 0 && in.k_row_stride < (1 << 26) && in.v_row_stride > 0 && in.v_row_stride < (1 << 26);
     if (const char *env = std::getenv("INFINIOP_AMD_PA_KERNEL")) {
         if (std::strcmp(env, "generic") == 0) {
             plan.tiled = false;
@@ -108,14 +110,15 @@ void launchGeneric(const DecodeArgs &a, const Plan &plan, hipStream_t stream) {
 }
 
 template <typename T, typename Tindex>
-void launchReduce(const DecodeArgs &a, const Plan &plan, hipStream_t stream) {
+void launchReduce(const DecodeArgs &a, hipStream_t stream) {
     const dim3 grid(a.num_heads, a.num_seqs);
-    switch (plan.dims_per_lane) {
-    case 1: decodeReduceKernel<T, Tindex, 1><<<grid, 64, 0, stream>>>(a); break;
-    case 2: decodeReduceKernel<T, Tindex, 2><<<grid, 64, 0, stream>>>(a); break;
-    case 3: decodeReduceKernel<T, Tindex, 3><<<grid, 64, 0, stream>>>(a); break;
-    case 4: decodeReduceKernel<T, Tindex, 4><<<grid, 64, 0, stream>>>(a); break;
-    default: decodeReduceKernel<T, Tindex, 9><<<grid, 64, 0, stream>>>(a); break;
+    switch (a.value_size / 16) { // value sizes the validator lets through: 64, 128, 192, 256, 512, 576
+    case 4: decodeReduceKernel<T, Tindex, 4><<<grid, kReduceThreads, 0, stream>>>(a); break;
+    case 8: decodeReduceKernel<T, Tindex, 8><<<grid, kReduceThreads, 0, stream>>>(a); break;
+    case 12: decodeReduceKernel<T, Tindex, 12><<<grid, kReduceThreads, 0, stream>>>(a); break;
+    case 16: decodeReduceKernel<T, Tindex, 16><<<grid, kReduceThreads, 0, stream>>>(a); break;
+    case 32: decodeReduceKernel<T, Tindex, 32><<<grid, kReduceThreads, 0, stream>>>(a); break;
+    default: decodeReduceKernel<T, Tindex, 36><<<grid, kReduceThreads, 0, stream>>>(a); break;
     }
 }
 
@@ -129,7 +132,7 @@ void launchAll(const DecodeArgs &a, const Plan &plan, bool tiled, hipStream_t st
         launchGeneric<typename T::Base, Tindex>(a, plan, stream);
     }
     if (plan.max_partitions > 1) {
-        launchReduce<typename T::Base, Tindex>(a, plan, stream);
+        launchReduce<typename T::Base, Tindex>(a, stream);
     }
 }
 
@@ -165,7 +168,8 @@ infiniStatus_t Descriptor::create(infiniopHandle_t handle, Descriptor **desc_ptr
     CHECK_RESULT(info);
     const PagedAttentionInfo in = info.take();
     const Plan plan = makePlan(in, device::amd::deviceInfo(handle->device_id));
-    const size_t workspace_bytes = plan.acc_bytes + 2 * plan.ml_bytes;
+    // 256 spare bytes let calculate() align the carve-up itself, whatever pointer the caller passes
+    const size_t workspace_bytes = plan.max_partitions > 1 ? plan.acc_bytes + 2 * plan.ml_bytes + 256 : 0;
     *desc_ptr = new Descriptor(new Opaque{plan}, in, workspace_bytes, handle->device, handle->device_id);
     return INFINI_STATUS_SUCCESS;
 }
@@ -201,7 +205,7 @@ infiniStatus_t Descriptor::calculate(void *workspace, size_t workspace_size, voi
     a.seq_lens = seq_lens;
     a.alibi_slopes = static_cast<const float *>(alibi_slopes);
     if (plan.max_partitions > 1) {
-        char *ws = static_cast<char *>(workspace);
+        char *ws = reinterpret_cast<char *>((reinterpret_cast<uintptr_t>(workspace) + 255) & ~static_cast<uintptr_t>(255));
         a.part_acc = reinterpret_cast<float *>(ws);
         a.part_m = reinterpret_cast<float *>(ws + plan.acc_bytes);
         a.part_l = reinterpret_cast<float *>(ws + plan.acc_bytes + plan.ml_bytes);
@@ -236,8 +240,7 @@ infiniStatus_t Descriptor::calculate(void *workspace, size_t workspace_size, voi
 
     // The tiled kernel moves 16 bytes per lane; base addresses that are not 16-byte aligned take
     // the element-wise kernel instead.
-    const bool tiled = plan.tiled && aligned16(out) && aligned16(q) && aligned16(k_cache) && aligned16(v_cache)
-                    && (plan.max_partitions == 1 || aligned16(workspace));
+    const bool tiled = plan.tiled && aligned16(out) && aligned16(q) && aligned16(k_cache) && aligned16(v_cache);
     auto stream = static_cast<hipStream_t>(stream_);
 
     infiniStatus_t status;
