@@ -9,6 +9,7 @@
 #include "decode_common.h"
 #include "decode_generic.h"
 #include "decode_reduce.h"
+#include "decode_balanced.h"
 #include "decode_tiled.h"
 #include <cstdlib>
 #include <cstring>
@@ -21,6 +22,9 @@ namespace {
 // device memory and are never read on the host).
 struct Plan {
     bool tiled;            // tiled matrix-core kernel (head 128, power-of-two pages >= 16, 16-byte aligned strides)
+    bool balanced;         // tiled kernel under the work-equalising schedule (decode_balanced.h)
+    int waves_per_stream;  // balanced: wavefronts that share the tiles of one (KV head, 16-head chunk)
+    int balanced_rows;     // balanced: workspace rows (waves_per_stream + num_seqs)
     int partition_tokens;  // tokens per unit of work
     int max_partitions;    // partitions the longest representable sequence needs
     int dims_per_lane;     // generic / reduce kernels: ceil(max(head_size, value_size) / 64)
@@ -89,7 +93,29 @@ Plan makePlan(const PagedAttentionInfo &in, const device::amd::DeviceInfo &dev) 
     const size_t widest = in.head_size > in.value_size ? in.head_size : in.value_size;
     plan.dims_per_lane = static_cast<int>((widest + 63) / 64);
 
-    if (plan.max_partitions > 1) {
+    // Ragged batches of up to kBalancedMaxSeqs sequences run the tiled kernel under the
+    // work-equalising schedule: as many wavefronts as the device holds at once (8 per compute unit
+    // at this kernel's register budget), each with an equal share of the tiles.
+    plan.balanced = plan.tiled && in.num_seqs <= static_cast<size_t>(kBalancedMaxSeqs);
+    if (const char *env = std::getenv("INFINIOP_AMD_PA_SCHEDULE")) {
+        if (std::strcmp(env, "grid") == 0) {
+            plan.balanced = false;
+        }
+    }
+    if (plan.balanced) {
+        int waves_per_cu = 8;
+        if (const char *env = std::getenv("INFINIOP_AMD_PA_WAVES_PER_CU")) {
+            const int forced = std::atoi(env);
+            waves_per_cu = forced >= 1 && forced <= 64 ? forced : waves_per_cu;
+        }
+        const long long stream_count = static_cast<long long>(in.num_kv_heads) * ((group + kHeadsPerWave - 1) / kHeadsPerWave);
+        long long wps = static_cast<long long>(dev.compute_units) * waves_per_cu / stream_count;
+        plan.waves_per_stream = static_cast<int>(wps < 1 ? 1 : wps);
+        plan.balanced_rows = plan.waves_per_stream + static_cast<int>(in.num_seqs);
+        const size_t slots = static_cast<size_t>(plan.balanced_rows) * in.num_heads;
+        plan.acc_bytes = alignUp(slots * in.value_size * sizeof(float), 256);
+        plan.ml_bytes = alignUp(slots * sizeof(float), 256);
+    } else if (plan.max_partitions > 1) {
         const size_t slots = in.num_seqs * in.num_heads * static_cast<size_t>(plan.max_partitions);
         plan.acc_bytes = alignUp(slots * in.value_size * sizeof(float), 256);
         plan.ml_bytes = alignUp(slots * sizeof(float), 256);
@@ -124,8 +150,14 @@ void launchReduce(const DecodeArgs &a, hipStream_t stream) {
 
 template <typename T, typename Tindex>
 void launchAll(const DecodeArgs &a, const Plan &plan, bool tiled, hipStream_t stream) {
+    const int head_chunks = (a.group + kHeadsPerWave - 1) / kHeadsPerWave;
+    if (tiled && plan.balanced) {
+        const dim3 grid(plan.waves_per_stream, a.num_kv_heads * head_chunks);
+        decodeBalancedKernel<T, Tindex><<<grid, 64, 0, stream>>>(a, plan.waves_per_stream);
+        decodeBalancedMergeKernel<T, Tindex><<<dim3(a.num_heads, a.num_seqs), kReduceThreads, 0, stream>>>(a, plan.waves_per_stream);
+        return;
+    }
     if (tiled) {
-        const int head_chunks = (a.group + kHeadsPerWave - 1) / kHeadsPerWave;
         const dim3 grid(plan.max_partitions, a.num_kv_heads * head_chunks, a.num_seqs);
         decodeTiledKernel<T, Tindex><<<grid, 64, 0, stream>>>(a);
     } else {
@@ -152,6 +184,23 @@ bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
 
 } // namespace
 
+#ifdef INFINIOP_AMD_PA_TRACE
+// Diagnostic build only: point the decode kernel's timestamp buffer at device memory.
+extern "C" __attribute__((visibility("default"))) int infiniopAmdPaTraceSet(void *device_buffer) {
+    return static_cast<int>(hipMemcpyToSymbol(HIP_SYMBOL(g_pa_trace), &device_buffer, sizeof(void *)));
+}
+// Diagnostic build only: workgroups of the balanced decode kernel the runtime expects to fit on one compute unit.
+extern "C" __attribute__((visibility("default"))) int infiniopAmdPaOccupancy() {
+    int blocks = -1;
+    hipFuncAttributes attr{};
+    (void)hipFuncGetAttributes(&attr, reinterpret_cast<const void *>(&decodeBalancedKernel<TileBF16, IndexI64>));
+    std::fprintf(stderr, "decodeBalancedKernel: numRegs=%d sharedSizeBytes=%zu localSizeBytes=%zu maxThreadsPerBlock=%d\n",
+                 attr.numRegs, attr.sharedSizeBytes, attr.localSizeBytes, attr.maxThreadsPerBlock);
+    (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, decodeBalancedKernel<TileBF16, IndexI64>, 64, 0);
+    return blocks;
+}
+#endif
+
 struct Descriptor::Opaque {
     Plan plan;
 };
@@ -169,7 +218,7 @@ infiniStatus_t Descriptor::create(infiniopHandle_t handle, Descriptor **desc_ptr
     const PagedAttentionInfo in = info.take();
     const Plan plan = makePlan(in, device::amd::deviceInfo(handle->device_id));
     // 256 spare bytes let calculate() align the carve-up itself, whatever pointer the caller passes
-    const size_t workspace_bytes = plan.max_partitions > 1 ? plan.acc_bytes + 2 * plan.ml_bytes + 256 : 0;
+    const size_t workspace_bytes = plan.acc_bytes > 0 ? plan.acc_bytes + 2 * plan.ml_bytes + 256 : 0;
     *desc_ptr = new Descriptor(new Opaque{plan}, in, workspace_bytes, handle->device, handle->device_id);
     return INFINI_STATUS_SUCCESS;
 }
@@ -204,7 +253,7 @@ infiniStatus_t Descriptor::calculate(void *workspace, size_t workspace_size, voi
     a.block_tables = block_tables;
     a.seq_lens = seq_lens;
     a.alibi_slopes = static_cast<const float *>(alibi_slopes);
-    if (plan.max_partitions > 1) {
+    if (plan.acc_bytes > 0) {
         char *ws = reinterpret_cast<char *>((reinterpret_cast<uintptr_t>(workspace) + 255) & ~static_cast<uintptr_t>(255));
         a.part_acc = reinterpret_cast<float *>(ws);
         a.part_m = reinterpret_cast<float *>(ws + plan.acc_bytes);

@@ -11,7 +11,11 @@ import ctypes
 from ctypes import POINTER, Structure, c_float, c_int, c_int64, c_size_t, c_uint32, c_uint64, c_void_p
 from pathlib import Path
 
-LIB_DIR = Path(__file__).resolve().parent / "lib"
+import os
+
+# INFINICORE_AMD_LIB_DIR points at another build of the two libraries (the reference's harness finds
+# them through INFINI_ROOT in the same way, test/infiniop/libinfiniop/liboperators.py:20-53).
+LIB_DIR = Path(os.environ.get("INFINICORE_AMD_LIB_DIR") or Path(__file__).resolve().parent / "lib")
 
 
 class InfiniStatus:
