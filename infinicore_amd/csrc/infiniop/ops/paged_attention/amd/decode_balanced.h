@@ -66,7 +66,9 @@ __device__ __forceinline__ int tilePrefixSums(const DecodeArgs &a, int lane, int
         running = __shfl(x, 63, 64);
     }
     __builtin_amdgcn_wave_barrier();
-    return running;
+    // every lane holds the same total; say so, or all index arithmetic derived from it is
+    // compiled as per-lane (vector) code with per-lane branches
+    return __builtin_amdgcn_readfirstlane(running);
 }
 
 // Tiles per piece: the flat range split evenly over the wavefronts of a stream, but never finer
@@ -76,9 +78,26 @@ __device__ __forceinline__ int tilesPerPiece(int total_tiles, int waves_per_stre
     return q < kBalancedMinTiles ? kBalancedMinTiles : q;
 }
 
+// The prefix sums are read from LDS with a wave-uniform index; readfirstlane tells the compiler the
+// value is uniform too, so everything derived from it stays in scalar registers and scalar branches.
+__device__ __forceinline__ int uniformRead(const int *lds_word) {
+    return __builtin_amdgcn_readfirstlane(*lds_word);
+}
+
+// A run = consecutive tiles of one sequence whose pages fit one page-id register (64 block-table
+// entries, one per lane). All members are wave-uniform.
+struct TileRun {
+    int seq;
+    int t0, t1;      // tiles [t0, t1) of the sequence
+    int seg_end;     // end of the segment (this wavefront's share of the sequence) the run belongs to
+    int first_entry; // block-table entry of tile t0
+    bool valid;      // false past the end of the wavefront's piece
+};
+
 template <typename T, typename Tindex>
 __global__ void __launch_bounds__(64) decodeBalancedKernel(DecodeArgs a, int waves_per_stream) {
     using S = typename T::storage;
+    constexpr int NBUF = INFINIOP_AMD_PA_BALANCED_BUFFERS;
     __shared__ uint4 k_lds[kTileTokens * kTiledHead / 8];
     __shared__ int pre_incl[kBalancedMaxSeqs];
 
@@ -91,6 +110,13 @@ __global__ void __launch_bounds__(64) decodeBalancedKernel(DecodeArgs a, int wav
     const int g = lane >> 4;
 
     PA_STAMP(0);
+#ifdef INFINIOP_AMD_PA_TRACE
+    if (g_pa_trace != nullptr && threadIdx.x == 0) {
+        const size_t w = static_cast<size_t>(blockIdx.y) * gridDim.x + blockIdx.x;
+        g_pa_trace[w * 8 + 6] = __builtin_amdgcn_s_getreg(63492); // HW_ID
+        g_pa_trace[w * 8 + 7] = __builtin_amdgcn_s_getreg(63508); // XCC_ID
+    }
+#endif
     const int total_tiles = tilePrefixSums<Tindex>(a, lane, pre_incl);
     PA_STAMP(1);
     const int q = tilesPerPiece(total_tiles, waves_per_stream);
@@ -100,11 +126,12 @@ __global__ void __launch_bounds__(64) decodeBalancedKernel(DecodeArgs a, int wav
         return;
     }
     // first sequence whose tiles reach past f0
-    int seq = 0;
+    int seq0 = 0;
     for (int base = 0; base < a.num_seqs; base += 64) {
         const int b = base + lane;
-        seq += __popcll(__builtin_amdgcn_ballot_w64(b < a.num_seqs && pre_incl[b] <= f0));
+        seq0 += __popcll(__builtin_amdgcn_ballot_w64(b < a.num_seqs && pre_incl[b] <= f0));
     }
+    seq0 = __builtin_amdgcn_readfirstlane(seq0);
 
     const int64_t max_len = static_cast<int64_t>(a.max_blocks_per_seq) << a.block_shift;
     const int head_in_group = chunk * kHeadsPerWave + c;
@@ -114,6 +141,7 @@ __global__ void __launch_bounds__(64) decodeBalancedKernel(DecodeArgs a, int wav
     const char *k_head = reinterpret_cast<const char *>(static_cast<const S *>(a.k_cache) + kv_head * a.k_head_stride);
     const char *v_head = reinterpret_cast<const char *>(static_cast<const S *>(a.v_cache) + kv_head * a.v_head_stride);
     const int block_mask = a.block_size - 1;
+    const int tiles_per_entry_shift = a.block_shift - 4; // log2(block_size / 16)
     const uint32_t k_row_bytes = static_cast<uint32_t>(a.k_row_stride) * sizeof(S);
     const uint32_t v_row_bytes = static_cast<uint32_t>(a.v_row_stride) * sizeof(S);
     uint32_t k_off[4], v_off[4];
@@ -123,81 +151,127 @@ __global__ void __launch_bounds__(64) decodeBalancedKernel(DecodeArgs a, int wav
         v_off[j] = (4 * g + j) * v_row_bytes + 16 * c;
     }
 
-    int f = f0;
-    while (f < f1) {
-        // ---- segment: tiles [t_begin, t_end) of sequence `seq` ----
-        const int seq_first = seq == 0 ? 0 : pre_incl[seq - 1];
-        const int seq_tiles = pre_incl[seq] - seq_first;
-        const int t_begin = f - seq_first;
-        const int t_end = min(seq_tiles, f1 - seq_first);
-        int64_t len64 = loadIndex<Tindex>(a.seq_lens, seq);
-        const int len = static_cast<int>(len64 < max_len ? len64 : max_len);
-
-        uint4 q_reg[4];
-        {
-            const S *q_ptr = static_cast<const S *>(a.q) + seq * a.q_stride + (head_valid ? head : 0) * a.q_head_stride;
-#pragma unroll
-            for (int kk = 0; kk < 4; ++kk) {
-                q_reg[kk] = head_valid ? *reinterpret_cast<const uint4 *>(q_ptr + 32 * kk + 8 * g) : make_uint4(0, 0, 0, 0);
-            }
+    // ---- wave-uniform walk over the piece: sequences -> segments -> runs ----
+    auto seqFirstTile = [&](int s) { return s == 0 ? 0 : uniformRead(&pre_incl[s - 1]); };
+    auto seqLastTile = [&](int s) { return uniformRead(&pre_incl[s]); };
+    auto makeRun = [&](int s, int t0, int seg_end) {
+        TileRun r;
+        r.seq = s;
+        r.t0 = t0;
+        r.seg_end = seg_end;
+        r.first_entry = t0 >> tiles_per_entry_shift;
+        const int last_entry = min((seg_end - 1) >> tiles_per_entry_shift, r.first_entry + 63);
+        r.t1 = min(seg_end, (last_entry + 1) << tiles_per_entry_shift);
+        r.valid = true;
+        return r;
+    };
+    // run that starts at flat tile `flat`, which lies in sequence s
+    auto runAtFlat = [&](int s, int flat) {
+        const int first = seqFirstTile(s);
+        return makeRun(s, flat - first, min(seqLastTile(s) - first, f1 - first));
+    };
+    auto nextRun = [&](const TileRun &r) {
+        if (r.t1 < r.seg_end) {
+            return makeRun(r.seq, r.t1, r.seg_end);
         }
-        TileState st;
+        const int flat = seqFirstTile(r.seq) + r.seg_end;
+        if (!r.valid || flat >= f1) {
+            TileRun none = r;
+            none.valid = false;
+            return none;
+        }
+        int s = r.seq + 1;
+        while (seqLastTile(s) <= flat) { // sequences without tokens
+            ++s;
+        }
+        return runAtFlat(s, flat);
+    };
+    auto loadPageIds = [&](const TileRun &r) {
+        int ids = 0;
+        const int last_entry = (r.t1 - 1) >> tiles_per_entry_shift;
+        if (r.valid && r.first_entry + lane <= last_entry) {
+            // low 32 bits, untouched: the value is clamped where it is used, so that nothing waits
+            // for this load while tiles are in flight
+            ids = static_cast<int>(loadIndex<Tindex>(a.block_tables, r.seq * a.block_table_batch_stride + r.first_entry + lane));
+        }
+        return ids;
+    };
+
+    // ---- load side: runs NBUF-1 tiles ahead of the compute side, across runs and sequences ----
+    TileRun ld_run = runAtFlat(seq0, f0);
+    int ld_ids = loadPageIds(ld_run);
+    TileRun ld_next = nextRun(ld_run);
+    int ld_next_ids = loadPageIds(ld_next);
+    int ld_t = ld_run.t0;
+
+    auto loadNextTile = [&]() -> TileRegs {
+        const bool real = ld_run.valid;
+        const uint32_t lane_mask = real ? 0xffffffffu : 0u;
+        const int entry = real ? (ld_t >> tiles_per_entry_shift) - ld_run.first_entry : 0;
+        const int page = real ? clampPage(__builtin_amdgcn_readlane(ld_ids, entry), a.num_blocks) : 0;
+        const int row0 = real ? (ld_t * kTileTokens) & block_mask : 0;
+        const char *k_tile = k_head + (page * a.k_batch_stride + row0 * a.k_row_stride) * static_cast<int64_t>(sizeof(S));
+        const char *v_tile = v_head + (page * a.v_batch_stride + row0 * a.v_row_stride) * static_cast<int64_t>(sizeof(S));
+        TileRegs r;
+        r.k0 = loadLane16(k_tile, k_off[0] & lane_mask);
+        r.k1 = loadLane16(k_tile, k_off[1] & lane_mask);
+        r.k2 = loadLane16(k_tile, k_off[2] & lane_mask);
+        r.k3 = loadLane16(k_tile, k_off[3] & lane_mask);
+        r.v0 = loadLane16(v_tile, v_off[0] & lane_mask);
+        r.v1 = loadLane16(v_tile, v_off[1] & lane_mask);
+        r.v2 = loadLane16(v_tile, v_off[2] & lane_mask);
+        r.v3 = loadLane16(v_tile, v_off[3] & lane_mask);
+        if (real && ++ld_t == ld_run.t1) {
+            // next run: its page ids were requested one run ago
+            ld_run = ld_next;
+            ld_ids = ld_next_ids;
+            ld_t = ld_run.t0;
+            ld_next = nextRun(ld_run);
+            ld_next_ids = loadPageIds(ld_next);
+        }
+        return r;
+    };
+
+    // ---- compute side ----
+    TileState st;
+    uint4 q_reg[4];
+    int c_seq = seq0, c_t = 0, c_t_begin = 0, c_seg_end = 0, c_seq_tiles = 0, c_len = 0;
+
+    auto beginSegment = [&](int s, int flat) {
+        const int first = seqFirstTile(s);
+        c_seq = s;
+        c_seq_tiles = seqLastTile(s) - first;
+        c_t_begin = flat - first;
+        c_t = c_t_begin;
+        c_seg_end = min(c_seq_tiles, f1 - first);
+        if (c_t_begin == 0 && blockIdx.y == 0 && lane == 0) {
+            // tell the merge kernel which pieces hold this sequence (one writer per sequence)
+            a.seq_pieces[s] = make_int2(piece, (first + c_seq_tiles - 1) / q - piece + 1);
+        }
+        const int64_t len64 = loadIndex<Tindex>(a.seq_lens, s);
+        c_len = __builtin_amdgcn_readfirstlane(static_cast<int>(len64 < max_len ? len64 : max_len));
+        const S *q_ptr = static_cast<const S *>(a.q) + s * a.q_stride + (head_valid ? head : 0) * a.q_head_stride;
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) {
+            q_reg[kk] = head_valid ? *reinterpret_cast<const uint4 *>(q_ptr + 32 * kk + 8 * g) : make_uint4(0, 0, 0, 0);
+        }
+        // Use the query here, inside the rarely taken segment switch: the wait for it lands here and
+        // the per-tile code keeps waiting for exactly its own tile, with the others still in flight.
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) {
+            asm volatile("" ::"v"(q_reg[kk].x), "v"(q_reg[kk].y), "v"(q_reg[kk].z), "v"(q_reg[kk].w));
+        }
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
             st.o[e] = f32x4{0.f, 0.f, 0.f, 0.f};
         }
         st.m = -INFINITY;
         st.l = 0.0f;
+    };
 
-        // The segment is walked in runs of at most 64 block-table entries (one page id per lane).
-        int t_run = t_begin;
-        while (t_run < t_end) {
-            const int first_entry = (t_run * kTileTokens) >> a.block_shift;
-            const int last_entry_all = ((t_end * kTileTokens) - 1) >> a.block_shift;
-            const int last_entry = min(last_entry_all, first_entry + 63);
-            // last tile of this run: the one that ends with table entry `last_entry`
-            const int run_end = min(t_end, (((last_entry + 1) << a.block_shift) + kTileTokens - 1) / kTileTokens);
-            int page_ids = 0;
-            if (first_entry + lane <= last_entry) {
-                page_ids = clampPage(
-                    loadIndex<Tindex>(a.block_tables, seq * a.block_table_batch_stride + first_entry + lane), a.num_blocks);
-            }
-            const int n_tiles = run_end - t_run;
-
-            // loads past the end of the run: all lanes read the run's first 16 bytes (see decode_tiled.h)
-            auto loadTile = [&](int t) -> TileRegs {
-                const bool real = t < n_tiles;
-                const uint32_t lane_mask = real ? 0xffffffffu : 0u;
-                const int tok0 = (t_run + (real ? t : 0)) * kTileTokens;
-                const int page = __builtin_amdgcn_readlane(page_ids, (tok0 >> a.block_shift) - first_entry);
-                const int row0 = tok0 & block_mask;
-                const char *k_tile = k_head + (page * a.k_batch_stride + row0 * a.k_row_stride) * static_cast<int64_t>(sizeof(S));
-                const char *v_tile = v_head + (page * a.v_batch_stride + row0 * a.v_row_stride) * static_cast<int64_t>(sizeof(S));
-                TileRegs r;
-                r.k0 = loadLane16(k_tile, k_off[0] & lane_mask);
-                r.k1 = loadLane16(k_tile, k_off[1] & lane_mask);
-                r.k2 = loadLane16(k_tile, k_off[2] & lane_mask);
-                r.k3 = loadLane16(k_tile, k_off[3] & lane_mask);
-                r.v0 = loadLane16(v_tile, v_off[0] & lane_mask);
-                r.v1 = loadLane16(v_tile, v_off[1] & lane_mask);
-                r.v2 = loadLane16(v_tile, v_off[2] & lane_mask);
-                r.v3 = loadLane16(v_tile, v_off[3] & lane_mask);
-                return r;
-            };
-            auto compute = [&](int t, const TileRegs &r) {
-                const int tok0 = (t_run + t) * kTileTokens;
-                computeTile<T>(st, r, q_reg, k_lds, c, g, a.scale_log2, slope, tok0 - (len - 1), min(kTileTokens, len - tok0));
-            };
-
-            PA_STAMP(2);
-            streamTiles<INFINIOP_AMD_PA_BALANCED_BUFFERS>(n_tiles, loadTile, compute);
-            t_run = run_end;
-        }
-        PA_STAMP(4);
-
-        // ---- segment epilogue ----
+    auto endSegment = [&]() {
         const float l_tot = sumAcrossTokenGroups(st.l);
-        const bool whole = t_begin == 0 && t_end == seq_tiles;
+        const bool whole = c_t_begin == 0 && c_seg_end == c_seq_tiles;
 #pragma unroll
         for (int rr = 0; rr < 4; ++rr) {
             const int hl = 4 * g + rr;
@@ -215,10 +289,10 @@ __global__ void __launch_bounds__(64) decodeBalancedKernel(DecodeArgs a, int wav
                 packed.y = T::pack2(st.o[2][rr] * inv_l, st.o[3][rr] * inv_l);
                 packed.z = T::pack2(st.o[4][rr] * inv_l, st.o[5][rr] * inv_l);
                 packed.w = T::pack2(st.o[6][rr] * inv_l, st.o[7][rr] * inv_l);
-                S *o_ptr = static_cast<S *>(a.out) + seq * a.o_stride + out_head * a.o_head_stride;
+                S *o_ptr = static_cast<S *>(a.out) + c_seq * a.o_stride + out_head * a.o_head_stride;
                 *reinterpret_cast<uint4 *>(o_ptr + 8 * c) = packed;
             } else {
-                const int64_t slot = static_cast<int64_t>(piece + seq) * a.num_heads + out_head;
+                const int64_t slot = static_cast<int64_t>(piece + c_seq) * a.num_heads + out_head;
                 float4 *pa = reinterpret_cast<float4 *>(a.part_acc + slot * kTiledHead + 8 * c);
                 pa[0] = make_float4(st.o[0][rr], st.o[1][rr], st.o[2][rr], st.o[3][rr]);
                 pa[1] = make_float4(st.o[4][rr], st.o[5][rr], st.o[6][rr], st.o[7][rr]);
@@ -228,24 +302,53 @@ __global__ void __launch_bounds__(64) decodeBalancedKernel(DecodeArgs a, int wav
                 }
             }
         }
+    };
 
-        PA_STAMP(5);
-        f = seq_first + t_end;
-        ++seq;
-        // skip sequences without tokens
-        while (f < f1 && seq < a.num_seqs && pre_incl[seq] <= f) {
-            ++seq;
+    auto computeNextTile = [&](const TileRegs &r) {
+        const int tok0 = c_t * kTileTokens;
+        computeTile<T>(st, r, q_reg, k_lds, c, g, a.scale_log2, slope, tok0 - (c_len - 1), min(kTileTokens, c_len - tok0));
+        if (++c_t == c_seg_end) {
+            PA_STAMP(3);
+            endSegment();
+            const int flat = seqFirstTile(c_seq) + c_seg_end;
+            if (flat < f1) {
+                int s = c_seq + 1;
+                while (seqLastTile(s) <= flat) {
+                    ++s;
+                }
+                beginSegment(s, flat);
+            }
+        }
+    };
+
+    // The first tiles are requested before the first query: the query's round trip then overlaps
+    // with theirs.
+    PA_STAMP(2);
+    const int n_flat = f1 - f0;
+    TileRegs buf[NBUF];
+#pragma unroll
+    for (int i = 0; i < NBUF - 1; ++i) {
+        buf[i] = loadNextTile();
+    }
+    beginSegment(seq0, f0);
+    for (int t = 0; t < n_flat; t += NBUF) {
+#pragma unroll
+        for (int i = 0; i < NBUF; ++i) {
+            buf[(i + NBUF - 1) % NBUF] = loadNextTile();
+            if (t + i < n_flat) {
+                computeNextTile(buf[i]);
+            }
         }
     }
+    PA_STAMP(4);
 }
 
 // Merge of the segment rows of one (query head, sequence); see decode_reduce.h for the arithmetic.
 // One 256-thread workgroup: thread = (row group rg = tid / 16, 8-column strip c = tid % 16).
 template <typename T, typename Tindex>
-__global__ void __launch_bounds__(kReduceThreads) decodeBalancedMergeKernel(DecodeArgs a, int waves_per_stream) {
+__global__ void __launch_bounds__(kReduceThreads) decodeBalancedMergeKernel(DecodeArgs a) {
     using S = typename T::storage;
     constexpr int COLS = kTiledHead / 16;
-    __shared__ int pre_incl[kBalancedMaxSeqs];
     __shared__ float wave_acc[4][16][COLS];
     __shared__ float wave_m[4][16];
     __shared__ float wave_l[4][16];
@@ -257,21 +360,13 @@ __global__ void __launch_bounds__(kReduceThreads) decodeBalancedMergeKernel(Deco
     const int rg = tid >> 4;
     const int wave = tid >> 6;
 
-    // every wavefront redoes the prefix sums (identical values land in the same LDS words)
-    const int total_tiles = tilePrefixSums<Tindex>(a, tid & 63, pre_incl);
-    __syncthreads();
-    const int q = tilesPerPiece(total_tiles, waves_per_stream);
-    const int seq_first = seq == 0 ? 0 : pre_incl[seq - 1];
-    const int seq_tiles = pre_incl[seq] - seq_first;
-    if (seq_tiles <= 0) {
-        return;
+    const int64_t len64 = loadIndex<Tindex>(a.seq_lens, seq);
+    const int2 pieces = a.seq_pieces[seq]; // written by the decode kernel for every sequence with tokens
+    if (len64 <= 0 || pieces.y <= 1) {
+        return; // no tokens, or one segment covered the whole sequence and wrote `out` itself
     }
-    const int piece_first = seq_first / q;
-    const int piece_last = (seq_first + seq_tiles - 1) / q;
-    if (piece_first == piece_last) {
-        return; // one segment covered the whole sequence and wrote `out` itself
-    }
-    const int parts = piece_last - piece_first + 1;
+    const int piece_first = pieces.x;
+    const int parts = pieces.y;
 
     float m_loc = -INFINITY, l_loc = 0.0f;
     float acc[COLS];

@@ -31,6 +31,7 @@ struct DecodeArgs {
     float *part_acc; // [.., value_size]
     float *part_m;
     float *part_l;
+    int2 *seq_pieces; // work-equalising schedule only: per sequence {first piece, number of pieces}
 
     float scale_log2; // scale * log2(e)
     int32_t num_seqs;

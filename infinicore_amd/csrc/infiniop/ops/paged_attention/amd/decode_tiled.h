@@ -228,7 +228,7 @@ __device__ __forceinline__ void streamTiles(int n_tiles, Load loadTile, Compute 
 #define INFINIOP_AMD_PA_GRID_BUFFERS 3
 #endif
 #ifndef INFINIOP_AMD_PA_BALANCED_BUFFERS
-#define INFINIOP_AMD_PA_BALANCED_BUFFERS 5
+#define INFINIOP_AMD_PA_BALANCED_BUFFERS 3
 #endif
 
 template <typename T, typename Tindex>

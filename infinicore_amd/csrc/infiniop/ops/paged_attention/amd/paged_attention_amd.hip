@@ -28,7 +28,8 @@ struct Plan {
     int partition_tokens;  // tokens per unit of work
     int max_partitions;    // partitions the longest representable sequence needs
     int dims_per_lane;     // generic / reduce kernels: ceil(max(head_size, value_size) / 64)
-    size_t acc_bytes, ml_bytes; // workspace carve-up: [acc][m][l], each region 256-byte aligned
+    size_t acc_bytes, ml_bytes; // workspace carve-up: [acc][m][l][pieces], each region 256-byte aligned
+    size_t pieces_bytes;        // balanced: {first piece, piece count} per sequence
 };
 
 size_t alignUp(size_t x, size_t a) { return (x + a - 1) / a * a; }
@@ -103,7 +104,7 @@ Plan makePlan(const PagedAttentionInfo &in, const device::amd::DeviceInfo &dev) 
         }
     }
     if (plan.balanced) {
-        int waves_per_cu = 8;
+        int waves_per_cu = 4;
         if (const char *env = std::getenv("INFINIOP_AMD_PA_WAVES_PER_CU")) {
             const int forced = std::atoi(env);
             waves_per_cu = forced >= 1 && forced <= 64 ? forced : waves_per_cu;
@@ -115,6 +116,7 @@ Plan makePlan(const PagedAttentionInfo &in, const device::amd::DeviceInfo &dev) 
         const size_t slots = static_cast<size_t>(plan.balanced_rows) * in.num_heads;
         plan.acc_bytes = alignUp(slots * in.value_size * sizeof(float), 256);
         plan.ml_bytes = alignUp(slots * sizeof(float), 256);
+        plan.pieces_bytes = alignUp(in.num_seqs * 2 * sizeof(int), 256);
     } else if (plan.max_partitions > 1) {
         const size_t slots = in.num_seqs * in.num_heads * static_cast<size_t>(plan.max_partitions);
         plan.acc_bytes = alignUp(slots * in.value_size * sizeof(float), 256);
@@ -154,7 +156,7 @@ void launchAll(const DecodeArgs &a, const Plan &plan, bool tiled, hipStream_t st
     if (tiled && plan.balanced) {
         const dim3 grid(plan.waves_per_stream, a.num_kv_heads * head_chunks);
         decodeBalancedKernel<T, Tindex><<<grid, 64, 0, stream>>>(a, plan.waves_per_stream);
-        decodeBalancedMergeKernel<T, Tindex><<<dim3(a.num_heads, a.num_seqs), kReduceThreads, 0, stream>>>(a, plan.waves_per_stream);
+        decodeBalancedMergeKernel<T, Tindex><<<dim3(a.num_heads, a.num_seqs), kReduceThreads, 0, stream>>>(a);
         return;
     }
     if (tiled) {
@@ -218,7 +220,7 @@ infiniStatus_t Descriptor::create(infiniopHandle_t handle, Descriptor **desc_ptr
     const PagedAttentionInfo in = info.take();
     const Plan plan = makePlan(in, device::amd::deviceInfo(handle->device_id));
     // 256 spare bytes let calculate() align the carve-up itself, whatever pointer the caller passes
-    const size_t workspace_bytes = plan.acc_bytes > 0 ? plan.acc_bytes + 2 * plan.ml_bytes + 256 : 0;
+    const size_t workspace_bytes = plan.acc_bytes > 0 ? plan.acc_bytes + 2 * plan.ml_bytes + plan.pieces_bytes + 256 : 0;
     *desc_ptr = new Descriptor(new Opaque{plan}, in, workspace_bytes, handle->device, handle->device_id);
     return INFINI_STATUS_SUCCESS;
 }
@@ -258,6 +260,7 @@ infiniStatus_t Descriptor::calculate(void *workspace, size_t workspace_size, voi
         a.part_acc = reinterpret_cast<float *>(ws);
         a.part_m = reinterpret_cast<float *>(ws + plan.acc_bytes);
         a.part_l = reinterpret_cast<float *>(ws + plan.acc_bytes + plan.ml_bytes);
+        a.seq_pieces = reinterpret_cast<int2 *>(ws + plan.acc_bytes + 2 * plan.ml_bytes);
     }
     a.scale_log2 = in.scale * kLog2e;
     a.num_seqs = static_cast<int32_t>(in.num_seqs);
