@@ -344,22 +344,25 @@ __global__ void __launch_bounds__(64) decodeBalancedKernel(DecodeArgs a, int wav
 }
 
 // Merge of the segment rows of one (query head, sequence); see decode_reduce.h for the arithmetic.
-// One 256-thread workgroup: thread = (row group rg = tid / 16, 8-column strip c = tid % 16).
+// One wavefront per (head, sequence), four of them per workgroup. Lane = (row group g = lane / 16,
+// 8-column strip c = lane % 16): row group g merges rows g, g+4, ... of the sequence, the four
+// groups are then combined with lane swaps, and the lanes of group 0 store 16 bytes each. The piece
+// range of the sequence was left in seq_pieces by the decode kernel, so the only dependent memory
+// round trips are {length, piece range} -> rows.
 template <typename T, typename Tindex>
-__global__ void __launch_bounds__(kReduceThreads) decodeBalancedMergeKernel(DecodeArgs a) {
+__global__ void __launch_bounds__(256) decodeBalancedMergeKernel(DecodeArgs a) {
     using S = typename T::storage;
-    constexpr int COLS = kTiledHead / 16;
-    __shared__ float wave_acc[4][16][COLS];
-    __shared__ float wave_m[4][16];
-    __shared__ float wave_l[4][16];
-
-    const int head = blockIdx.x;
+    const int head = blockIdx.x * 4 + (threadIdx.x >> 6);
     const int seq = blockIdx.y;
-    const int tid = threadIdx.x;
-    const int c = tid & 15;
-    const int rg = tid >> 4;
-    const int wave = tid >> 6;
-
+    const int lane = threadIdx.x & 63;
+    const int c = lane & 15;
+    const int g = lane >> 4;
+    if (head >= a.num_heads) {
+        return;
+    }
+#ifdef PA_EXPERIMENT_EMPTY_MERGE
+    return;
+#endif
     const int64_t len64 = loadIndex<Tindex>(a.seq_lens, seq);
     const int2 pieces = a.seq_pieces[seq]; // written by the decode kernel for every sequence with tokens
     if (len64 <= 0 || pieces.y <= 1) {
@@ -369,16 +372,12 @@ __global__ void __launch_bounds__(kReduceThreads) decodeBalancedMergeKernel(Deco
     const int parts = pieces.y;
 
     float m_loc = -INFINITY, l_loc = 0.0f;
-    float acc[COLS];
-#pragma unroll
-    for (int i = 0; i < COLS; ++i) {
-        acc[i] = 0.0f;
-    }
-    for (int p = rg; p < parts; p += kReduceRowGroups) {
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    for (int p = g; p < parts; p += 4) {
         const int64_t slot = static_cast<int64_t>(piece_first + p + seq) * a.num_heads + head;
         const float m_p = a.part_m[slot];
         const float l_p = a.part_l[slot];
-        const float4 *row = reinterpret_cast<const float4 *>(a.part_acc + slot * kTiledHead + c * COLS);
+        const float4 *row = reinterpret_cast<const float4 *>(a.part_acc + slot * kTiledHead + 8 * c);
         const float4 v0 = row[0], v1 = row[1];
         const float m_new = fmaxf(m_loc, m_p);
         const float w_old = mergeWeight(m_loc, m_new), w_p = mergeWeight(m_p, m_new);
@@ -393,52 +392,22 @@ __global__ void __launch_bounds__(kReduceThreads) decodeBalancedMergeKernel(Deco
         acc[7] = acc[7] * w_old + v1.w * w_p;
         m_loc = m_new;
     }
-
-    const float m_w = swapMax(m_loc);
-    const float fct = mergeWeight(m_loc, m_w);
-    const float l_w = swapSum(l_loc * fct);
+    const float m_all = swapMax(m_loc);
+    const float f = mergeWeight(m_loc, m_all);
+    const float l_all = swapSum(l_loc * f);
 #pragma unroll
-    for (int i = 0; i < COLS; ++i) {
-        acc[i] = swapSum(acc[i] * fct);
+    for (int i = 0; i < 8; ++i) {
+        acc[i] = swapSum(acc[i] * f);
     }
-    if ((tid & 63) < 16) {
-        wave_m[wave][c] = m_w;
-        wave_l[wave][c] = l_w;
-#pragma unroll
-        for (int i = 0; i < COLS; ++i) {
-            wave_acc[wave][c][i] = acc[i];
-        }
-    }
-    __syncthreads();
-
-    if (tid < 16) {
-        float m = wave_m[0][c];
-#pragma unroll
-        for (int w = 1; w < 4; ++w) {
-            m = fmaxf(m, wave_m[w][c]);
-        }
-        float l = 0.0f, out_acc[COLS];
-#pragma unroll
-        for (int i = 0; i < COLS; ++i) {
-            out_acc[i] = 0.0f;
-        }
-#pragma unroll
-        for (int w = 0; w < 4; ++w) {
-            const float fw = mergeWeight(wave_m[w][c], m);
-            l += wave_l[w][c] * fw;
-#pragma unroll
-            for (int i = 0; i < COLS; ++i) {
-                out_acc[i] += wave_acc[w][c][i] * fw;
-            }
-        }
-        const float inv_l = 1.0f / (l + 1e-6f);
+    if (g == 0) {
+        const float inv_l = 1.0f / (l_all + 1e-6f);
         uint4 packed;
-        packed.x = T::pack2(out_acc[0] * inv_l, out_acc[1] * inv_l);
-        packed.y = T::pack2(out_acc[2] * inv_l, out_acc[3] * inv_l);
-        packed.z = T::pack2(out_acc[4] * inv_l, out_acc[5] * inv_l);
-        packed.w = T::pack2(out_acc[6] * inv_l, out_acc[7] * inv_l);
+        packed.x = T::pack2(acc[0] * inv_l, acc[1] * inv_l);
+        packed.y = T::pack2(acc[2] * inv_l, acc[3] * inv_l);
+        packed.z = T::pack2(acc[4] * inv_l, acc[5] * inv_l);
+        packed.w = T::pack2(acc[6] * inv_l, acc[7] * inv_l);
         S *o_ptr = static_cast<S *>(a.out) + seq * a.o_stride + head * a.o_head_stride;
-        *reinterpret_cast<uint4 *>(o_ptr + c * COLS) = packed;
+        *reinterpret_cast<uint4 *>(o_ptr + 8 * c) = packed;
     }
 }
 

@@ -156,7 +156,7 @@ void launchAll(const DecodeArgs &a, const Plan &plan, bool tiled, hipStream_t st
     if (tiled && plan.balanced) {
         const dim3 grid(plan.waves_per_stream, a.num_kv_heads * head_chunks);
         decodeBalancedKernel<T, Tindex><<<grid, 64, 0, stream>>>(a, plan.waves_per_stream);
-        decodeBalancedMergeKernel<T, Tindex><<<dim3(a.num_heads, a.num_seqs), kReduceThreads, 0, stream>>>(a);
+        decodeBalancedMergeKernel<T, Tindex><<<dim3((a.num_heads + 3) / 4, a.num_seqs), 256, 0, stream>>>(a);
         return;
     }
     if (tiled) {
