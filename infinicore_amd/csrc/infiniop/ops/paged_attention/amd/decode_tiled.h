@@ -44,6 +44,7 @@ typedef float f32x2 __attribute__((ext_vector_type(2)));
 // Matrix-instruction and packing flavours of the two storage dtypes.
 struct TileBF16 : BFloat16 {
     using Base = BFloat16;
+    static constexpr bool kSplitProbabilities = true; // 8-bit significand: feed p as hi + lo
     static __device__ __forceinline__ f32x4 mfmaK32(uint4 a, uint4 b, f32x4 c) {
         return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
     }
@@ -60,6 +61,7 @@ struct TileBF16 : BFloat16 {
 };
 struct TileF16 : Half {
     using Base = Half;
+    static constexpr bool kSplitProbabilities = false; // 11 bits of a value in [0, 1] are enough
     static __device__ __forceinline__ f32x4 mfmaK32(uint4 a, uint4 b, f32x4 c) {
         return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
     }
@@ -182,11 +184,23 @@ __device__ __forceinline__ void computeTile(TileState &st, const TileRegs r, con
         }
     }
 
-    // probabilities, rounded to the storage dtype: A operand of P.V
-    uint2 p_op;
-    p_op.x = T::pack2(fastExp2(sc[0] - st.m), fastExp2(sc[1] - st.m));
-    p_op.y = T::pack2(fastExp2(sc[2] - st.m), fastExp2(sc[3] - st.m));
-    st.l += (T::unpackLo(p_op.x) + T::unpackHi(p_op.x)) + (T::unpackLo(p_op.y) + T::unpackHi(p_op.y));
+    // Probabilities as the A operand of P.V. The matrix instruction takes them in the storage dtype;
+    // fp16 keeps 11 significant bits of a value in [0, 1], bf16 only 8. For bf16 the probability is
+    // therefore fed as two terms, p = hi + lo with lo = bf16(p - hi), and P.V takes two matrix
+    // instructions per output tile: the product then carries ~16 bits of p, close to the fp32
+    // probabilities of the reference kernel. The denominator sums exactly what the numerator used.
+    const float p0 = fastExp2(sc[0] - st.m), p1 = fastExp2(sc[1] - st.m);
+    const float p2 = fastExp2(sc[2] - st.m), p3 = fastExp2(sc[3] - st.m);
+    uint2 p_op, p_lo;
+    p_op.x = T::pack2(p0, p1);
+    p_op.y = T::pack2(p2, p3);
+    float p_used = (T::unpackLo(p_op.x) + T::unpackHi(p_op.x)) + (T::unpackLo(p_op.y) + T::unpackHi(p_op.y));
+    if constexpr (T::kSplitProbabilities) {
+        p_lo.x = T::pack2(p0 - T::unpackLo(p_op.x), p1 - T::unpackHi(p_op.x));
+        p_lo.y = T::pack2(p2 - T::unpackLo(p_op.y), p3 - T::unpackHi(p_op.y));
+        p_used += (T::unpackLo(p_lo.x) + T::unpackHi(p_lo.x)) + (T::unpackLo(p_lo.y) + T::unpackHi(p_lo.y));
+    }
+    st.l += p_used;
 
     // V rows beyond the sequence may hold anything (NaN included) and 0 * NaN is NaN: zero them.
     typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
@@ -210,6 +224,10 @@ __device__ __forceinline__ void computeTile(TileState &st, const TileRegs r, con
         odd.y = __builtin_amdgcn_perm(v3[w], v2[w], 0x07060302u);
         st.o[2 * w] = T::mfmaK16(p_op, even, st.o[2 * w]);
         st.o[2 * w + 1] = T::mfmaK16(p_op, odd, st.o[2 * w + 1]);
+        if constexpr (T::kSplitProbabilities) {
+            st.o[2 * w] = T::mfmaK16(p_lo, even, st.o[2 * w]);
+            st.o[2 * w + 1] = T::mfmaK16(p_lo, odd, st.o[2 * w + 1]);
+        }
     }
 }
 

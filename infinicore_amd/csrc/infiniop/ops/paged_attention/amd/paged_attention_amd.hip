@@ -23,13 +23,15 @@ namespace {
 struct Plan {
     bool tiled;            // tiled matrix-core kernel (head 128, power-of-two pages >= 16, 16-byte aligned strides)
     bool balanced;         // tiled kernel under the work-equalising schedule (decode_balanced.h)
+    int partition_tokens;  // grid schedule: tokens per unit of work
+    int max_partitions;    // grid schedule: partitions the longest representable sequence needs
+    int dims_per_lane;     // element-wise kernel: ceil(max(head_size, value_size) / 64)
     int waves_per_stream;  // balanced: wavefronts that share the tiles of one (KV head, 16-head chunk)
-    int balanced_rows;     // balanced: workspace rows (waves_per_stream + num_seqs)
-    int partition_tokens;  // tokens per unit of work
-    int max_partitions;    // partitions the longest representable sequence needs
-    int dims_per_lane;     // generic / reduce kernels: ceil(max(head_size, value_size) / 64)
-    size_t acc_bytes, ml_bytes; // workspace carve-up: [acc][m][l][pieces], each region 256-byte aligned
-    size_t pieces_bytes;        // balanced: {first piece, piece count} per sequence
+    // Workspace regions, each 256-byte aligned: [acc][m][l][pieces]. A descriptor planned for the
+    // balanced schedule can still be run with the element-wise kernel (operands that turn out not
+    // to be 16-byte aligned), so the regions are sized for whichever schedule needs more.
+    size_t acc_bytes, ml_bytes, pieces_bytes;
+    size_t workspaceBytes() const { return acc_bytes > 0 ? acc_bytes + 2 * ml_bytes + pieces_bytes + 256 : 0; }
 };
 
 size_t alignUp(size_t x, size_t a) { return (x + a - 1) / a * a; }
@@ -55,6 +57,7 @@ Plan makePlan(const PagedAttentionInfo &in, const device::amd::DeviceInfo &dev) 
               && multipleOf8(in.o_head_stride) && multipleOf8(in.k_batch_stride) && multipleOf8(in.k_head_stride)
               && multipleOf8(in.k_row_stride) && multipleOf8(in.v_batch_stride) && multipleOf8(in.v_head_stride)
               && multipleOf8(in.v_row_stride) && in.num_blocks > 0 && in.num_blocks <= 0x7fffffff
+              && max_tokens < (1LL << 30)
               // lane offsets inside a tile (15 rows + one row of bytes) are kept in 32 bits
               && in.k_row_stride > 0 && in.k_row_stride < (1 << 26) && in.v_row_stride > 0 && in.v_row_stride < (1 << 26);
     if (const char *env = std::getenv("INFINIOP_AMD_PA_KERNEL")) {
@@ -63,13 +66,13 @@ Plan makePlan(const PagedAttentionInfo &in, const device::amd::DeviceInfo &dev) 
         }
     }
 
-    // Units of work the kernel is launched with = sequences x KV heads (x query heads for the
-    // generic kernel) x partitions. Aim at ~16 units per compute unit for the longest sequences, so
-    // that ragged batches still fill the device; keep a partition between 64 and 512 tokens.
+    // ---- grid schedule: units of work = sequences x KV heads (x query heads for the element-wise
+    // kernel) x partitions. Aim at ~16 units per compute unit for the longest sequences; keep a
+    // partition between 64 and 512 tokens.
     const long long group = static_cast<long long>(in.num_heads / in.num_kv_heads);
-    const long long streams = static_cast<long long>(in.num_seqs)
-                            * (plan.tiled ? in.num_kv_heads * ((group + kHeadsPerWave - 1) / kHeadsPerWave) : in.num_heads);
-    long long want = streams * max_tokens / (16LL * dev.compute_units);
+    const long long stream_count = static_cast<long long>(in.num_kv_heads) * ((group + kHeadsPerWave - 1) / kHeadsPerWave);
+    const long long units = static_cast<long long>(in.num_seqs) * (plan.tiled ? stream_count : static_cast<long long>(in.num_heads));
+    long long want = units * max_tokens / (16LL * dev.compute_units);
     int p = floorPow2(want < 1 ? 1 : want);
     p = p < 64 ? 64 : (p > 512 ? 512 : p);
     if (const char *env = std::getenv("INFINIOP_AMD_PA_PARTITION")) {
@@ -78,8 +81,8 @@ Plan makePlan(const PagedAttentionInfo &in, const device::amd::DeviceInfo &dev) 
             p = (forced + 15) / 16 * 16;
         }
     }
-    // Bound the workspace: at most 128 partitions, unless that would exceed what one wavefront can
-    // address through its single page-id load (64 table entries).
+    // Bound the workspace: at most 128 partitions, unless that would exceed what one wavefront of
+    // the tiled kernel can address through its single page-id load (64 table entries).
     const long long cap = plan.tiled ? 64 * bs : (1LL << 30);
     if (max_tokens > 128LL * p) {
         long long grown = (max_tokens + 127) / 128;
@@ -93,10 +96,12 @@ Plan makePlan(const PagedAttentionInfo &in, const device::amd::DeviceInfo &dev) 
     plan.max_partitions = static_cast<int>(max_tokens > 0 ? (max_tokens + p - 1) / p : 1);
     const size_t widest = in.head_size > in.value_size ? in.head_size : in.value_size;
     plan.dims_per_lane = static_cast<int>((widest + 63) / 64);
+    size_t rows = plan.max_partitions > 1 ? in.num_seqs * static_cast<size_t>(plan.max_partitions) : 0;
 
-    // Ragged batches of up to kBalancedMaxSeqs sequences run the tiled kernel under the
-    // work-equalising schedule: as many wavefronts as the device holds at once (8 per compute unit
-    // at this kernel's register budget), each with an equal share of the tiles.
+    // ---- balanced schedule: ragged batches of up to kBalancedMaxSeqs sequences run the tiled kernel
+    // with as many wavefronts as fill the device once at one wavefront per SIMD (4 per compute unit,
+    // the setting that measured best: every compute unit gets the same number, each wavefront streams
+    // as long as possible), each with an equal share of the tiles.
     plan.balanced = plan.tiled && in.num_seqs <= static_cast<size_t>(kBalancedMaxSeqs);
     if (const char *env = std::getenv("INFINIOP_AMD_PA_SCHEDULE")) {
         if (std::strcmp(env, "grid") == 0) {
@@ -109,18 +114,15 @@ Plan makePlan(const PagedAttentionInfo &in, const device::amd::DeviceInfo &dev) 
             const int forced = std::atoi(env);
             waves_per_cu = forced >= 1 && forced <= 64 ? forced : waves_per_cu;
         }
-        const long long stream_count = static_cast<long long>(in.num_kv_heads) * ((group + kHeadsPerWave - 1) / kHeadsPerWave);
-        long long wps = static_cast<long long>(dev.compute_units) * waves_per_cu / stream_count;
+        const long long wps = static_cast<long long>(dev.compute_units) * waves_per_cu / stream_count;
         plan.waves_per_stream = static_cast<int>(wps < 1 ? 1 : wps);
-        plan.balanced_rows = plan.waves_per_stream + static_cast<int>(in.num_seqs);
-        const size_t slots = static_cast<size_t>(plan.balanced_rows) * in.num_heads;
-        plan.acc_bytes = alignUp(slots * in.value_size * sizeof(float), 256);
-        plan.ml_bytes = alignUp(slots * sizeof(float), 256);
+        const size_t balanced_rows = static_cast<size_t>(plan.waves_per_stream) + in.num_seqs;
+        rows = rows > balanced_rows ? rows : balanced_rows;
         plan.pieces_bytes = alignUp(in.num_seqs * 2 * sizeof(int), 256);
-    } else if (plan.max_partitions > 1) {
-        const size_t slots = in.num_seqs * in.num_heads * static_cast<size_t>(plan.max_partitions);
-        plan.acc_bytes = alignUp(slots * in.value_size * sizeof(float), 256);
-        plan.ml_bytes = alignUp(slots * sizeof(float), 256);
+    }
+    if (rows > 0) {
+        plan.acc_bytes = alignUp(rows * in.num_heads * in.value_size * sizeof(float), 256);
+        plan.ml_bytes = alignUp(rows * in.num_heads * sizeof(float), 256);
     }
     return plan;
 }
@@ -219,8 +221,8 @@ infiniStatus_t Descriptor::create(infiniopHandle_t handle, Descriptor **desc_ptr
     CHECK_RESULT(info);
     const PagedAttentionInfo in = info.take();
     const Plan plan = makePlan(in, device::amd::deviceInfo(handle->device_id));
-    // 256 spare bytes let calculate() align the carve-up itself, whatever pointer the caller passes
-    const size_t workspace_bytes = plan.acc_bytes > 0 ? plan.acc_bytes + 2 * plan.ml_bytes + plan.pieces_bytes + 256 : 0;
+    // includes 256 spare bytes that let calculate() align the carve-up itself, whatever pointer the caller passes
+    const size_t workspace_bytes = plan.workspaceBytes();
     *desc_ptr = new Descriptor(new Opaque{plan}, in, workspace_bytes, handle->device, handle->device_id);
     return INFINI_STATUS_SUCCESS;
 }

@@ -176,8 +176,11 @@ static void attend_range(const oracle_attention_shape *s, const uint16_t *q_row,
     *l_out = l;
 }
 
-/* Unsplit decode, kernel_v2.cuh:134-336. Returns 0, or -1 on a bad argument. */
-int oracle_paged_attention(void *out_, const void *q_, const void *k_cache_, const void *v_cache_,
+/* Unsplit decode, kernel_v2.cuh:134-336. Returns 0, or -1 on a bad argument.
+ * out_f32 (optional, packed [num_seqs, num_heads, value_size]) receives acc / (l + 1e-6) as the fp32
+ * value the kernel holds just before it rounds to the storage dtype (:320-334); comparing a device
+ * result with it is free of the double rounding that comparing two rounded results carries. */
+int oracle_paged_attention(void *out_, float *out_f32, const void *q_, const void *k_cache_, const void *v_cache_,
                            const int64_t *block_tables, const int64_t *seq_lens, const float *alibi_slopes,
                            const oracle_attention_shape *s, int num_threads) {
     if (s->num_kv_heads <= 0 || s->num_heads % s->num_kv_heads != 0 || s->block_size <= 0) {
@@ -208,6 +211,9 @@ int oracle_paged_attention(void *out_, const void *q_, const void *k_cache_, con
             uint16_t *o_row = out + seq * s->o_stride + head * s->o_head_stride;
             for (int64_t d = 0; d < s->value_size; ++d) {
                 o_row[d] = store_elem(acc[d] * inv_l, s->dtype);
+                if (out_f32 != NULL) {
+                    out_f32[(seq * s->num_heads + head) * s->value_size + d] = acc[d] * inv_l;
+                }
             }
         }
         free(acc);

@@ -64,7 +64,7 @@ def load():
             build()
         lib = ctypes.CDLL(str(_LIB_PATH))
         common = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, POINTER(AttentionShape)]
-        lib.oracle_paged_attention.argtypes = common + [c_int]
+        lib.oracle_paged_attention.argtypes = [c_void_p] + common + [c_int]
         lib.oracle_paged_attention.restype = c_int
         lib.oracle_paged_attention_splitkv.argtypes = common + [c_int, c_int]
         lib.oracle_paged_attention_splitkv.restype = c_int
@@ -85,9 +85,10 @@ def _cpu(t: torch.Tensor) -> torch.Tensor:
 
 
 def paged_attention(q, k_cache, v_cache, block_tables, seq_lens, scale, alibi_slopes=None, *, out=None,
-                    num_splits: int | None = None, num_threads: int = 1):
+                    num_splits: int | None = None, num_threads: int = 1, return_fp32: bool = False):
     """C oracle on torch CPU tensors (any strides with a packed last dimension). ``num_splits`` selects
-    the split-KV + combine formulation instead of the single pass."""
+    the split-KV + combine formulation instead of the single pass. ``return_fp32`` also returns the
+    result as the kernel holds it before rounding to the storage dtype (rows of empty sequences NaN)."""
     lib = load()
     q, k_cache, v_cache = _cpu(q), _cpu(k_cache), _cpu(v_cache)
     block_tables = _cpu(block_tables).to(torch.int64).contiguous()
@@ -106,15 +107,19 @@ def paged_attention(q, k_cache, v_cache, block_tables, seq_lens, scale, alibi_sl
     if alibi_slopes is not None:
         alibi_slopes = _cpu(alibi_slopes).to(torch.float32).contiguous()
         alibi_ptr = alibi_slopes.data_ptr()
-    args = [out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), block_tables.data_ptr(),
+    args = [q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), block_tables.data_ptr(),
             seq_lens.data_ptr(), alibi_ptr, ctypes.byref(s)]
+    out_f32 = None
     if num_splits is None:
-        rc = lib.oracle_paged_attention(*args, num_threads)
+        if return_fp32:
+            out_f32 = torch.full((q.shape[0], q.shape[1], v_cache.shape[-1]), float("nan"), dtype=torch.float32)
+        rc = lib.oracle_paged_attention(out.data_ptr(), out_f32.data_ptr() if return_fp32 else None, *args, num_threads)
     else:
-        rc = lib.oracle_paged_attention_splitkv(*args, num_splits, num_threads)
+        assert not return_fp32
+        rc = lib.oracle_paged_attention_splitkv(out.data_ptr(), *args, num_splits, num_threads)
     if rc != 0:
         raise ValueError("oracle rejected the arguments")
-    return out
+    return (out, out_f32) if return_fp32 else out
 
 
 def paged_caching(k_cache, v_cache, k, v, slot_mapping):

@@ -1,4 +1,5 @@
 """GPU parity of infiniopPagedCaching (through the C ABI): bit-exact against the CPU oracle."""
+import numpy as np
 import pytest
 import torch
 
@@ -7,18 +8,172 @@ from infinicore_amd import workloads
 from capi import run_paged_caching
 
 pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
 
 
 def bits(t):
-    return t.contiguous().view(torch.int16 if t.element_size() == 2 else torch.int32)
+    t = t.contiguous().cpu()
+    return t.view(torch.int16 if t.element_size() == 2 else torch.int32)
+
+
+def check(gpu_handle, oracle, k_cache, v_cache, k, v, slots, what):
+    """Runs the operator on device copies and the oracle on host copies; pools must match bit for bit."""
+    print("case", what, tuple(k.shape), tuple(k_cache.shape), k.dtype, flush=True)
+    kd, vd = k_cache.to(DEV), v_cache.to(DEV)
+    if not k_cache.is_contiguous():  # keep the permuted view on the device as well
+        kd = k_cache.permute(0, 2, 1, 3).contiguous().to(DEV).permute(0, 2, 1, 3)
+        vd = v_cache.permute(0, 2, 1, 3).contiguous().to(DEV).permute(0, 2, 1, 3)
+    run_paged_caching(gpu_handle, kd, vd, k.to(DEV), v.to(DEV), slots.to(DEV))
+    k_want, v_want = oracle.paged_caching(k_cache.clone(), v_cache.clone(), k, v, slots)
+    assert torch.equal(bits(kd), bits(k_want)), what
+    assert torch.equal(bits(vd), bits(v_want)), what
 
 
 def test_c5_prefill_scatter_bit_exact(gpu_handle, oracle):
     inp = workloads.make_caching_inputs(workloads.CACHING_CONFIGS["c5_prefill_scatter"])
-    dev = torch.device("cuda:0")
-    k_cache, v_cache = inp.k_cache.to(dev), inp.v_cache.to(dev)
-    print("case c5 tokens", inp.k.shape[0], "padding", int((inp.slot_mapping < 0).sum()), flush=True)
-    run_paged_caching(gpu_handle, k_cache, v_cache, inp.k.to(dev), inp.v.to(dev), inp.slot_mapping.to(dev))
-    k_want, v_want = oracle.paged_caching(inp.k_cache.clone(), inp.v_cache.clone(), inp.k, inp.v, inp.slot_mapping)
-    assert torch.equal(bits(k_cache.cpu()), bits(k_want))
-    assert torch.equal(bits(v_cache.cpu()), bits(v_want))
+    check(gpu_handle, oracle, inp.k_cache, inp.v_cache, inp.k, inp.v, inp.slot_mapping, "c5")
+    # 5 % of the tokens are padding: their slots keep the sentinel
+    assert int((inp.slot_mapping < 0).sum()) > 100
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize(
+    "num_seqs,max_seq_len,Hkv,D,bs,Dv",
+    [
+        # test/infiniop/paged_caching.py:61-70
+        (1, 128, 8, 128, 16, 128),
+        (5, 512, 40, 128, 16, 128),
+        (16, 1024, 8, 64, 32, 64),
+        (10, 1024, 40, 64, 32, 64),
+        (2, 128, 1, 576, 16, 512),
+    ],
+)
+def test_reference_test_shapes(gpu_handle, oracle, dtype, num_seqs, max_seq_len, Hkv, D, bs, Dv):
+    """Same construction as the reference test: contiguous slot ranges per sequence in a 4096-page pool
+    (the reference fills the pool with uniform random numbers; a sentinel serves as well)."""
+    rng = np.random.default_rng(num_seqs * 1000 + Hkv + D)
+    lens = rng.integers(1, max_seq_len + 1, size=num_seqs)
+    ntok = int(lens.sum())
+    slots = torch.arange(ntok, dtype=torch.int64)
+    num_blocks = 4096 if dtype != torch.float32 or Hkv < 40 else 1024  # keep host memory modest
+    assert ntok <= num_blocks * bs
+    k = torch.from_numpy(rng.random((ntok, Hkv, D), dtype=np.float32)).to(dtype)
+    v = torch.from_numpy(rng.random((ntok, Hkv, Dv), dtype=np.float32)).to(dtype)
+    k_cache = torch.full((num_blocks, Hkv, bs, D), -3.0, dtype=dtype)
+    v_cache = torch.full((num_blocks, Hkv, bs, Dv), 5.0, dtype=dtype)
+    check(gpu_handle, oracle, k_cache, v_cache, k, v, slots, "reference shape")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_permuted_cache_layout(gpu_handle, oracle, dtype):
+    """Pool stored [pages, rows, heads, d], passed as a [pages, heads, rows, d] view
+    (test/infinicore/ops/paged_caching.py:22-34)."""
+    rng = np.random.default_rng(5)
+    ntok, Hkv, D, bs, NB = 300, 8, 128, 16, 64
+    k = torch.from_numpy(rng.standard_normal((ntok, Hkv, D), dtype=np.float32)).to(dtype)
+    v = torch.from_numpy(rng.standard_normal((ntok, Hkv, D), dtype=np.float32)).to(dtype)
+    slots = torch.from_numpy(rng.permutation(NB * bs)[:ntok].astype(np.int64))
+    k_cache = torch.full((NB, bs, Hkv, D), -777.0, dtype=dtype).permute(0, 2, 1, 3)
+    v_cache = torch.full((NB, bs, Hkv, D), 555.0, dtype=dtype).permute(0, 2, 1, 3)
+    check(gpu_handle, oracle, k_cache, v_cache, k, v, slots, "permuted")
+
+
+def test_strided_source_tokens_and_odd_sizes(gpu_handle, oracle):
+    """Token stride larger than heads * d, a head size that only allows 4-byte copy units, a page size
+    that is not a power of two."""
+    rng = np.random.default_rng(6)
+    ntok, Hkv, D, Dv, bs, NB = 77, 3, 34, 18, 12, 20
+    k_store = torch.from_numpy(rng.standard_normal((ntok, Hkv * D + 10), dtype=np.float32)).to(torch.float16)
+    v_store = torch.from_numpy(rng.standard_normal((ntok, Hkv * Dv + 6), dtype=np.float32)).to(torch.float16)
+    k = k_store[:, :Hkv * D].view(ntok, Hkv, D)
+    v = v_store[:, :Hkv * Dv].view(ntok, Hkv, Dv)
+    assert k.stride(0) == Hkv * D + 10
+    slots = torch.from_numpy(rng.permutation(NB * bs)[:ntok].astype(np.int64))
+    slots[5] = -1
+    k_cache = torch.full((NB, Hkv, bs, D), -777.0, dtype=torch.float16)
+    v_cache = torch.full((NB, Hkv, bs, Dv), 555.0, dtype=torch.float16)
+    kd, vd = k_cache.to(DEV), v_cache.to(DEV)
+    k_dev = k_store.to(DEV)[:, :Hkv * D].view(ntok, Hkv, D)
+    v_dev = v_store.to(DEV)[:, :Hkv * Dv].view(ntok, Hkv, Dv)
+    run_paged_caching(gpu_handle, kd, vd, k_dev, v_dev, slots.to(DEV))
+    k_want, v_want = oracle.paged_caching(k_cache.clone(), v_cache.clone(), k, v, slots)
+    assert torch.equal(bits(kd), bits(k_want)) and torch.equal(bits(vd), bits(v_want))
+
+
+def test_padding_and_out_of_pool_slots_touch_nothing(gpu_handle):
+    """Negative slots are padding (reference kernel.cuh:61-63). Slots beyond the pool would be an
+    out-of-bounds write in the reference; here they are dropped."""
+    ntok, Hkv, D, bs, NB = 64, 4, 128, 16, 8
+    k = torch.ones(ntok, Hkv, D, dtype=torch.bfloat16, device=DEV)
+    v = torch.ones(ntok, Hkv, D, dtype=torch.bfloat16, device=DEV) * 2
+    slots = torch.full((ntok,), -1, dtype=torch.int64, device=DEV)
+    slots[1] = NB * bs          # first slot past the pool
+    slots[2] = 2 ** 40
+    slots[3] = 5                # the only valid one
+    k_cache = torch.zeros(NB, Hkv, bs, D, dtype=torch.bfloat16, device=DEV)
+    v_cache = torch.zeros(NB, Hkv, bs, D, dtype=torch.bfloat16, device=DEV)
+    run_paged_caching(gpu_handle, k_cache, v_cache, k, v, slots)
+    assert torch.all(k_cache[0, :, 5, :] == 1) and torch.all(v_cache[0, :, 5, :] == 2)
+    assert int(k_cache.count_nonzero()) == Hkv * D and int(v_cache.count_nonzero()) == Hkv * D
+
+
+def test_incremental_rounds_with_a_block_allocator(gpu_handle, oracle):
+    """Several rounds of appends, sequences growing page by page from a free list - the scenario of
+    the reference's test/infiniop/paged_caching_prefill.py:97-248."""
+    rng = np.random.default_rng(8)
+    Hkv, D, bs, NB, num_seqs = 8, 128, 16, 256, 5
+    free = list(rng.permutation(NB))
+    tables = [[] for _ in range(num_seqs)]
+    lens = [0] * num_seqs
+    k_cache = torch.zeros(NB, Hkv, bs, D, dtype=torch.bfloat16)
+    v_cache = torch.zeros(NB, Hkv, bs, D, dtype=torch.bfloat16)
+    kd, vd = k_cache.to(DEV), v_cache.to(DEV)
+    for rnd in range(4):
+        slots, chunks = [], []
+        for s in range(num_seqs):
+            new = int(rng.integers(1, 50))
+            for t in range(lens[s], lens[s] + new):
+                if t // bs >= len(tables[s]):
+                    tables[s].append(int(free.pop()))
+                slots.append(tables[s][t // bs] * bs + t % bs)
+            lens[s] += new
+            chunks.append(new)
+        ntok = sum(chunks)
+        k = torch.from_numpy(rng.standard_normal((ntok, Hkv, D), dtype=np.float32)).to(torch.bfloat16)
+        v = torch.from_numpy(rng.standard_normal((ntok, Hkv, D), dtype=np.float32)).to(torch.bfloat16)
+        slot_t = torch.tensor(slots, dtype=torch.int64)
+        run_paged_caching(gpu_handle, kd, vd, k.to(DEV), v.to(DEV), slot_t.to(DEV))
+        oracle.paged_caching(k_cache, v_cache, k, v, slot_t)
+        assert torch.equal(bits(kd), bits(k_cache)) and torch.equal(bits(vd), bits(v_cache)), f"round {rnd}"
+
+
+def test_scatter_then_attend_round_trip(gpu_handle, oracle):
+    """The two operators together: scatter a sequence's K/V into shuffled pages with paged_caching,
+    then decode over it; the result must equal the oracle's attention over the same pool."""
+    from capi import run_paged_attention
+    rng = np.random.default_rng(9)
+    B, H, Hkv, D, bs = 3, 16, 4, 128, 16
+    lens = [100, 257, 33]
+    nb_per = [(n + bs - 1) // bs for n in lens]
+    NB = sum(nb_per) + 5
+    pages = rng.permutation(NB)
+    table = torch.zeros(B, max(nb_per), dtype=torch.int64)
+    slots, cur = [], 0
+    for s, n in enumerate(lens):
+        table[s, :nb_per[s]] = torch.from_numpy(pages[cur:cur + nb_per[s]].astype(np.int64))
+        cur += nb_per[s]
+        slots += [int(table[s, t // bs]) * bs + t % bs for t in range(n)]
+    ntok = sum(lens)
+    k = torch.from_numpy(rng.standard_normal((ntok, Hkv, D), dtype=np.float32)).to(torch.float16)
+    v = torch.from_numpy(rng.standard_normal((ntok, Hkv, D), dtype=np.float32)).to(torch.float16)
+    q = torch.from_numpy(rng.standard_normal((B, H, D), dtype=np.float32)).to(torch.float16)
+    slot_t = torch.tensor(slots, dtype=torch.int64)
+    k_cache = torch.zeros(NB, Hkv, bs, D, dtype=torch.float16)
+    v_cache = torch.zeros(NB, Hkv, bs, D, dtype=torch.float16)
+    kd, vd = k_cache.to(DEV), v_cache.to(DEV)
+    run_paged_caching(gpu_handle, kd, vd, k.to(DEV), v.to(DEV), slot_t.to(DEV))
+    oracle.paged_caching(k_cache, v_cache, k, v, slot_t)
+    sl = torch.tensor(lens, dtype=torch.int64)
+    got = run_paged_attention(gpu_handle, q.to(DEV), kd, vd, table.to(DEV), sl.to(DEV), D ** -0.5)
+    want = oracle.paged_attention(q, k_cache, v_cache, table, sl, D ** -0.5)
+    assert torch.all((got.float().cpu() - want.float()).abs() <= 1e-2 + 2e-3 * want.float().abs())
