@@ -29,6 +29,12 @@ sys.path.insert(0, str(ROOT))
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E
 
+# HBM bytes per launch of the decode kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
+# file, each scaled by what the same counter reads for a 256 MiB copy (summary and commands:
+# profiles/decode_balanced_c2_llama3_8b_b32_hbm_traffic.md). Counters cannot be read from inside this
+# process, so the figure is recorded here; it belongs to the default workload only.
+MEASURED_TRAFFIC_BYTES = {"c2_llama3_8b_b32": 322_300_000}
+
 
 def parse_args():
     ap = argparse.ArgumentParser()
@@ -39,6 +45,9 @@ def parse_args():
     ap.add_argument("--pools", type=int, default=4, help="distinct KV pools the steps rotate over")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-check", action="store_true", help="skip the oracle check of the output")
+    ap.add_argument("--pmc-calibration", action="store_true",
+                    help="also run three plain 256 MiB device copies, so that a rocprofv3 --pmc run of this "
+                         "command records FETCH_SIZE / WRITE_SIZE of a kernel whose traffic is known")
     return ap.parse_args()
 
 
@@ -102,6 +111,14 @@ def main():
             c_void_p(k_pools[p].data_ptr()), c_void_p(v_pools[p].data_ptr()), c_void_p(bt.data_ptr()),
             c_void_p(sl.data_ptr()), c_void_p(0), stream))
 
+    if args.pmc_calibration:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(3)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
     torch.cuda.synchronize()
     for i in range(args.warmup):
         step(i)
@@ -152,9 +169,11 @@ def main():
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": round(gbps_dev / HBM_PEAK_GBPS, 4),
-            "traffic": None,
+            "traffic": MEASURED_TRAFFIC_BYTES.get(cfg.name),
             "us_per_call_device": round(us_dev, 2),
-            "note": "device events bracket the whole call: decode kernel + partition-merge kernel",
+            "note": "achieved = algorithmic bytes / device time per CALL (events on the kernels' stream bracket the "
+                    "decode kernel and the small segment-merge kernel that follows it); traffic = HBM bytes of the "
+                    "decode kernel per launch from rocprofv3 FETCH_SIZE + WRITE_SIZE",
         },
     }
 
