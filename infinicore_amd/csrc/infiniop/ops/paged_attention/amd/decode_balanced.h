@@ -360,9 +360,6 @@ __global__ void __launch_bounds__(256) decodeBalancedMergeKernel(DecodeArgs a) {
     if (head >= a.num_heads) {
         return;
     }
-#ifdef PA_EXPERIMENT_EMPTY_MERGE
-    return;
-#endif
     const int64_t len64 = loadIndex<Tindex>(a.seq_lens, seq);
     const int2 pieces = a.seq_pieces[seq]; // written by the decode kernel for every sequence with tokens
     if (len64 <= 0 || pieces.y <= 1) {

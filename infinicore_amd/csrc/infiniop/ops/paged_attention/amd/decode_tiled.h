@@ -132,17 +132,6 @@ struct TileState {
 template <typename T>
 __device__ __forceinline__ void computeTile(TileState &st, const TileRegs r, const uint4 (&q_reg)[4], uint4 *k_lds,
                                             int c, int g, float scale_log2, float slope, int rel_pos0, int valid) {
-#ifdef PA_EXPERIMENT_NO_COMPUTE
-    {
-        uint4 x = r.k0;
-        x.x ^= r.k1.x ^ r.k2.x ^ r.k3.x ^ r.v0.x ^ r.v1.x ^ r.v2.x ^ r.v3.x;
-        x.y ^= r.k1.y ^ r.k2.y ^ r.k3.y ^ r.v0.y ^ r.v1.y ^ r.v2.y ^ r.v3.y;
-        x.z ^= r.k1.z ^ r.k2.z ^ r.k3.z ^ r.v0.z ^ r.v1.z ^ r.v2.z ^ r.v3.z;
-        x.w ^= r.k1.w ^ r.k2.w ^ r.k3.w ^ r.v0.w ^ r.v1.w ^ r.v2.w ^ r.v3.w;
-        st.l += __uint_as_float((x.x ^ x.y ^ x.z ^ x.w) & 0x007fffffu);
-        return;
-    }
-#endif
     // K: registers -> swizzled LDS -> matrix-operand layout (token c, columns 32*kk + 8g .. +7)
     k_lds[(g) * 16 + (c ^ (g))] = r.k0;
     k_lds[(4 + g) * 16 + (c ^ (4 + g))] = r.k1;
