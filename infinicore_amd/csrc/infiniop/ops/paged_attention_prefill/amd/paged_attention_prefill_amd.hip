@@ -1,0 +1,221 @@
+// paged_attention_prefill on AMD Instinct MI355X: descriptor, kernel choice and launches.
+// Takes the place of the reference's nvidia backend host code
+// (src/infiniop/ops/paged_attention_prefill/nvidia/paged_attention_prefill_nvidia.cu:1572-1886)
+// for the AMD device.
+#include "paged_attention_prefill_amd.h"
+#include "../../../handle.h"
+#include "../../../../utils/check.h"
+#include "../../../devices/amd/amd_device.h"
+#include "prefill_common.h"
+#include "prefill_generic.h"
+#include "prefill_tiled.h"
+#include <cstdlib>
+#include <cstring>
+
+namespace op::paged_attention_prefill::amd {
+
+namespace {
+
+using op::paged_attention::amd::BFloat16;
+using op::paged_attention::amd::Half;
+using op::paged_attention::amd::IndexI32;
+using op::paged_attention::amd::IndexI64;
+using op::paged_attention::amd::IndexU32;
+
+// Decided once, at descriptor creation, from shapes and the device alone (sequence lengths live in
+// device memory and are never read on the host).
+struct Plan {
+    bool tiled;          // matrix-core kernel (head 128, power-of-two pages >= 8, 16-byte aligned strides)
+    int groups_per_wave; // tiled: R = 1, 2 or 4 column groups per wavefront -> 64 R rows per workgroup
+    int dims_per_lane;   // element-wise kernel: ceil(max(head_size, value_size) / 64)
+};
+
+bool multipleOf8(ptrdiff_t x) { return (x % 8) == 0; }
+
+Plan makePlan(const PagedAttentionPrefillInfo &in, const device::amd::DeviceInfo &dev) {
+    Plan plan{};
+    const long long bs = static_cast<long long>(in.page_block_size);
+    const bool pow2_page = bs >= 8 && (bs & (bs - 1)) == 0;
+    const long long group = static_cast<long long>(in.num_heads / in.num_kv_heads);
+    const long long rows = static_cast<long long>(in.total_q_tokens) * group; // per KV head
+    plan.tiled = in.head_size == kPrefillHead && in.value_size == kPrefillHead && pow2_page
+              && multipleOf8(in.q_stride) && multipleOf8(in.q_head_stride) && multipleOf8(in.o_stride)
+              && multipleOf8(in.o_head_stride) && multipleOf8(in.k_batch_stride) && multipleOf8(in.k_head_stride)
+              && multipleOf8(in.k_row_stride) && multipleOf8(in.v_batch_stride) && multipleOf8(in.v_head_stride)
+              && multipleOf8(in.v_row_stride) && in.num_blocks > 0 && in.num_blocks <= 0x7fffffff
+              && rows < (1LL << 30) && in.num_kv_heads <= 65535
+              && static_cast<long long>(in.max_num_blocks_per_seq) * bs < (1LL << 30);
+    if (const char *env = std::getenv("INFINIOP_AMD_PREFILL_KERNEL")) {
+        if (std::strcmp(env, "generic") == 0) {
+            plan.tiled = false;
+        }
+    }
+    // Rows per workgroup: as many as the average sequence fills, but keep at least two workgroups
+    // per compute unit in flight when the batch is large enough to allow it.
+    const long long seqs = in.num_seqs > 0 ? static_cast<long long>(in.num_seqs) : 1;
+    const long long rows_per_seq = rows / seqs;
+    int r = 4;
+    while (r > 1 && (rows_per_seq <= 32LL * r || rows / (64LL * r) * static_cast<long long>(in.num_kv_heads) < 2LL * dev.compute_units)) {
+        r /= 2;
+    }
+    if (const char *env = std::getenv("INFINIOP_AMD_PREFILL_GROUPS")) {
+        const int forced = std::atoi(env);
+        if (forced == 1 || forced == 2 || forced == 4) {
+            r = forced;
+        }
+    }
+    plan.groups_per_wave = r;
+    const size_t widest = in.head_size > in.value_size ? in.head_size : in.value_size;
+    plan.dims_per_lane = static_cast<int>((widest + 63) / 64);
+    return plan;
+}
+
+template <typename T, typename Tindex>
+void launchGeneric(const PrefillArgs &a, const Plan &plan, hipStream_t stream) {
+    const dim3 grid(a.total_q_tokens, a.num_heads);
+    switch (plan.dims_per_lane) {
+    case 1: prefillGenericKernel<T, Tindex, 1><<<grid, 64, 0, stream>>>(a); break;
+    case 2: prefillGenericKernel<T, Tindex, 2><<<grid, 64, 0, stream>>>(a); break;
+    case 3: prefillGenericKernel<T, Tindex, 3><<<grid, 64, 0, stream>>>(a); break;
+    case 4: prefillGenericKernel<T, Tindex, 4><<<grid, 64, 0, stream>>>(a); break;
+    default: prefillGenericKernel<T, Tindex, 9><<<grid, 64, 0, stream>>>(a); break;
+    }
+}
+
+template <typename T, typename Tindex>
+void launchTiled(const PrefillArgs &a, const Plan &plan, hipStream_t stream) {
+    // sum over sequences of ceil(rows / block_rows) is at most floor(total rows / block_rows) + num_seqs
+    const long long rows = static_cast<long long>(a.total_q_tokens) * a.group;
+    const int block_rows = prefillBlockRows(plan.groups_per_wave);
+    const dim3 grid(static_cast<unsigned>(rows / block_rows + a.num_seqs), a.num_kv_heads);
+    switch (plan.groups_per_wave) {
+    case 1: prefillTiledKernel<T, Tindex, 1><<<grid, kPrefillThreads, 0, stream>>>(a); break;
+    case 2: prefillTiledKernel<T, Tindex, 2><<<grid, kPrefillThreads, 0, stream>>>(a); break;
+    default: prefillTiledKernel<T, Tindex, 4><<<grid, kPrefillThreads, 0, stream>>>(a); break;
+    }
+}
+
+template <typename T>
+infiniStatus_t launchByIndex(infiniDtype_t index_dtype, const PrefillArgs &a, const Plan &plan, bool tiled,
+                             hipStream_t stream) {
+    switch (index_dtype) {
+    case INFINI_DTYPE_I64:
+        tiled ? launchTiled<T, IndexI64>(a, plan, stream) : launchGeneric<typename T::Base, IndexI64>(a, plan, stream);
+        break;
+    case INFINI_DTYPE_I32:
+        tiled ? launchTiled<T, IndexI32>(a, plan, stream) : launchGeneric<typename T::Base, IndexI32>(a, plan, stream);
+        break;
+    case INFINI_DTYPE_U32:
+        tiled ? launchTiled<T, IndexU32>(a, plan, stream) : launchGeneric<typename T::Base, IndexU32>(a, plan, stream);
+        break;
+    default: return INFINI_STATUS_BAD_TENSOR_DTYPE;
+    }
+    return INFINI_STATUS_SUCCESS;
+}
+
+bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+} // namespace
+
+struct Descriptor::Opaque {
+    Plan plan;
+};
+
+Descriptor::~Descriptor() { delete _opaque; }
+
+infiniStatus_t Descriptor::create(infiniopHandle_t handle, Descriptor **desc_ptr, infiniopTensorDescriptor_t out_desc,
+                                  infiniopTensorDescriptor_t q_desc, infiniopTensorDescriptor_t k_cache_desc,
+                                  infiniopTensorDescriptor_t v_cache_desc, infiniopTensorDescriptor_t block_tables_desc,
+                                  infiniopTensorDescriptor_t seq_lens_desc, infiniopTensorDescriptor_t cum_seq_lens_q_desc,
+                                  infiniopTensorDescriptor_t alibi_slopes_desc, float scale) {
+    auto info = PagedAttentionPrefillInfo::create(out_desc, q_desc, k_cache_desc, v_cache_desc, block_tables_desc,
+                                                  seq_lens_desc, cum_seq_lens_q_desc, alibi_slopes_desc, scale);
+    CHECK_RESULT(info);
+    const PagedAttentionPrefillInfo in = info.take();
+    const Plan plan = makePlan(in, device::amd::deviceInfo(handle->device_id));
+    // every row block keeps its softmax state in registers from the first to the last K/V token: no scratch
+    *desc_ptr = new Descriptor(new Opaque{plan}, in, 0, handle->device, handle->device_id);
+    return INFINI_STATUS_SUCCESS;
+}
+
+infiniStatus_t Descriptor::calculate(void *workspace, size_t workspace_size, void *out, const void *q,
+                                     const void *k_cache, const void *v_cache, const void *block_tables,
+                                     const void *seq_lens, const void *cum_seq_lens_q, const void *alibi_slopes,
+                                     void *stream_) const {
+    (void)workspace;
+    const PagedAttentionPrefillInfo &in = _info;
+    const Plan &plan = _opaque->plan;
+    if (workspace_size < _workspace_size) {
+        return INFINI_STATUS_INSUFFICIENT_WORKSPACE;
+    }
+    if (in.num_seqs == 0 || in.num_heads == 0 || in.total_q_tokens == 0) {
+        return INFINI_STATUS_SUCCESS;
+    }
+    if (out == nullptr || q == nullptr || k_cache == nullptr || v_cache == nullptr || block_tables == nullptr
+        || seq_lens == nullptr || cum_seq_lens_q == nullptr) {
+        return INFINI_STATUS_NULL_POINTER;
+    }
+    if (in.has_alibi && alibi_slopes == nullptr) {
+        return INFINI_STATUS_NULL_POINTER;
+    }
+    if (in.max_num_blocks_per_seq == 0 || in.num_blocks == 0 || in.page_block_size == 0) {
+        return INFINI_STATUS_SUCCESS; // no sequence can hold a token
+    }
+    if (in.total_q_tokens > 0x7fffffff || in.num_seqs > 0x7fffffff || in.num_heads > 65535) {
+        return INFINI_STATUS_BAD_TENSOR_SHAPE;
+    }
+
+    PrefillArgs a{};
+    a.out = out;
+    a.q = q;
+    a.k_cache = k_cache;
+    a.v_cache = v_cache;
+    a.block_tables = block_tables;
+    a.kv_lens = seq_lens;
+    a.cu_seqlens_q = cum_seq_lens_q;
+    a.alibi_slopes = static_cast<const float *>(alibi_slopes);
+    a.scale_log2 = in.scale * kLog2e;
+    a.num_seqs = static_cast<int32_t>(in.num_seqs);
+    a.total_q_tokens = static_cast<int32_t>(in.total_q_tokens);
+    a.num_heads = static_cast<int32_t>(in.num_heads);
+    a.num_kv_heads = static_cast<int32_t>(in.num_kv_heads);
+    a.group = static_cast<int32_t>(in.num_heads / in.num_kv_heads);
+    a.head_size = static_cast<int32_t>(in.head_size);
+    a.value_size = static_cast<int32_t>(in.value_size);
+    a.block_size = static_cast<int32_t>(in.page_block_size);
+    a.block_shift = -1;
+    if ((in.page_block_size & (in.page_block_size - 1)) == 0) {
+        a.block_shift = __builtin_ctzll(in.page_block_size);
+    }
+    a.num_blocks = static_cast<int32_t>(in.num_blocks > 0x7fffffff ? 0x7fffffff : in.num_blocks);
+    a.max_blocks_per_seq = static_cast<int32_t>(in.max_num_blocks_per_seq > 0x7fffffff ? 0x7fffffff : in.max_num_blocks_per_seq);
+    a.q_stride = in.q_stride;
+    a.q_head_stride = in.q_head_stride;
+    a.o_stride = in.o_stride;
+    a.o_head_stride = in.o_head_stride;
+    a.k_batch_stride = in.k_batch_stride;
+    a.k_head_stride = in.k_head_stride;
+    a.k_row_stride = in.k_row_stride;
+    a.v_batch_stride = in.v_batch_stride;
+    a.v_head_stride = in.v_head_stride;
+    a.v_row_stride = in.v_row_stride;
+    a.block_table_batch_stride = in.block_table_batch_stride;
+
+    // The tiled kernel moves 16 bytes per lane; base addresses that are not 16-byte aligned take
+    // the element-wise kernel instead.
+    const bool tiled = plan.tiled && aligned16(out) && aligned16(q) && aligned16(k_cache) && aligned16(v_cache);
+    auto stream = static_cast<hipStream_t>(stream_);
+
+    infiniStatus_t status;
+    if (in.dtype == INFINI_DTYPE_F16) {
+        status = launchByIndex<TileF16>(in.index_dtype, a, plan, tiled, stream);
+    } else {
+        status = launchByIndex<TileBF16>(in.index_dtype, a, plan, tiled, stream);
+    }
+    if (status != INFINI_STATUS_SUCCESS) {
+        return status;
+    }
+    return hipGetLastError() == hipSuccess ? INFINI_STATUS_SUCCESS : INFINI_STATUS_INTERNAL_ERROR;
+}
+
+} // namespace op::paged_attention_prefill::amd

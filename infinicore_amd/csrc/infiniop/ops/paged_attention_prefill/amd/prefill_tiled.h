@@ -1,0 +1,377 @@
+// Tiled prefill kernel for head_size = value_size = 128 on gfx950 (CDNA4, 64-lane wavefronts).
+//
+// Work unit: one 256-thread workgroup = 64*R "rows" of one (sequence, KV head). A row is a (new
+// token, query head of the KV head's group) pair, token-major: row = token * group + head_in_group.
+// Packing the heads of a group into the row dimension means a K/V tile fetched once serves all of
+// them, and short prompts still fill the matrix instructions. Each of the four wavefronts owns 16*R
+// consecutive rows (R column groups of 16).
+//
+// The K/V tokens the rows may see are consumed in steps of 64. Per step the workgroup copies
+// 64 K rows and 64 V rows (16 KiB each) from the paged pool into LDS, every wavefront 16 tokens of
+// each, double-buffered: the global loads of step j+1 are in flight while step j is computed, and one
+// barrier per step separates writers and readers.
+//   * K is stored as it comes (16-byte chunks, XOR-swizzled so the later row-wise reads are
+//     conflict-free): the matrix instruction wants lane i to hold token i.
+//   * V is stored already transposed into matrix-operand order: the lane that loaded rows 4g..4g+3
+//     of an 8-column strip interleaves them per column with byte permutes and writes, for each of
+//     its 8 columns, the four tokens as one 8-byte word. A reader fetches two such words (tokens
+//     4g..4g+3 of two 16-token tiles) and has the 8-deep operand of one 16x16x32 instruction.
+//
+// Arithmetic per step and column group, lane = 16*g + c:
+//   S[token][row] = K . Q^T   16 x v_mfma_f32_16x16x32 (A = K tile from LDS, B = Q held in registers
+//                             for the whole kernel; lane holds S[16T + 4g + 0..3][row c], T = 0..3)
+//   causal mask (only in steps that touch the diagonal), online softmax in fp32 / log2 domain
+//   O[row][dim] += P . V      16 x v_mfma_f32_16x16x32 (A = P rounded to the storage dtype, straight
+//                             from the registers S came out in; B = V words from LDS; lane holds
+//                             O[row 4g + 0..3][8c + e], e = 0..7)
+// K/V fragments read from LDS are shared by the R column groups of a wavefront. The denominator sums
+// the rounded probabilities. A step whose tokens lie beyond everything a wavefront's rows may see
+// is skipped by that wavefront (it still takes part in the copy).
+//
+// The math follows the reference's prefill kernels (src/infiniop/ops/paged_attention_prefill/cuda/
+// kernel_v2.cuh:254-472: visible range, ALiBi distance, 1e-6 in the normaliser, rounding).
+#ifndef INFINICORE_AMD_PA_PREFILL_TILED_H
+#define INFINICORE_AMD_PA_PREFILL_TILED_H
+
+#include "../../paged_attention/amd/decode_tiled.h"
+#include "prefill_common.h"
+
+namespace op::paged_attention_prefill::amd {
+
+using op::paged_attention::amd::f32x4;
+using op::paged_attention::amd::maxAcrossTokenGroups;
+using op::paged_attention::amd::sumAcrossTokenGroups;
+using op::paged_attention::amd::TileBF16;
+using op::paged_attention::amd::TileF16;
+
+constexpr int kPrefillThreads = 256;
+constexpr int kPrefillStepTokens = 64;
+constexpr int kPrefillHead = 128;
+
+// Rows of one workgroup for R column groups per wavefront.
+__host__ __device__ constexpr int prefillBlockRows(int r) { return 64 * r; }
+
+// Which (sequence, row block) workgroup `x` of a KV head works on. Blocks are numbered from the last
+// block of the last sequence backwards, so that within a sequence the blocks that see the most
+// tokens start first. Every wavefront runs this on its own (no LDS, no barrier); all values are
+// wave-uniform. Returns false for a workgroup beyond the last block.
+template <typename Tindex>
+__device__ __forceinline__ bool findRowBlock(const PrefillArgs &a, int lane, int block_rows, int x, int &seq, int &block) {
+    int running = 0;
+    for (int base = 0; base < a.num_seqs; base += 64) {
+        const int idx = base + lane;
+        const int s = a.num_seqs - 1 - idx;
+        int nb = 0;
+        if (idx < a.num_seqs) {
+            const SeqSpan span = loadSeqSpan<Tindex>(a, s);
+            const int64_t rows = static_cast<int64_t>(span.q_len) * a.group;
+            nb = rows > 0 ? static_cast<int>((rows + block_rows - 1) / block_rows) : 0;
+        }
+        int incl = nb;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const int y = __shfl_up(incl, off, 64);
+            incl += lane >= off ? y : 0;
+        }
+        incl += running;
+        const unsigned long long hit = __builtin_amdgcn_ballot_w64(incl > x);
+        if (hit != 0) {
+            const int first = __builtin_ctzll(hit);
+            const int incl_f = __builtin_amdgcn_readlane(incl, first);
+            const int nb_f = __builtin_amdgcn_readlane(nb, first);
+            seq = a.num_seqs - 1 - (base + first);
+            block = nb_f - 1 - (x - (incl_f - nb_f));
+            return true;
+        }
+        running = __builtin_amdgcn_readlane(incl, 63);
+    }
+    return false;
+}
+
+template <typename T, typename Tindex, int R>
+__global__ void __launch_bounds__(kPrefillThreads) prefillTiledKernel(PrefillArgs a) {
+    using S = typename T::storage;
+    constexpr int BM = prefillBlockRows(R);
+    __shared__ uint4 k_lds[2][kPrefillStepTokens * 16];    // [token][16-byte chunk ^ (token & 15)]
+    __shared__ uint2 v_lds[2][8 * 4 * 4 * 16];             // [column e][16-token tile][token group g][strip c]
+
+    const int lane = threadIdx.x & 63;
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int c = lane & 15;
+    const int g = lane >> 4;
+    const int kv_head = blockIdx.y;
+
+    int seq = 0, block = 0;
+    if (!findRowBlock<Tindex>(a, lane, BM, blockIdx.x, seq, block)) {
+        return;
+    }
+    const SeqSpan span = loadSeqSpan<Tindex>(a, seq);
+    const int total_rows = span.q_len * a.group; // > 0 here
+    const int block_row0 = block * BM;
+    const int last_row = min(block_row0 + BM, total_rows) - 1;
+    // tokens the block's last row may see = the most any of its rows may see
+    const int block_visible = __builtin_amdgcn_readfirstlane(visibleTokens(span, last_row / a.group));
+    if (block_visible <= 0) {
+        return;
+    }
+    int64_t kv_len64 = loadIndex<Tindex>(a.kv_lens, seq);
+    kv_len64 = kv_len64 < 0 ? 0 : (kv_len64 > span.capacity ? span.capacity : kv_len64);
+    // tokens that exist; rows beyond it are zeroed in V (they may hold anything, NaN included)
+    const int kv_len = __builtin_amdgcn_readfirstlane(max(static_cast<int>(kv_len64), block_visible));
+    const int n_steps = (block_visible + kPrefillStepTokens - 1) / kPrefillStepTokens;
+
+    // ---- this lane's columns: row c of each of the wavefront's R column groups ----
+    uint4 q_reg[R][4];
+    int visible[R];
+    float slope[R];
+    int wave_max_visible = 0, wave_min_visible = 0x7fffffff;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int row = block_row0 + (w * R + r) * 16 + c;
+        const bool valid = row < total_rows;
+        const int token = valid ? row / a.group : 0;
+        const int head = kv_head * a.group + (valid ? row - token * a.group : 0);
+        visible[r] = valid ? visibleTokens(span, token) : 0;
+        slope[r] = (a.alibi_slopes != nullptr && valid) ? a.alibi_slopes[head] * kLog2e : 0.0f;
+        const S *q_ptr = static_cast<const S *>(a.q) + (span.q_start + token) * a.q_stride + head * a.q_head_stride;
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) {
+            q_reg[r][kk] = valid ? *reinterpret_cast<const uint4 *>(q_ptr + 32 * kk + 8 * g) : make_uint4(0, 0, 0, 0);
+        }
+        wave_max_visible = max(wave_max_visible, visible[r]);
+        wave_min_visible = min(wave_min_visible, valid ? visible[r] : 0x7fffffff);
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        wave_max_visible = max(wave_max_visible, __shfl_xor(wave_max_visible, off, 64));
+        wave_min_visible = min(wave_min_visible, __shfl_xor(wave_min_visible, off, 64));
+    }
+    wave_max_visible = __builtin_amdgcn_readfirstlane(wave_max_visible);
+    wave_min_visible = __builtin_amdgcn_readfirstlane(wave_min_visible);
+
+    // ---- copy side: this wavefront moves tokens [64 j + 16 w, +16) of step j ----
+    const char *k_head = reinterpret_cast<const char *>(static_cast<const S *>(a.k_cache) + kv_head * a.k_head_stride);
+    const char *v_head = reinterpret_cast<const char *>(static_cast<const S *>(a.v_cache) + kv_head * a.v_head_stride);
+    const int64_t table_row = seq * a.block_table_batch_stride;
+    const int block_mask = a.block_size - 1;
+    const bool small_pages = a.block_size < 16; // pages of 8 tokens: a 16-token tile spans two
+    const int last_entry = (kv_len - 1) >> a.block_shift;
+
+    // page ids of the 16-token tile that starts at token t (wave-uniform)
+    auto loadPageIds = [&](int t, int &id0, int &id1) {
+        id0 = 0;
+        id1 = 0;
+        if (t < kv_len) {
+            const int e0 = t >> a.block_shift;
+            id0 = clampPage(loadIndex<Tindex>(a.block_tables, table_row + e0), a.num_blocks);
+            id1 = id0;
+            if (small_pages && e0 + 1 <= last_entry) {
+                id1 = clampPage(loadIndex<Tindex>(a.block_tables, table_row + e0 + 1), a.num_blocks);
+            }
+        }
+    };
+    uint4 k_stage[4], v_stage[4];
+    auto loadStage = [&](int t, int id0, int id1) {
+        // K: rows 4 jj + g of the tile; V: rows 4 g + i. Tokens past kv_len are not fetched.
+        const int row0 = small_pages ? 0 : (t & block_mask);
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj) {
+            const int o = 4 * jj + g;
+            const int page = (small_pages && jj >= 2) ? id1 : id0;
+            const int page_row = small_pages ? (o & 7) : row0 + o;
+            const char *src = k_head + (page * a.k_batch_stride + page_row * a.k_row_stride) * static_cast<int64_t>(sizeof(S)) + 16 * c;
+            k_stage[jj] = (t + o < kv_len) ? *reinterpret_cast<const uint4 *>(src) : make_uint4(0, 0, 0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int o = 4 * g + i;
+            const int page = (small_pages && g >= 2) ? id1 : id0;
+            const int page_row = small_pages ? (o & 7) : row0 + o;
+            const char *src = v_head + (page * a.v_batch_stride + page_row * a.v_row_stride) * static_cast<int64_t>(sizeof(S)) + 16 * c;
+            v_stage[i] = (t + o < kv_len) ? *reinterpret_cast<const uint4 *>(src) : make_uint4(0, 0, 0, 0);
+        }
+    };
+    auto storeStage = [&](int buf) {
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj) {
+            const int o = 4 * jj + g;
+            k_lds[buf][(16 * w + o) * 16 + (c ^ o)] = k_stage[jj];
+        }
+        typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+        const u32x4 v0 = __builtin_bit_cast(u32x4, v_stage[0]), v1 = __builtin_bit_cast(u32x4, v_stage[1]);
+        const u32x4 v2 = __builtin_bit_cast(u32x4, v_stage[2]), v3 = __builtin_bit_cast(u32x4, v_stage[3]);
+#pragma unroll
+        for (int wd = 0; wd < 4; ++wd) {
+            uint2 even, odd;
+            even.x = __builtin_amdgcn_perm(v1[wd], v0[wd], 0x05040100u);
+            even.y = __builtin_amdgcn_perm(v3[wd], v2[wd], 0x05040100u);
+            odd.x = __builtin_amdgcn_perm(v1[wd], v0[wd], 0x07060302u);
+            odd.y = __builtin_amdgcn_perm(v3[wd], v2[wd], 0x07060302u);
+            v_lds[buf][(((2 * wd) * 4 + w) * 4 + g) * 16 + c] = even;
+            v_lds[buf][(((2 * wd + 1) * 4 + w) * 4 + g) * 16 + c] = odd;
+        }
+    };
+
+    // ---- softmax state: o[r][e][rr] = O[row 4g+rr of group r][column 8c+e] ----
+    f32x4 o[R][8];
+    float m[R], l[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            o[r][e] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+        m[r] = -INFINITY;
+        l[r] = 0.0f;
+    }
+
+    auto computeStep = [&](int buf, int t0) {
+        f32x4 s[R][4];
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+#pragma unroll
+            for (int tt = 0; tt < 4; ++tt) {
+                s[r][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
+            }
+        }
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt) {
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk) {
+                const uint4 kf = k_lds[buf][(16 * tt + c) * 16 + ((4 * kk + g) ^ c)];
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    s[r][tt] = T::mfmaK32(kf, q_reg[r][kk], s[r][tt]);
+                }
+            }
+        }
+
+        const bool on_diagonal = t0 + kPrefillStepTokens > wave_min_visible; // some score of this step is masked
+        const bool has_alibi = a.alibi_slopes != nullptr;
+        uint4 p_op[R][2];
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            float sc[4][4];
+            float mx = -INFINITY;
+#pragma unroll
+            for (int tt = 0; tt < 4; ++tt) {
+#pragma unroll
+                for (int rr = 0; rr < 4; ++rr) {
+                    const int tok = t0 + 16 * tt + 4 * g + rr;
+                    float x = s[r][tt][rr] * a.scale_log2;
+                    if (has_alibi) {
+                        x += slope[r] * static_cast<float>(tok - (visible[r] - 1));
+                    }
+                    x = (on_diagonal && tok >= visible[r]) ? -INFINITY : x;
+                    sc[tt][rr] = x;
+                    mx = fmaxf(mx, x);
+                }
+            }
+            mx = maxAcrossTokenGroups(mx);
+            const float m_new = fmaxf(m[r], mx);
+            if (__builtin_amdgcn_ballot_w64(m_new > m[r]) != 0) {
+                // some row's maximum moved: rescale. Lane holds accumulators of rows 4g..4g+3, whose
+                // factors live in lanes 4g..4g+3.
+                const float alpha = m_new > m[r] ? fastExp2(m[r] - m_new) : 1.0f;
+                l[r] *= alpha;
+                m[r] = m_new;
+#pragma unroll
+                for (int rr = 0; rr < 4; ++rr) {
+                    const float alpha_r = __shfl(alpha, 4 * g + rr, 64);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        o[r][e][rr] *= alpha_r;
+                    }
+                }
+            }
+            const float m_use = m[r] == -INFINITY ? 0.0f : m[r]; // a row that has seen nothing yet: p = 2^-inf = 0
+            float p_sum = 0.0f;
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                uint32_t wds[4];
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const int tt = 2 * u + h;
+                    wds[2 * h] = T::pack2(fastExp2(sc[tt][0] - m_use), fastExp2(sc[tt][1] - m_use));
+                    wds[2 * h + 1] = T::pack2(fastExp2(sc[tt][2] - m_use), fastExp2(sc[tt][3] - m_use));
+                }
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    p_sum += T::unpackLo(wds[i]) + T::unpackHi(wds[i]);
+                }
+                p_op[r][u] = make_uint4(wds[0], wds[1], wds[2], wds[3]);
+            }
+            l[r] += p_sum;
+        }
+
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const uint2 lo = v_lds[buf][((e * 4 + 2 * u) * 4 + g) * 16 + c];
+                const uint2 hi = v_lds[buf][((e * 4 + 2 * u + 1) * 4 + g) * 16 + c];
+                const uint4 vf = make_uint4(lo.x, lo.y, hi.x, hi.y);
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    o[r][e] = T::mfmaK32(p_op[r][u], vf, o[r][e]);
+                }
+            }
+        }
+    };
+
+    // ---- pipeline ----
+    int id0, id1, next_id0, next_id1;
+    loadPageIds(16 * w, id0, id1);
+    loadStage(16 * w, id0, id1);
+    loadPageIds(kPrefillStepTokens + 16 * w, id0, id1);
+    storeStage(0);
+    __syncthreads();
+    if (n_steps > 1) {
+        loadStage(kPrefillStepTokens + 16 * w, id0, id1);
+    }
+    loadPageIds(2 * kPrefillStepTokens + 16 * w, next_id0, next_id1);
+    for (int j = 0; j < n_steps; ++j) {
+        const int t0 = j * kPrefillStepTokens;
+        if (t0 < wave_max_visible) {
+            computeStep(j & 1, t0);
+        }
+        if (j + 1 < n_steps) {
+            storeStage((j + 1) & 1);
+        }
+        __syncthreads();
+        if (j + 2 < n_steps) {
+            loadStage((j + 2) * kPrefillStepTokens + 16 * w, next_id0, next_id1);
+            loadPageIds((j + 3) * kPrefillStepTokens + 16 * w, next_id0, next_id1);
+        }
+    }
+
+    // ---- normalise and store: lane writes columns 8c..8c+7 of rows 4g..4g+3 of each group ----
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const float l_tot = sumAcrossTokenGroups(l[r]);
+#pragma unroll
+        for (int rr = 0; rr < 4; ++rr) {
+            const int src_lane = 4 * g + rr;
+            const float l_row = __shfl(l_tot, src_lane, 64);
+            const int visible_row = __shfl(visible[r], src_lane, 64);
+            const int row = block_row0 + (w * R + r) * 16 + src_lane;
+            if (row >= total_rows || visible_row <= 0) {
+                continue;
+            }
+            const int token = row / a.group;
+            const int head = kv_head * a.group + (row - token * a.group);
+            const float inv_l = 1.0f / (l_row + 1e-6f);
+            uint4 packed;
+            packed.x = T::pack2(o[r][0][rr] * inv_l, o[r][1][rr] * inv_l);
+            packed.y = T::pack2(o[r][2][rr] * inv_l, o[r][3][rr] * inv_l);
+            packed.z = T::pack2(o[r][4][rr] * inv_l, o[r][5][rr] * inv_l);
+            packed.w = T::pack2(o[r][6][rr] * inv_l, o[r][7][rr] * inv_l);
+            S *o_ptr = static_cast<S *>(a.out) + (span.q_start + token) * a.o_stride + head * a.o_head_stride;
+            *reinterpret_cast<uint4 *>(o_ptr + 8 * c) = packed;
+        }
+    }
+}
+
+} // namespace op::paged_attention_prefill::amd
+
+#endif

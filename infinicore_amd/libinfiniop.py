@@ -152,6 +152,12 @@ def _open():
     _declare(op, "infiniopPagedAttention", [D, vp, c_size_t, vp, vp, vp, vp, vp, vp, vp, vp])
     _declare(op, "infiniopDestroyPagedAttentionDescriptor", [D])
 
+    # ---- paged_attention_prefill ----
+    _declare(op, "infiniopCreatePagedAttentionPrefillDescriptor", [infiniopHandle_t, POINTER(D), T, T, T, T, T, T, T, T, c_float])
+    _declare(op, "infiniopGetPagedAttentionPrefillWorkspaceSize", [D, POINTER(c_size_t)])
+    _declare(op, "infiniopPagedAttentionPrefill", [D, vp, c_size_t, vp, vp, vp, vp, vp, vp, vp, vp, vp])
+    _declare(op, "infiniopDestroyPagedAttentionPrefillDescriptor", [D])
+
     # ---- paged_caching ----
     _declare(op, "infiniopCreatePagedCachingDescriptor", [infiniopHandle_t, POINTER(D), T, T, T, T, T])
     _declare(op, "infiniopGetPagedCachingWorkspaceSize", [D, POINTER(c_size_t)])

@@ -1,7 +1,8 @@
-"""``paged_attention`` / ``paged_caching`` on torch CUDA tensors, executed by ``libinfiniop.so``.
+"""``paged_attention`` / ``paged_attention_prefill`` / ``paged_caching`` on torch CUDA tensors, executed by ``libinfiniop.so``.
 
 Argument order and meaning are those of the reference's Python operators
-(``python/infinicore/ops/paged_attention.py:5-40``, ``python/infinicore/ops/paged_caching.py:5-21``).
+(``python/infinicore/ops/paged_attention.py:5-40``, ``python/infinicore/ops/paged_attention_prefill.py:5-45``,
+``python/infinicore/ops/paged_caching.py:5-21``).
 What the reference's C++ adaptor does between that call and the C API
 (``src/infinicore/ops/paged_attention/paged_attention_infiniop.cc:16-58``: build tensor descriptors,
 fetch or create a cached operator descriptor keyed by the tensors' metadata, allocate a byte
@@ -136,6 +137,53 @@ def paged_attention(q, k_cache, v_cache, block_tables, cache_lens, alibi_slopes=
             _ptr(v_cache), _ptr(block_tables), _ptr(cache_lens), _ptr(alibi_slopes), _stream_ptr(index),
         ),
         "infiniopPagedAttention",
+    )
+    return out
+
+
+def paged_attention_prefill(q, k_cache, v_cache, block_tables, seq_lens, cum_seq_lens_q, alibi_slopes=None,
+                            scale: float = 1.0, *, out=None):
+    """Causal attention of each sequence's run of new tokens over its paged K/V; returns ``out``.
+
+    q [total_q_tokens, num_heads, head_size] holds the new tokens of all sequences back to back;
+    seq_lens [num_seqs] are the total K/V lengths (history + new), cum_seq_lens_q [num_seqs + 1] the
+    prefix sums of the new-token counts; both and block_tables share one index dtype.
+    """
+    index = _device_index(q)
+    if out is None:
+        out = torch.empty((*q.shape[:-1], v_cache.shape[-1]), dtype=q.dtype, device=q.device)
+    tensors = (out, q, k_cache, v_cache, block_tables, seq_lens, cum_seq_lens_q)
+    key = ("paged_attention_prefill", index, float(scale), *(_meta(t) for t in tensors), _meta(alibi_slopes))
+
+    def make():
+        handle = _handle_for(index)
+        descs = [_describe(t) for t in tensors]
+        alibi_desc = _describe(alibi_slopes) if alibi_slopes is not None else lib.infiniopTensorDescriptor_t()
+        op = lib.infiniopOperatorDescriptor_t()
+        try:
+            check_error(
+                LIBINFINIOP.infiniopCreatePagedAttentionPrefillDescriptor(handle, ctypes.byref(op), *descs, alibi_desc,
+                                                                          scale),
+                "infiniopCreatePagedAttentionPrefillDescriptor",
+            )
+        finally:
+            for d in descs:
+                lib.destroy_tensor_descriptor(d)
+            if alibi_slopes is not None:
+                lib.destroy_tensor_descriptor(alibi_desc)
+        size = c_size_t(0)
+        check_error(LIBINFINIOP.infiniopGetPagedAttentionPrefillWorkspaceSize(op, ctypes.byref(size)))
+        return _Plan(op, LIBINFINIOP.infiniopDestroyPagedAttentionPrefillDescriptor, size.value, q.device)
+
+    plan = _cached_plan(key, make)
+    lib.set_device(InfiniDevice.AMD, index)
+    check_error(
+        LIBINFINIOP.infiniopPagedAttentionPrefill(
+            plan.descriptor, _ptr(plan.workspace), plan.workspace_bytes, _ptr(out), _ptr(q), _ptr(k_cache),
+            _ptr(v_cache), _ptr(block_tables), _ptr(seq_lens), _ptr(cum_seq_lens_q), _ptr(alibi_slopes),
+            _stream_ptr(index),
+        ),
+        "infiniopPagedAttentionPrefill",
     )
     return out
 

@@ -3,7 +3,8 @@
 Every generator is a pure function of its seed (numpy PCG64), so the CPU container and the GPU box
 build bit-identical inputs. Shapes follow the five benchmark configurations: a small MHA plumbing
 case, the Llama-3-8B GQA batch-32 decode shape, a long-context peaked-softmax case, a 70B-class
-one-GPU share, and a paged_caching scatter of a prefill chunk.
+one-GPU share, and a paged_caching scatter of a prefill chunk; plus prefill shapes (a small plumbing
+case, whole-prompt prefill and chunked prefill over a long history at the Llama-3-8B head layout).
 """
 from __future__ import annotations
 
@@ -47,6 +48,27 @@ class CachingConfig:
     seed: int = 0
 
 
+@dataclass
+class PrefillConfig:
+    name: str
+    dtype: torch.dtype
+    num_seqs: int
+    num_heads: int
+    num_kv_heads: int
+    head_size: int
+    block_size: int
+    min_new: int       # new (query) tokens per sequence
+    max_new: int
+    min_history: int   # tokens already in the cache before them
+    max_history: int
+    spare_block_fraction: float = 0.0
+    seed: int = 0
+
+    @property
+    def scale(self) -> float:
+        return 1.0 / float(self.head_size) ** 0.5
+
+
 DECODE_CONFIGS = {
     "c1_plumbing_mha": DecodeConfig("c1_plumbing_mha", torch.float16, 4, 8, 8, 128, 16, 1, 256, seed=101),
     "c2_llama3_8b_b32": DecodeConfig("c2_llama3_8b_b32", torch.bfloat16, 32, 32, 8, 128, 16, 512, 4096,
@@ -57,6 +79,15 @@ DECODE_CONFIGS = {
 }
 CACHING_CONFIGS = {
     "c5_prefill_scatter": CachingConfig("c5_prefill_scatter", torch.bfloat16, 4096, 8, 128, 16, 65536, 0.05, seed=105),
+}
+
+
+PREFILL_CONFIGS = {
+    "p1_plumbing_mha": PrefillConfig("p1_plumbing_mha", torch.float16, 4, 8, 8, 128, 16, 1, 64, 0, 128, seed=201),
+    "p2_llama3_8b_prompt": PrefillConfig("p2_llama3_8b_prompt", torch.bfloat16, 4, 32, 8, 128, 16, 1024, 4096, 0, 0,
+                                         spare_block_fraction=0.10, seed=202),
+    "p3_llama3_8b_chunked": PrefillConfig("p3_llama3_8b_chunked", torch.bfloat16, 16, 32, 8, 128, 16, 128, 512,
+                                          1024, 8192, spare_block_fraction=0.10, seed=203),
 }
 
 
@@ -118,6 +149,68 @@ def make_decode_inputs(cfg: DecodeConfig, seed_offset: int = 0) -> DecodeInputs:
     k_cache = k_cache.to(cfg.dtype)
     v_cache = _normal(rng, cache_shape, cfg.dtype)
     return DecodeInputs(cfg, q, k_cache, v_cache, torch.from_numpy(table), torch.from_numpy(lens), cfg.scale)
+
+
+@dataclass
+class PrefillInputs:
+    config: PrefillConfig
+    q: torch.Tensor               # [total_q, H, D]
+    k_cache: torch.Tensor         # [NB, Hkv, bs, D]
+    v_cache: torch.Tensor
+    block_tables: torch.Tensor    # [B, max_blocks] int64, unused entries 0
+    seq_lens: torch.Tensor        # [B] int64, history + new
+    cum_seq_lens_q: torch.Tensor  # [B + 1] int64
+    scale: float
+
+
+def draw_prefill_lens(cfg: PrefillConfig):
+    rng = np.random.default_rng(cfg.seed)
+    new = rng.integers(cfg.min_new, cfg.max_new + 1, size=cfg.num_seqs, dtype=np.int64)
+    history = rng.integers(cfg.min_history, cfg.max_history + 1, size=cfg.num_seqs, dtype=np.int64)
+    return new, history
+
+
+def prefill_flops(cfg: PrefillConfig, new, history) -> int:
+    """Multiply-adds x 2 of Q.K^T and P.V over the (query token, visible K/V token) pairs."""
+    new, history = np.asarray(new, dtype=np.int64), np.asarray(history, dtype=np.int64)
+    pairs = int((new * history + new * (new + 1) // 2).sum())
+    return pairs * cfg.num_heads * 4 * cfg.head_size
+
+
+def prefill_algorithmic_bytes(cfg: PrefillConfig, new, history) -> int:
+    """Q in, O out, K and V of every sequence once per KV head, table entries and lengths."""
+    e = 2
+    new, history = np.asarray(new, dtype=np.int64), np.asarray(history, dtype=np.int64)
+    total = new + history
+    qo = 2 * int(new.sum()) * cfg.num_heads * cfg.head_size * e
+    kv = int(total.sum()) * cfg.num_kv_heads * 2 * cfg.head_size * e
+    idx = int(((total + cfg.block_size - 1) // cfg.block_size).sum()) * 8 + (2 * cfg.num_seqs + 1) * 8
+    return qo + kv + idx
+
+
+def make_prefill_inputs(cfg: PrefillConfig) -> PrefillInputs:
+    """Pool of exactly the needed pages (plus the spare fraction), pages dealt to sequences by a seeded
+    random permutation, Q/K/V ~ N(0,1) rounded to the storage dtype; the cache already holds the new
+    tokens' K/V, as it does when the operator runs after paged_caching."""
+    new, history = draw_prefill_lens(cfg)
+    total = new + history
+    rng = np.random.default_rng([cfg.seed, 13])
+    blocks_per_seq = (total + cfg.block_size - 1) // cfg.block_size
+    needed = int(blocks_per_seq.sum())
+    num_blocks = int(np.ceil(needed * (1.0 + cfg.spare_block_fraction)))
+    perm = rng.permutation(num_blocks)[:needed]
+    table = np.zeros((cfg.num_seqs, int(blocks_per_seq.max())), dtype=np.int64)
+    cursor = 0
+    for s, nb in enumerate(blocks_per_seq):
+        table[s, :nb] = perm[cursor:cursor + nb]
+        cursor += nb
+    cum = np.concatenate([[0], np.cumsum(new)]).astype(np.int64)
+    q = _normal(rng, (int(cum[-1]), cfg.num_heads, cfg.head_size), cfg.dtype)
+    cache_shape = (num_blocks, cfg.num_kv_heads, cfg.block_size, cfg.head_size)
+    k_cache = _normal(rng, cache_shape, cfg.dtype)
+    v_cache = _normal(rng, cache_shape, cfg.dtype)
+    return PrefillInputs(cfg, q, k_cache, v_cache, torch.from_numpy(table), torch.from_numpy(total),
+                         torch.from_numpy(cum), cfg.scale)
 
 
 @dataclass

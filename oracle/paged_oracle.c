@@ -1,5 +1,5 @@
 /*
- * CPU oracle for InfiniOP paged_attention (decode) and paged_caching.
+ * CPU oracle for InfiniOP paged_attention (decode), paged_attention_prefill and paged_caching.
  *
  * TEST INFRASTRUCTURE ONLY. This file restates, in plain C, the algorithm of the reference's device
  * kernels so that the HIP kernels of this repository can be checked against it. Only tests/,
@@ -11,7 +11,8 @@
  * tests/test_oracle_pinning.py): an independent fp64 two-pass softmax on gathered K/V, torch's
  * scaled_dot_product_attention on the gathered sequence, closed forms (length 1, equal V rows,
  * zero query, one dominant key), invariance under page permutation, GQA == MHA on repeated heads,
- * split == unsplit, and a byte-exact scatter model for paged_caching.
+ * split == unsplit, prefill row j == decode over the first history + j + 1 tokens, prefill against an
+ * fp64 masked softmax, and a byte-exact scatter model for paged_caching.
  *
  * Functions and the reference code each one follows:
  *   oracle_paged_attention         src/infiniop/ops/paged_attention/cuda/kernel_v2.cuh:134-336
@@ -20,6 +21,8 @@
  *                                  round-to-nearest-even to fp16 / bf16; seq_len <= 0 leaves out untouched)
  *   oracle_paged_attention_splitkv kernel_v2.cuh:340-554 (token shards of ceil(len / splits), partial
  *                                  (m, l, acc) per shard, empty shard = (-inf, 0, 0)) and :556-616 (combine)
+ *   oracle_paged_attention_prefill src/infiniop/ops/paged_attention_prefill/cuda/kernel_v2.cuh:254-472 (row ->
+ *                                  sequence lookup, visible range history + j + 1, then the decode recurrence)
  *   oracle_paged_caching           src/infiniop/ops/paged_caching/cuda/kernel.cuh:22-89
  *                                  (slot < 0 skipped, page = slot / block_size, row = slot % block_size,
  *                                  source heads packed, element-wise copy)
@@ -290,6 +293,75 @@ int oracle_paged_attention_splitkv(void *out_, const void *q_, const void *k_cac
         free(part_acc);
         free(part_m);
         free(part_l);
+    }
+    return 0;
+}
+
+/* Prefill, src/infiniop/ops/paged_attention_prefill/cuda/kernel_v2.cuh:254-472: query row i belongs to the
+ * sequence s with cu_seqlens_q[s] <= i < cu_seqlens_q[s+1] (:20-38; a row no sequence owns is skipped, :297-300);
+ * with q_len = cu[s+1] - cu[s] and history = kv_lens[s] - q_len, local token j = i - cu[s] attends over tokens
+ * [0, history + j + 1) (:302-306, nothing is written when that range is empty) with the decode recurrence;
+ * ALiBi distance is t - (history + j) (:383-386). s->num_seqs is the number of sequences, the row count of q and
+ * out is total_q_tokens. rows (optional) lists the query rows to evaluate, NULL = all of them; only those rows of
+ * out and out_f32 (packed [total_q_tokens, num_heads, value_size], optional) are written. */
+int oracle_paged_attention_prefill(void *out_, float *out_f32, const void *q_, const void *k_cache_,
+                                   const void *v_cache_, const int64_t *block_tables, const int64_t *kv_lens,
+                                   const int64_t *cu_seqlens_q, const float *alibi_slopes,
+                                   const oracle_attention_shape *s, int64_t total_q_tokens, const int64_t *rows,
+                                   int64_t num_rows, int num_threads) {
+    if (s->num_kv_heads <= 0 || s->num_heads % s->num_kv_heads != 0 || s->block_size <= 0) {
+        return -1;
+    }
+    uint16_t *out = (uint16_t *)out_;
+    const uint16_t *q = (const uint16_t *)q_;
+    const int64_t group = s->num_heads / s->num_kv_heads;
+    if (rows == NULL) {
+        num_rows = total_q_tokens;
+    }
+    const int64_t work = num_rows * s->num_heads;
+    if (num_threads < 1) {
+        num_threads = 1;
+    }
+#pragma omp parallel num_threads(num_threads)
+    {
+        float *acc = (float *)malloc(sizeof(float) * (size_t)(s->value_size > 0 ? s->value_size : 1));
+#pragma omp for schedule(dynamic, 1)
+        for (int64_t w = 0; w < work; ++w) {
+            const int64_t row = rows ? rows[w / s->num_heads] : w / s->num_heads;
+            const int64_t head = w % s->num_heads;
+            if (row < 0 || row >= total_q_tokens) {
+                continue;
+            }
+            int64_t seq = -1;
+            for (int64_t i = 0; i < s->num_seqs; ++i) {
+                if (row >= cu_seqlens_q[i] && row < cu_seqlens_q[i + 1]) {
+                    seq = i;
+                    break;
+                }
+            }
+            if (seq < 0) {
+                continue;
+            }
+            const int64_t q_len = cu_seqlens_q[seq + 1] - cu_seqlens_q[seq];
+            const int64_t history = kv_lens[seq] - q_len;
+            const int64_t visible = history + (row - cu_seqlens_q[seq]) + 1;
+            if (visible <= 0) {
+                continue;
+            }
+            float m, l;
+            attend_range(s, q + row * s->q_stride + head * s->q_head_stride, (const uint16_t *)k_cache_,
+                         (const uint16_t *)v_cache_, block_tables + seq * s->block_table_stride, head / group,
+                         alibi_slopes ? alibi_slopes[head] : 0.0f, visible, 0, visible, acc, &m, &l);
+            const float inv_l = 1.0f / (l + 1e-6f);
+            uint16_t *o_row = out + row * s->o_stride + head * s->o_head_stride;
+            for (int64_t d = 0; d < s->value_size; ++d) {
+                o_row[d] = store_elem(acc[d] * inv_l, s->dtype);
+                if (out_f32 != NULL) {
+                    out_f32[(row * s->num_heads + head) * s->value_size + d] = acc[d] * inv_l;
+                }
+            }
+        }
+        free(acc);
     }
     return 0;
 }

@@ -4,7 +4,7 @@ Two independent restatements of the reference live here:
 
 * the C oracle ``liboracle.so`` (device-kernel arithmetic: fp32 online softmax in the log2 domain,
   ``1 / (l + 1e-6)``, round-to-nearest-even), reached through ctypes on torch CPU tensors;
-* ``torch_reference_attention`` / ``torch_reference_caching``: the torch functions the reference's
+* ``torch_reference_attention`` / ``torch_reference_prefill`` / ``torch_reference_caching``: the torch functions the reference's
   own tests compare against (``test/infiniop/paged_attention.py:38-88``: gather the sequence's
   tokens through the block table, repeat KV heads for GQA, logits = scale * einsum in the storage
   dtype, softmax in fp32, probabilities cast back to the storage dtype, einsum with V;
@@ -68,6 +68,10 @@ def load():
         lib.oracle_paged_attention.restype = c_int
         lib.oracle_paged_attention_splitkv.argtypes = common + [c_int, c_int]
         lib.oracle_paged_attention_splitkv.restype = c_int
+        lib.oracle_paged_attention_prefill.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                                       c_void_p, c_void_p, POINTER(AttentionShape), c_int64, c_void_p,
+                                                       c_int64, c_int]
+        lib.oracle_paged_attention_prefill.restype = c_int
         lib.oracle_paged_caching.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, POINTER(CachingShape)]
         lib.oracle_paged_caching.restype = c_int
         lib.oracle_to_float.argtypes = [ctypes.c_uint16, c_int]
@@ -117,6 +121,47 @@ def paged_attention(q, k_cache, v_cache, block_tables, seq_lens, scale, alibi_sl
     else:
         assert not return_fp32
         rc = lib.oracle_paged_attention_splitkv(out.data_ptr(), *args, num_splits, num_threads)
+    if rc != 0:
+        raise ValueError("oracle rejected the arguments")
+    return (out, out_f32) if return_fp32 else out
+
+
+def paged_attention_prefill(q, k_cache, v_cache, block_tables, seq_lens, cum_seq_lens_q, scale, alibi_slopes=None, *,
+                            out=None, rows=None, num_threads: int = 1, return_fp32: bool = False):
+    """C oracle of the prefill operator on torch CPU tensors. ``rows`` (optional 1-D sequence of query
+    row numbers) restricts the evaluation to those rows; all other rows of the result keep the content
+    of ``out`` (zeros when ``out`` is not given; NaN in the fp32 result)."""
+    lib = load()
+    q, k_cache, v_cache = _cpu(q), _cpu(k_cache), _cpu(v_cache)
+    block_tables = _cpu(block_tables).to(torch.int64).contiguous()
+    seq_lens = _cpu(seq_lens).to(torch.int64).contiguous()
+    cum = _cpu(cum_seq_lens_q).to(torch.int64).contiguous()
+    if out is None:
+        out = torch.zeros((*q.shape[:-1], v_cache.shape[-1]), dtype=q.dtype)
+    assert q.stride(-1) == 1 and out.stride(-1) == 1 and k_cache.stride(-1) == 1 and v_cache.stride(-1) == 1
+    assert cum.shape[0] == seq_lens.shape[0] + 1
+    s = AttentionShape(
+        DTYPE_CODE[q.dtype], seq_lens.shape[0], q.shape[1], k_cache.shape[1], q.shape[2], v_cache.shape[3],
+        k_cache.shape[2], block_tables.shape[1], q.stride(0), q.stride(1), out.stride(0), out.stride(1),
+        k_cache.stride(0), k_cache.stride(1), k_cache.stride(2),
+        v_cache.stride(0), v_cache.stride(1), v_cache.stride(2),
+        block_tables.stride(0), float(scale),
+    )
+    alibi_ptr = None
+    if alibi_slopes is not None:
+        alibi_slopes = _cpu(alibi_slopes).to(torch.float32).contiguous()
+        alibi_ptr = alibi_slopes.data_ptr()
+    rows_t, rows_ptr, num_rows = None, None, 0
+    if rows is not None:
+        rows_t = torch.as_tensor(rows, dtype=torch.int64).contiguous()
+        rows_ptr, num_rows = rows_t.data_ptr(), rows_t.numel()
+    out_f32 = None
+    if return_fp32:
+        out_f32 = torch.full((q.shape[0], q.shape[1], v_cache.shape[-1]), float("nan"), dtype=torch.float32)
+    rc = lib.oracle_paged_attention_prefill(
+        out.data_ptr(), out_f32.data_ptr() if return_fp32 else None, q.data_ptr(), k_cache.data_ptr(),
+        v_cache.data_ptr(), block_tables.data_ptr(), seq_lens.data_ptr(), cum.data_ptr(), alibi_ptr, ctypes.byref(s),
+        q.shape[0], rows_ptr, num_rows, num_threads)
     if rc != 0:
         raise ValueError("oracle rejected the arguments")
     return (out, out_f32) if return_fp32 else out
@@ -183,6 +228,35 @@ def torch_reference_attention(q, k_cache, v_cache, block_tables, seq_lens, scale
             rel = (torch.arange(length, device=q.device).int() - length + 1).float()
             bias = alibi_slopes.view(-1, 1, 1) * rel.view(1, 1, -1)
         out[s] = _attend_one(q[s].unsqueeze(0), keys, values, scale, bias).view(num_heads, -1)
+    return out
+
+
+def torch_reference_prefill(q, k_cache, v_cache, block_tables, seq_lens, cum_seq_lens_q, scale):
+    """test/infiniop/paged_attention_prefill.py:88-125: per sequence, gather all of its K/V tokens, logits =
+    einsum in the storage dtype -> fp32 * scale, add a -inf mask above position cache_len + q_idx, softmax in
+    fp32 cast to the storage dtype, einsum with V. KV heads are repeated for grouped-query shapes (the
+    reference test only draws num_heads == num_kv_heads, or one shared KV head)."""
+    block_size = k_cache.shape[2]
+    group = q.shape[1] // k_cache.shape[1]
+    out = torch.zeros((*q.shape[:-1], v_cache.shape[3]), dtype=q.dtype, device=q.device)
+    for i in range(len(cum_seq_lens_q) - 1):
+        q0, q1 = int(cum_seq_lens_q[i]), int(cum_seq_lens_q[i + 1])
+        num_new, total_len = q1 - q0, int(seq_lens[i])
+        cache_len = total_len - num_new
+        if num_new <= 0 or total_len <= 0:
+            continue
+        pos = torch.arange(total_len, device=q.device)
+        pages = block_tables[i].to(torch.int64)[pos // block_size]
+        keys = k_cache[pages, :, pos % block_size, :]
+        values = v_cache[pages, :, pos % block_size, :]
+        if group > 1:
+            keys = torch.repeat_interleave(keys, group, dim=1)
+            values = torch.repeat_interleave(values, group, dim=1)
+        scores = torch.einsum("qhd,khd->hqk", q[q0:q1], keys).float() * scale
+        limit = cache_len + torch.arange(num_new, device=q.device).view(-1, 1)
+        mask = torch.where(pos.view(1, -1) <= limit, 0.0, float("-inf"))
+        probs = torch.softmax(scores + mask.unsqueeze(0), dim=-1).to(q.dtype)
+        out[q0:q1] = torch.einsum("hqk,khd->qhd", probs, values)
     return out
 
 

@@ -69,6 +69,45 @@ def run_paged_attention(handle, q, k_cache, v_cache, block_tables, seq_lens, sca
     return out
 
 
+def create_paged_attention_prefill(handle, out, q, k_cache, v_cache, block_tables, seq_lens, cum_seq_lens_q, alibi,
+                                   scale):
+    """Returns (status, descriptor). Tensor descriptors are destroyed before returning."""
+    descs = [describe(t) for t in (out, q, k_cache, v_cache, block_tables, seq_lens, cum_seq_lens_q)]
+    alibi_desc = describe(alibi) if alibi is not None else L.infiniopTensorDescriptor_t()
+    op = L.infiniopOperatorDescriptor_t()
+    status = L.LIBINFINIOP.infiniopCreatePagedAttentionPrefillDescriptor(handle, ctypes.byref(op), *descs, alibi_desc,
+                                                                         scale)
+    for d in descs:
+        L.destroy_tensor_descriptor(d)
+    if alibi is not None:
+        L.destroy_tensor_descriptor(alibi_desc)
+    return status, op
+
+
+def run_paged_attention_prefill(handle, q, k_cache, v_cache, block_tables, seq_lens, cum_seq_lens_q, scale, alibi=None,
+                                out=None, stream=None):
+    """Full create / query / run / destroy cycle on device tensors (the sequence of calls of
+    test/infiniop/paged_attention_prefill.py:259-310); returns ``out``."""
+    if out is None:
+        out = torch.zeros((*q.shape[:-1], v_cache.shape[-1]), dtype=q.dtype, device=q.device)
+    status, op = create_paged_attention_prefill(handle, out, q, k_cache, v_cache, block_tables, seq_lens,
+                                                cum_seq_lens_q, alibi, scale)
+    L.check_error(status, "infiniopCreatePagedAttentionPrefillDescriptor")
+    size = c_size_t(123)
+    L.check_error(L.LIBINFINIOP.infiniopGetPagedAttentionPrefillWorkspaceSize(op, ctypes.byref(size)))
+    workspace = torch.full((max(size.value, 1),), 1, dtype=torch.uint8, device=q.device)
+    torch.cuda.synchronize()
+    L.check_error(
+        L.LIBINFINIOP.infiniopPagedAttentionPrefill(op, ptr(workspace), size.value, ptr(out), ptr(q), ptr(k_cache),
+                                                    ptr(v_cache), ptr(block_tables), ptr(seq_lens),
+                                                    ptr(cum_seq_lens_q), ptr(alibi), c_void_p(stream or 0)),
+        "infiniopPagedAttentionPrefill",
+    )
+    torch.cuda.synchronize()
+    L.check_error(L.LIBINFINIOP.infiniopDestroyPagedAttentionPrefillDescriptor(op))
+    return out
+
+
 def create_paged_caching(handle, k_cache, v_cache, k, v, slot_mapping):
     descs = [describe(t) for t in (k_cache, v_cache, k, v, slot_mapping)]
     op = L.infiniopOperatorDescriptor_t()

@@ -21,7 +21,9 @@ def test_headers_declare_the_expected_entry_points():
     names = {n for _, n in declared_symbols()}
     for required in (
         "infiniopCreatePagedAttentionDescriptor", "infiniopGetPagedAttentionWorkspaceSize", "infiniopPagedAttention",
-        "infiniopDestroyPagedAttentionDescriptor", "infiniopCreatePagedCachingDescriptor",
+        "infiniopDestroyPagedAttentionDescriptor", "infiniopCreatePagedAttentionPrefillDescriptor",
+        "infiniopGetPagedAttentionPrefillWorkspaceSize", "infiniopPagedAttentionPrefill",
+        "infiniopDestroyPagedAttentionPrefillDescriptor", "infiniopCreatePagedCachingDescriptor",
         "infiniopGetPagedCachingWorkspaceSize", "infiniopPagedCaching", "infiniopDestroyPagedCachingDescriptor",
         "infiniopCreateHandle", "infiniopDestroyHandle", "infiniopCreateTensorDescriptor",
         "infiniopDestroyTensorDescriptor", "infinirtSetDevice", "infinirtMalloc", "infinirtStreamCreate",
