@@ -26,7 +26,7 @@ using op::paged_attention::amd::IndexU32;
 // device memory and are never read on the host).
 struct Plan {
     bool tiled;          // matrix-core kernel (head 128, power-of-two pages >= 8, 16-byte aligned strides)
-    int groups_per_wave; // tiled: R = 1, 2 or 4 column groups per wavefront -> 64 R rows per workgroup
+    int groups_per_wave; // tiled: R = 1 or 2 column groups per wavefront -> 64 R rows per workgroup
     int dims_per_lane;   // element-wise kernel: ceil(max(head_size, value_size) / 64)
 };
 
@@ -43,24 +43,27 @@ Plan makePlan(const PagedAttentionPrefillInfo &in, const device::amd::DeviceInfo
               && multipleOf8(in.o_head_stride) && multipleOf8(in.k_batch_stride) && multipleOf8(in.k_head_stride)
               && multipleOf8(in.k_row_stride) && multipleOf8(in.v_batch_stride) && multipleOf8(in.v_head_stride)
               && multipleOf8(in.v_row_stride) && in.num_blocks > 0 && in.num_blocks <= 0x7fffffff
-              && rows < (1LL << 30) && in.num_kv_heads <= 65535
+              && rows < (1LL << 30) && (rows / 64 + static_cast<long long>(in.num_seqs)) * static_cast<long long>(in.num_kv_heads) < (1LL << 31)
+              // lane offsets inside a tile (15 rows + one row of bytes) are kept in 32 bits
+              && in.k_row_stride > 0 && in.k_row_stride < (1 << 26) && in.v_row_stride > 0 && in.v_row_stride < (1 << 26)
               && static_cast<long long>(in.max_num_blocks_per_seq) * bs < (1LL << 30);
     if (const char *env = std::getenv("INFINIOP_AMD_PREFILL_KERNEL")) {
         if (std::strcmp(env, "generic") == 0) {
             plan.tiled = false;
         }
     }
-    // Rows per workgroup: as many as the average sequence fills, but keep at least two workgroups
-    // per compute unit in flight when the batch is large enough to allow it.
+    // Rows per workgroup: 128 (two column groups per wavefront; both sizes keep two workgroups per
+    // compute unit) unless the average sequence fills no more than 64, or the batch is too small to
+    // give every compute unit two workgroups of 128.
     const long long seqs = in.num_seqs > 0 ? static_cast<long long>(in.num_seqs) : 1;
     const long long rows_per_seq = rows / seqs;
-    int r = 4;
-    while (r > 1 && (rows_per_seq <= 32LL * r || rows / (64LL * r) * static_cast<long long>(in.num_kv_heads) < 2LL * dev.compute_units)) {
-        r /= 2;
+    int r = 2;
+    if (rows_per_seq <= 64 || rows / 128 * static_cast<long long>(in.num_kv_heads) < 2LL * dev.compute_units) {
+        r = 1;
     }
     if (const char *env = std::getenv("INFINIOP_AMD_PREFILL_GROUPS")) {
         const int forced = std::atoi(env);
-        if (forced == 1 || forced == 2 || forced == 4) {
+        if (forced == 1 || forced == 2) {
             r = forced;
         }
     }
@@ -82,16 +85,24 @@ void launchGeneric(const PrefillArgs &a, const Plan &plan, hipStream_t stream) {
     }
 }
 
-template <typename T, typename Tindex>
-void launchTiled(const PrefillArgs &a, const Plan &plan, hipStream_t stream) {
+template <typename T, typename Tindex, bool PLAIN>
+void launchTiledGroups(const PrefillArgs &a, const Plan &plan, hipStream_t stream) {
     // sum over sequences of ceil(rows / block_rows) is at most floor(total rows / block_rows) + num_seqs
     const long long rows = static_cast<long long>(a.total_q_tokens) * a.group;
     const int block_rows = prefillBlockRows(plan.groups_per_wave);
-    const dim3 grid(static_cast<unsigned>(rows / block_rows + a.num_seqs), a.num_kv_heads);
+    const dim3 grid(static_cast<unsigned>((rows / block_rows + a.num_seqs) * a.num_kv_heads));
     switch (plan.groups_per_wave) {
-    case 1: prefillTiledKernel<T, Tindex, 1><<<grid, kPrefillThreads, 0, stream>>>(a); break;
-    case 2: prefillTiledKernel<T, Tindex, 2><<<grid, kPrefillThreads, 0, stream>>>(a); break;
-    default: prefillTiledKernel<T, Tindex, 4><<<grid, kPrefillThreads, 0, stream>>>(a); break;
+    case 1: prefillTiledKernel<T, Tindex, 1, PLAIN><<<grid, kPrefillThreads, 0, stream>>>(a); break;
+    default: prefillTiledKernel<T, Tindex, 2, PLAIN><<<grid, kPrefillThreads, 0, stream>>>(a); break;
+    }
+}
+
+template <typename T, typename Tindex>
+void launchTiled(const PrefillArgs &a, const Plan &plan, hipStream_t stream) {
+    if (a.alibi_slopes == nullptr && a.scale_log2 > 0.0f) {
+        launchTiledGroups<T, Tindex, true>(a, plan, stream);
+    } else {
+        launchTiledGroups<T, Tindex, false>(a, plan, stream);
     }
 }
 

@@ -4,7 +4,7 @@
 // token, query head of the KV head's group) pair, token-major: row = token * group + head_in_group.
 // Packing the heads of a group into the row dimension means a K/V tile fetched once serves all of
 // them, and short prompts still fill the matrix instructions. Each of the four wavefronts owns 16*R
-// consecutive rows (R column groups of 16).
+// consecutive rows (R = 1 or 2 column groups of 16).
 //
 // The K/V tokens the rows may see are consumed in steps of 64. Per step the workgroup copies
 // 64 K rows and 64 V rows (16 KiB each) from the paged pool into LDS, every wavefront 16 tokens of
@@ -24,8 +24,8 @@
 //   O[row][dim] += P . V      16 x v_mfma_f32_16x16x32 (A = P rounded to the storage dtype, straight
 //                             from the registers S came out in; B = V words from LDS; lane holds
 //                             O[row 4g + 0..3][8c + e], e = 0..7)
-// K/V fragments read from LDS are shared by the R column groups of a wavefront. The denominator sums
-// the rounded probabilities. A step whose tokens lie beyond everything a wavefront's rows may see
+//   l[row]      += P . 1       2 x v_mfma_f32_16x16x32: the denominator sums the rounded probabilities
+// K/V fragments read from LDS are shared by the R column groups of a wavefront. A step whose tokens lie beyond everything a wavefront's rows may see
 // is skipped by that wavefront (it still takes part in the copy).
 //
 // The math follows the reference's prefill kernels (src/infiniop/ops/paged_attention_prefill/cuda/
@@ -44,9 +44,19 @@ using op::paged_attention::amd::sumAcrossTokenGroups;
 using op::paged_attention::amd::TileBF16;
 using op::paged_attention::amd::TileF16;
 
+using op::paged_attention::amd::kTileTokens;
+
 constexpr int kPrefillThreads = 256;
 constexpr int kPrefillStepTokens = 64;
 constexpr int kPrefillHead = 128;
+
+// 16-byte load from (wave-uniform base) + (32-bit per-lane byte offset), through the caches: K/V tiles
+// are read again by the other row blocks of the sequence. The empty asm keeps the offset a value
+// defined where it is used, so that the scalar-base form of the load is selected.
+__device__ __forceinline__ uint4 loadLane16Cached(const char *uniform_base, uint32_t lane_offset) {
+    asm volatile("" : "+v"(lane_offset));
+    return *reinterpret_cast<const uint4 *>(uniform_base + lane_offset);
+}
 
 // Rows of one workgroup for R column groups per wavefront.
 __host__ __device__ constexpr int prefillBlockRows(int r) { return 64 * r; }
@@ -88,8 +98,10 @@ __device__ __forceinline__ bool findRowBlock(const PrefillArgs &a, int lane, int
     return false;
 }
 
-template <typename T, typename Tindex, int R>
-__global__ void __launch_bounds__(kPrefillThreads) prefillTiledKernel(PrefillArgs a) {
+// PLAIN: no ALiBi and scale > 0. The running maximum is then kept in units of the raw dot product
+// (a positive scale keeps the order) and each probability costs one fused multiply-add and one exp2.
+template <typename T, typename Tindex, int R, bool PLAIN>
+__global__ void __launch_bounds__(kPrefillThreads, 2) prefillTiledKernel(PrefillArgs a) {
     using S = typename T::storage;
     constexpr int BM = prefillBlockRows(R);
     __shared__ uint4 k_lds[2][kPrefillStepTokens * 16];    // [token][16-byte chunk ^ (token & 15)]
@@ -99,10 +111,14 @@ __global__ void __launch_bounds__(kPrefillThreads) prefillTiledKernel(PrefillArg
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int c = lane & 15;
     const int g = lane >> 4;
-    const int kv_head = blockIdx.y;
+    // KV head fastest: workgroup ids go round-robin over the 8 accelerator dies, so with 8 (or a
+    // multiple of 8) KV heads every die works on its own heads and the row blocks resident on a die
+    // at one time are neighbours that stream the same K/V through that die's L2.
+    const int kv_head = blockIdx.x % a.num_kv_heads;
+    const int block_index = blockIdx.x / a.num_kv_heads;
 
     int seq = 0, block = 0;
-    if (!findRowBlock<Tindex>(a, lane, BM, blockIdx.x, seq, block)) {
+    if (!findRowBlock<Tindex>(a, lane, BM, block_index, seq, block)) {
         return;
     }
     const SeqSpan span = loadSeqSpan<Tindex>(a, seq);
@@ -157,22 +173,60 @@ __global__ void __launch_bounds__(kPrefillThreads) prefillTiledKernel(PrefillArg
     const bool small_pages = a.block_size < 16; // pages of 8 tokens: a 16-token tile spans two
     const int last_entry = (kv_len - 1) >> a.block_shift;
 
-    // page ids of the 16-token tile that starts at token t (wave-uniform)
-    auto loadPageIds = [&](int t, int &id0, int &id1) {
-        id0 = 0;
-        id1 = 0;
-        if (t < kv_len) {
-            const int e0 = t >> a.block_shift;
-            id0 = clampPage(loadIndex<Tindex>(a.block_tables, table_row + e0), a.num_blocks);
-            id1 = id0;
-            if (small_pages && e0 + 1 <= last_entry) {
-                id1 = clampPage(loadIndex<Tindex>(a.block_tables, table_row + e0 + 1), a.num_blocks);
-            }
+    // Page ids: 64 block-table entries at a time, one per lane, fetched a whole batch ahead of their
+    // use with an ordinary vector load. No load in the loop waits for another load, and nothing in the
+    // loop goes through the scalar cache, whose out-of-order returns would make every LDS wait a wait
+    // for it too.
+    auto loadIdBatch = [&](int batch) {
+        const int entry = batch * 64 + lane;
+        int id = 0;
+        if (entry <= last_entry) {
+            id = static_cast<int>(loadIndex<Tindex>(a.block_tables, table_row + entry)); // low 32 bits; clamped where used
         }
+        return id;
     };
+    int id_batch = 0;
+    int ids_cur = loadIdBatch(0), ids_next = loadIdBatch(1);
+    auto pageOfEntry = [&](int entry) {
+        const int e = min(entry, last_entry);
+        const int raw = (e >> 6) == id_batch ? __builtin_amdgcn_readlane(ids_cur, e & 63)
+                                             : __builtin_amdgcn_readlane(ids_next, e & 63);
+        return clampPage(raw, a.num_blocks);
+    };
+
+    uint32_t k_off[4], v_off[4]; // byte offsets of this lane's rows inside a 16-token tile (pages >= 16 tokens)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        k_off[j] = static_cast<uint32_t>((4 * j + g) * a.k_row_stride * static_cast<int64_t>(sizeof(S))) + 16 * c;
+        v_off[j] = static_cast<uint32_t>((4 * g + j) * a.v_row_stride * static_cast<int64_t>(sizeof(S))) + 16 * c;
+    }
     uint4 k_stage[4], v_stage[4];
-    auto loadStage = [&](int t, int id0, int id1) {
+    auto loadStage = [&](int t) {
         // K: rows 4 jj + g of the tile; V: rows 4 g + i. Tokens past kv_len are not fetched.
+        const int e0 = t >> a.block_shift;
+        if ((min(e0, last_entry) >> 6) > id_batch) {
+            ids_cur = ids_next;
+            ++id_batch;
+            ids_next = loadIdBatch(id_batch + 1);
+        }
+        if (t + kTileTokens <= kv_len && !small_pages) {
+            const int page = pageOfEntry(e0);
+            const int row0 = t & block_mask;
+            const char *k_tile = k_head + (page * a.k_batch_stride + row0 * a.k_row_stride) * static_cast<int64_t>(sizeof(S));
+            const char *v_tile = v_head + (page * a.v_batch_stride + row0 * a.v_row_stride) * static_cast<int64_t>(sizeof(S));
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                k_stage[j] = loadLane16Cached(k_tile, k_off[j]);
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                v_stage[j] = loadLane16Cached(v_tile, v_off[j]);
+            }
+            return;
+        }
+        // last tile of the sequence, or two pages per tile
+        const int id0 = t < kv_len ? pageOfEntry(e0) : 0;
+        const int id1 = (small_pages && t < kv_len) ? pageOfEntry(e0 + 1) : id0;
         const int row0 = small_pages ? 0 : (t & block_mask);
 #pragma unroll
         for (int jj = 0; jj < 4; ++jj) {
@@ -212,20 +266,29 @@ __global__ void __launch_bounds__(kPrefillThreads) prefillTiledKernel(PrefillArg
         }
     };
 
-    // ---- softmax state: o[r][e][rr] = O[row 4g+rr of group r][column 8c+e] ----
-    f32x4 o[R][8];
-    float m[R], l[R];
+    // ---- softmax state ----
+    // o[r][e][rr] = O[row 4g+rr of group r][column 8c+e]; ol[r][rr] = sum of that row's probabilities
+    // (computed by the matrix unit as P . 1, so it sums exactly the rounded probabilities the numerator
+    // used and already sits in the accumulators' row layout); m[r] = running maximum of row c, in units
+    // of the raw dot product when there is no ALiBi (scale > 0 keeps the order), else of the scaled score.
+    f32x4 o[R][8], ol[R];
+    float m[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
             o[r][e] = f32x4{0.f, 0.f, 0.f, 0.f};
         }
+        ol[r] = f32x4{0.f, 0.f, 0.f, 0.f};
         m[r] = -INFINITY;
-        l[r] = 0.0f;
     }
+    const uint32_t one2 = T::pack2(1.0f, 1.0f);
+    const uint4 ones = make_uint4(one2, one2, one2, one2);
+    const float unit = PLAIN ? a.scale_log2 : 1.0f; // log2-domain size of one unit of m
 
-    auto computeStep = [&](int buf, int t0) {
+    // One step over the 64 tokens in LDS buffer `buf`. masked: some score of the step lies beyond
+    // what its row may see (steps on the causal diagonal); the other steps skip the comparison.
+    auto computeStep = [&](int buf, int t0, bool masked) {
         f32x4 s[R][4];
 #pragma unroll
         for (int r = 0; r < R; ++r) {
@@ -236,76 +299,87 @@ __global__ void __launch_bounds__(kPrefillThreads) prefillTiledKernel(PrefillArg
         }
 #pragma unroll
         for (int tt = 0; tt < 4; ++tt) {
+            uint4 kf[4];
 #pragma unroll
             for (int kk = 0; kk < 4; ++kk) {
-                const uint4 kf = k_lds[buf][(16 * tt + c) * 16 + ((4 * kk + g) ^ c)];
+                kf[kk] = k_lds[buf][(16 * tt + c) * 16 + ((4 * kk + g) ^ c)];
+            }
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk) {
 #pragma unroll
                 for (int r = 0; r < R; ++r) {
-                    s[r][tt] = T::mfmaK32(kf, q_reg[r][kk], s[r][tt]);
+                    s[r][tt] = T::mfmaK32(kf[kk], q_reg[r][kk], s[r][tt]);
                 }
             }
         }
 
-        const bool on_diagonal = t0 + kPrefillStepTokens > wave_min_visible; // some score of this step is masked
-        const bool has_alibi = a.alibi_slopes != nullptr;
         uint4 p_op[R][2];
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            float sc[4][4];
-            float mx = -INFINITY;
+            // scores in the units m[r] is kept in
+            if constexpr (!PLAIN) {
 #pragma unroll
-            for (int tt = 0; tt < 4; ++tt) {
+                for (int tt = 0; tt < 4; ++tt) {
 #pragma unroll
-                for (int rr = 0; rr < 4; ++rr) {
-                    const int tok = t0 + 16 * tt + 4 * g + rr;
-                    float x = s[r][tt][rr] * a.scale_log2;
-                    if (has_alibi) {
-                        x += slope[r] * static_cast<float>(tok - (visible[r] - 1));
+                    for (int rr = 0; rr < 4; ++rr) {
+                        const int tok = t0 + 16 * tt + 4 * g + rr;
+                        s[r][tt][rr] = s[r][tt][rr] * a.scale_log2 + slope[r] * static_cast<float>(tok - (visible[r] - 1));
                     }
-                    x = (on_diagonal && tok >= visible[r]) ? -INFINITY : x;
-                    sc[tt][rr] = x;
-                    mx = fmaxf(mx, x);
                 }
+            }
+            if (masked) {
+#pragma unroll
+                for (int tt = 0; tt < 4; ++tt) {
+#pragma unroll
+                    for (int rr = 0; rr < 4; ++rr) {
+                        const int tok = t0 + 16 * tt + 4 * g + rr;
+                        s[r][tt][rr] = tok >= visible[r] ? -INFINITY : s[r][tt][rr];
+                    }
+                }
+            }
+            float mx = fmaxf(fmaxf(s[r][0][0], s[r][0][1]), fmaxf(s[r][0][2], s[r][0][3]));
+#pragma unroll
+            for (int tt = 1; tt < 4; ++tt) {
+                mx = fmaxf(mx, fmaxf(fmaxf(s[r][tt][0], s[r][tt][1]), fmaxf(s[r][tt][2], s[r][tt][3])));
             }
             mx = maxAcrossTokenGroups(mx);
             const float m_new = fmaxf(m[r], mx);
             if (__builtin_amdgcn_ballot_w64(m_new > m[r]) != 0) {
                 // some row's maximum moved: rescale. Lane holds accumulators of rows 4g..4g+3, whose
                 // factors live in lanes 4g..4g+3.
-                const float alpha = m_new > m[r] ? fastExp2(m[r] - m_new) : 1.0f;
-                l[r] *= alpha;
+                const float alpha = m_new > m[r] ? fastExp2((m[r] - m_new) * unit) : 1.0f;
                 m[r] = m_new;
 #pragma unroll
                 for (int rr = 0; rr < 4; ++rr) {
                     const float alpha_r = __shfl(alpha, 4 * g + rr, 64);
+                    ol[r][rr] *= alpha_r;
 #pragma unroll
                     for (int e = 0; e < 8; ++e) {
                         o[r][e][rr] *= alpha_r;
                     }
                 }
             }
-            const float m_use = m[r] == -INFINITY ? 0.0f : m[r]; // a row that has seen nothing yet: p = 2^-inf = 0
-            float p_sum = 0.0f;
+            // a row that has seen nothing yet keeps m = -inf: subtract 0, p = 2^-inf = 0
+            const float shift = m[r] == -INFINITY ? 0.0f : -m[r] * unit;
 #pragma unroll
             for (int u = 0; u < 2; ++u) {
                 uint32_t wds[4];
 #pragma unroll
                 for (int h = 0; h < 2; ++h) {
-                    const int tt = 2 * u + h;
-                    wds[2 * h] = T::pack2(fastExp2(sc[tt][0] - m_use), fastExp2(sc[tt][1] - m_use));
-                    wds[2 * h + 1] = T::pack2(fastExp2(sc[tt][2] - m_use), fastExp2(sc[tt][3] - m_use));
-                }
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    p_sum += T::unpackLo(wds[i]) + T::unpackHi(wds[i]);
+                    const f32x4 x = s[r][2 * u + h];
+                    wds[2 * h] = T::pack2(fastExp2(__builtin_fmaf(x[0], unit, shift)), fastExp2(__builtin_fmaf(x[1], unit, shift)));
+                    wds[2 * h + 1] = T::pack2(fastExp2(__builtin_fmaf(x[2], unit, shift)), fastExp2(__builtin_fmaf(x[3], unit, shift)));
                 }
                 p_op[r][u] = make_uint4(wds[0], wds[1], wds[2], wds[3]);
             }
-            l[r] += p_sum;
         }
 
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                ol[r] = T::mfmaK32(p_op[r][u], ones, ol[r]);
+            }
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 const uint2 lo = v_lds[buf][((e * 4 + 2 * u) * 4 + g) * 16 + c];
@@ -320,39 +394,32 @@ __global__ void __launch_bounds__(kPrefillThreads) prefillTiledKernel(PrefillArg
     };
 
     // ---- pipeline ----
-    int id0, id1, next_id0, next_id1;
-    loadPageIds(16 * w, id0, id1);
-    loadStage(16 * w, id0, id1);
-    loadPageIds(kPrefillStepTokens + 16 * w, id0, id1);
+    loadStage(16 * w);
     storeStage(0);
     __syncthreads();
     if (n_steps > 1) {
-        loadStage(kPrefillStepTokens + 16 * w, id0, id1);
+        loadStage(kPrefillStepTokens + 16 * w);
     }
-    loadPageIds(2 * kPrefillStepTokens + 16 * w, next_id0, next_id1);
     for (int j = 0; j < n_steps; ++j) {
         const int t0 = j * kPrefillStepTokens;
         if (t0 < wave_max_visible) {
-            computeStep(j & 1, t0);
+            computeStep(j & 1, t0, t0 + kPrefillStepTokens > wave_min_visible);
         }
         if (j + 1 < n_steps) {
             storeStage((j + 1) & 1);
         }
         __syncthreads();
         if (j + 2 < n_steps) {
-            loadStage((j + 2) * kPrefillStepTokens + 16 * w, next_id0, next_id1);
-            loadPageIds((j + 3) * kPrefillStepTokens + 16 * w, next_id0, next_id1);
+            loadStage((j + 2) * kPrefillStepTokens + 16 * w);
         }
     }
 
     // ---- normalise and store: lane writes columns 8c..8c+7 of rows 4g..4g+3 of each group ----
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-        const float l_tot = sumAcrossTokenGroups(l[r]);
 #pragma unroll
         for (int rr = 0; rr < 4; ++rr) {
             const int src_lane = 4 * g + rr;
-            const float l_row = __shfl(l_tot, src_lane, 64);
             const int visible_row = __shfl(visible[r], src_lane, 64);
             const int row = block_row0 + (w * R + r) * 16 + src_lane;
             if (row >= total_rows || visible_row <= 0) {
@@ -360,7 +427,7 @@ __global__ void __launch_bounds__(kPrefillThreads) prefillTiledKernel(PrefillArg
             }
             const int token = row / a.group;
             const int head = kv_head * a.group + (row - token * a.group);
-            const float inv_l = 1.0f / (l_row + 1e-6f);
+            const float inv_l = 1.0f / (ol[r][rr] + 1e-6f);
             uint4 packed;
             packed.x = T::pack2(o[r][0][rr] * inv_l, o[r][1][rr] * inv_l);
             packed.y = T::pack2(o[r][2][rr] * inv_l, o[r][3][rr] * inv_l);
