@@ -1,5 +1,5 @@
 #!/usr/bin/env python3
-"""Paged-attention decode benchmark on one MI355X.
+"""Paged-attention benchmark on one MI355X: decode (default, the headline) or prefill.
 
 A step is one ``infiniopPagedAttention`` call (decode kernel + partition merge) through the C ABI on
 the Llama-3-8B GQA batch-32 decode shape (bf16, 32 query / 8 KV heads, head 128, pages of 16
@@ -7,6 +7,10 @@ tokens, ragged lengths 512..4096 through a shuffled block table). Inputs are res
 the timed region. Consecutive steps read different KV pools (same content, different addresses,
 together far larger than the 256 MiB last-level cache), so every step streams its K/V from HBM as a
 real model does when it moves from layer to layer.
+
+With ``--workload p2_llama3_8b_prompt`` or ``p3_llama3_8b_chunked`` a step is one
+``infiniopPagedAttentionPrefill`` call instead, bounded by the bf16 matrix-core peak; the line then
+reports TFLOP/s (2 x multiply-adds of Q.K^T and P.V over the visible query/key pairs).
 
 Prints one JSON line: throughput in algorithmic GB/s (K and V once per KV head + Q + O + the
 needed table entries + lengths), the time per call, the HBM roofline of the step measured with
@@ -28,6 +32,7 @@ ROOT = Path(__file__).resolve().parent
 sys.path.insert(0, str(ROOT))
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E
+MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 / fp16 matrix peak
 
 # HBM bytes per launch of the decode kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
 # file, each scaled by what the same counter reads for a 256 MiB copy (summary and commands:
@@ -39,8 +44,8 @@ MEASURED_TRAFFIC_BYTES = {"c2_llama3_8b_b32": 322_300_000}
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=400)
-    ap.add_argument("--warmup", type=int, default=40)
+    ap.add_argument("--steps", type=int, default=None, help="default 400 (decode) / 50 (prefill)")
+    ap.add_argument("--warmup", type=int, default=None, help="default 40 (decode) / 5 (prefill)")
     ap.add_argument("--workload", default="c2_llama3_8b_b32")
     ap.add_argument("--pools", type=int, default=4, help="distinct KV pools the steps rotate over")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -49,6 +54,154 @@ def parse_args():
                     help="also run three plain 256 MiB device copies, so that a rocprofv3 --pmc run of this "
                          "command records FETCH_SIZE / WRITE_SIZE of a kernel whose traffic is known")
     return ap.parse_args()
+
+
+def run_prefill(args, torch, L, workloads, dev):
+    """One step = one infiniopPagedAttentionPrefill call; inputs resident in HBM."""
+    import numpy as np
+
+    cfg = workloads.PREFILL_CONFIGS[args.workload]
+    inp = workloads.make_prefill_inputs(cfg)
+    new, history = workloads.draw_prefill_lens(cfg)
+    flops = workloads.prefill_flops(cfg, new, history)
+    algo_bytes = workloads.prefill_algorithmic_bytes(cfg, new, history)
+
+    L.set_device(L.InfiniDevice.AMD, 0)
+    handle = L.create_handle()
+    tensors = [t.to(dev) for t in (inp.q, inp.k_cache, inp.v_cache, inp.block_tables, inp.seq_lens, inp.cum_seq_lens_q)]
+    q, k_cache, v_cache, bt, sl, cu = tensors
+    out = torch.zeros_like(q)
+    DTYPES = {torch.float16: L.InfiniDtype.F16, torch.bfloat16: L.InfiniDtype.BF16, torch.int64: L.InfiniDtype.I64}
+    descs = [L.create_tensor_descriptor(tuple(t.shape), tuple(t.stride()), DTYPES[t.dtype]) for t in (out, *tensors)]
+    op = L.infiniopOperatorDescriptor_t()
+    L.check_error(L.LIBINFINIOP.infiniopCreatePagedAttentionPrefillDescriptor(
+        handle, ctypes.byref(op), *descs, L.infiniopTensorDescriptor_t(), inp.scale))
+    for d in descs:
+        L.destroy_tensor_descriptor(d)
+    ws_size = c_size_t(0)
+    L.check_error(L.LIBINFINIOP.infiniopGetPagedAttentionPrefillWorkspaceSize(op, ctypes.byref(ws_size)))
+    workspace = torch.empty(max(ws_size.value, 1), dtype=torch.uint8, device=dev)
+
+    stream = c_void_p()
+    L.check_error(L.LIBINFINIRT.infinirtStreamCreate(ctypes.byref(stream)))
+    ev0, ev1 = c_void_p(), c_void_p()
+    L.check_error(L.LIBINFINIRT.infinirtEventCreate(ctypes.byref(ev0)))
+    L.check_error(L.LIBINFINIRT.infinirtEventCreate(ctypes.byref(ev1)))
+
+    def step():
+        L.check_error(L.LIBINFINIOP.infiniopPagedAttentionPrefill(
+            op, c_void_p(workspace.data_ptr()), ws_size.value, c_void_p(out.data_ptr()), c_void_p(q.data_ptr()),
+            c_void_p(k_cache.data_ptr()), c_void_p(v_cache.data_ptr()), c_void_p(bt.data_ptr()), c_void_p(sl.data_ptr()),
+            c_void_p(cu.data_ptr()), c_void_p(0), stream))
+
+    torch.cuda.synchronize()
+    for _ in range(args.warmup):
+        step()
+    L.check_error(L.LIBINFINIRT.infinirtStreamSynchronize(stream))
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    L.check_error(L.LIBINFINIRT.infinirtEventRecord(ev0, stream))
+    for _ in range(args.steps):
+        step()
+    L.check_error(L.LIBINFINIRT.infinirtEventRecord(ev1, stream))
+    L.check_error(L.LIBINFINIRT.infinirtStreamSynchronize(stream))
+    torch.cuda.synchronize()
+    wall_s = time.perf_counter() - t0
+    ms = c_float(0)
+    L.check_error(L.LIBINFINIRT.infinirtEventElapsedTime(ctypes.byref(ms), ev0, ev1))
+    us_wall = wall_s / args.steps * 1e6
+    us_dev = ms.value / args.steps * 1e3
+    tflops_wall = flops / (us_wall * 1e-6) / 1e12
+    tflops_dev = flops / (us_dev * 1e-6) / 1e12
+
+    result = {
+        "metric": "PagedAttn prefill achieved TFLOP/s (4 * head_size * heads * visible query-key pairs / time per call), "
+                  "8B-GQA, 1 GPU",
+        "value": round(tflops_wall, 1),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(us_wall / 1e3, 6),
+        "us_per_call": round(us_wall, 2),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16" if cfg.dtype == torch.bfloat16 else "f16",
+        "data": "synthetic",
+        "config": {
+            "workload": cfg.name,
+            "num_seqs": cfg.num_seqs, "num_heads": cfg.num_heads, "num_kv_heads": cfg.num_kv_heads,
+            "head_size": cfg.head_size, "block_size": cfg.block_size,
+            "new_tokens": f"uniform[{cfg.min_new},{cfg.max_new}] sum={int(new.sum())}",
+            "history_tokens": f"uniform[{cfg.min_history},{cfg.max_history}] sum={int(history.sum())}",
+            "flops_per_call": flops,
+            "algorithmic_bytes_per_call": algo_bytes,
+        },
+        "roofline": {
+            "bound": "mfma",
+            "achieved": round(tflops_dev, 1),
+            "peak": MFMA_PEAK_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": round(tflops_dev / MFMA_PEAK_TFLOPS, 4),
+            "traffic": None,
+            "us_per_call_device": round(us_dev, 2),
+            "note": "achieved = flops per call / device time per call (events on the kernel's stream); one kernel per call",
+        },
+    }
+
+    from oracle import paged_oracle
+
+    threads = min(16, os.cpu_count() or 1)
+    # a bounded sample of query rows: first, middle and last row of every sequence plus random ones
+    rng = np.random.default_rng(1)
+    cum = inp.cum_seq_lens_q.tolist()
+    rows = []
+    for s in range(cfg.num_seqs):
+        n = cum[s + 1] - cum[s]
+        if n > 0:
+            rows += [cum[s] + j for j in sorted({0, n // 2, n - 1} | set(rng.integers(0, n, 5).tolist()))]
+    if not args.no_check:
+        step()
+        L.check_error(L.LIBINFINIRT.infinirtStreamSynchronize(stream))
+        sel = torch.as_tensor(rows)
+        _, want32 = paged_oracle.paged_attention_prefill(inp.q, inp.k_cache, inp.v_cache, inp.block_tables, inp.seq_lens,
+                                                         inp.cum_seq_lens_q, inp.scale, rows=rows, num_threads=threads,
+                                                         return_fp32=True)
+        err = (out.float().cpu()[sel] - want32[sel]).abs()
+        ok = bool((err <= 1e-2 + 2e-3 * want32[sel].abs()).all())
+        result["parity"] = {"rows_checked": len(rows), "max_abs_err": float(err.max()), "within_atol1e-2_rtol2e-3": ok}
+        if not ok:
+            print(json.dumps(result))
+            print("bench.py: output does not match the oracle", file=sys.stderr)
+            sys.exit(4)
+    if not args.no_cpu_baseline:
+        # the C oracle on the sampled rows, scaled by the flops those rows stand for
+        sample_pairs = 0
+        for r in rows:
+            s = int(np.searchsorted(np.asarray(cum), r, side="right") - 1)
+            sample_pairs += int(history[s]) + (r - cum[s]) + 1
+        sample_flops = sample_pairs * cfg.num_heads * 4 * cfg.head_size
+        reps, t0 = 0, time.perf_counter()
+        while reps < 50 and time.perf_counter() - t0 < 12.0:
+            paged_oracle.paged_attention_prefill(inp.q, inp.k_cache, inp.v_cache, inp.block_tables, inp.seq_lens,
+                                                 inp.cum_seq_lens_q, inp.scale, rows=rows, num_threads=threads)
+            reps += 1
+        cpu_s = (time.perf_counter() - t0) / reps
+        result["cpu_baseline"] = {
+            "value": round(sample_flops / cpu_s / 1e12, 5),
+            "unit": "TFLOP/s",
+            "cores": threads,
+            "kind": "port",
+            "sample": f"{reps} passes of the C oracle over {len(rows)} of the {cum[-1]} query rows "
+                      f"({sample_flops / flops * 100:.2f} % of the call's flops), {cpu_s * 1e3:.1f} ms per pass",
+        }
+    print(json.dumps(result))
+    L.check_error(L.LIBINFINIOP.infiniopDestroyPagedAttentionPrefillDescriptor(op))
+    L.check_error(L.LIBINFINIRT.infinirtEventDestroy(ev0))
+    L.check_error(L.LIBINFINIRT.infinirtEventDestroy(ev1))
+    L.check_error(L.LIBINFINIRT.infinirtStreamDestroy(stream))
+    L.destroy_handle(handle)
 
 
 def main():
@@ -66,6 +219,12 @@ def main():
         print("bench.py: no GPU visible; the HIP path has no CPU fallback", file=sys.stderr)
         sys.exit(3)
     dev = torch.device("cuda:0")
+    if args.workload in workloads.PREFILL_CONFIGS:
+        args.steps = 50 if args.steps is None else args.steps
+        args.warmup = 5 if args.warmup is None else args.warmup
+        return run_prefill(args, torch, L, workloads, dev)
+    args.steps = 400 if args.steps is None else args.steps
+    args.warmup = 40 if args.warmup is None else args.warmup
     cfg = workloads.DECODE_CONFIGS[args.workload]
     inp = workloads.make_decode_inputs(cfg)
     algo_bytes = workloads.decode_algorithmic_bytes(cfg, inp.seq_lens.numpy())
