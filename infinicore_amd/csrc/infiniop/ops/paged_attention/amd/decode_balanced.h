@@ -94,11 +94,12 @@ struct TileRun {
     bool valid;      // false past the end of the wavefront's piece
 };
 
-template <typename T, typename Tindex>
+template <typename T, typename Tindex, int HEAD>
 __global__ void __launch_bounds__(64) decodeBalancedKernel(DecodeArgs a, int waves_per_stream) {
     using S = typename T::storage;
-    constexpr int NBUF = INFINIOP_AMD_PA_BALANCED_BUFFERS;
-    __shared__ uint4 k_lds[kTileTokens * kTiledHead / 8];
+    using G = TileGeometry<HEAD>;
+    constexpr int NBUF = G::kBuffers;
+    __shared__ uint4 k_lds[kTileTokens * G::kChunksPerRow];
     __shared__ int pre_incl[kBalancedMaxSeqs];
 
     const int piece = blockIdx.x;
@@ -142,14 +143,8 @@ __global__ void __launch_bounds__(64) decodeBalancedKernel(DecodeArgs a, int wav
     const char *v_head = reinterpret_cast<const char *>(static_cast<const S *>(a.v_cache) + kv_head * a.v_head_stride);
     const int block_mask = a.block_size - 1;
     const int tiles_per_entry_shift = a.block_shift - 4; // log2(block_size / 16)
-    const uint32_t k_row_bytes = static_cast<uint32_t>(a.k_row_stride) * sizeof(S);
-    const uint32_t v_row_bytes = static_cast<uint32_t>(a.v_row_stride) * sizeof(S);
-    uint32_t k_off[4], v_off[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        k_off[j] = (4 * j + g) * k_row_bytes + 16 * c;
-        v_off[j] = (4 * g + j) * v_row_bytes + 16 * c;
-    }
+    const LaneOffsets<HEAD> off(lane, static_cast<uint32_t>(a.k_row_stride) * sizeof(S),
+                                static_cast<uint32_t>(a.v_row_stride) * sizeof(S));
 
     // ---- wave-uniform walk over the piece: sequences -> segments -> runs ----
     auto seqFirstTile = [&](int s) { return s == 0 ? 0 : uniformRead(&pre_incl[s - 1]); };
@@ -204,7 +199,7 @@ __global__ void __launch_bounds__(64) decodeBalancedKernel(DecodeArgs a, int wav
     int ld_next_ids = loadPageIds(ld_next);
     int ld_t = ld_run.t0;
 
-    auto loadNextTile = [&]() -> TileRegs {
+    auto loadNextTile = [&]() -> TileRegs<HEAD> {
         const bool real = ld_run.valid;
         const uint32_t lane_mask = real ? 0xffffffffu : 0u;
         const int entry = real ? (ld_t >> tiles_per_entry_shift) - ld_run.first_entry : 0;
@@ -212,15 +207,7 @@ __global__ void __launch_bounds__(64) decodeBalancedKernel(DecodeArgs a, int wav
         const int row0 = real ? (ld_t * kTileTokens) & block_mask : 0;
         const char *k_tile = k_head + (page * a.k_batch_stride + row0 * a.k_row_stride) * static_cast<int64_t>(sizeof(S));
         const char *v_tile = v_head + (page * a.v_batch_stride + row0 * a.v_row_stride) * static_cast<int64_t>(sizeof(S));
-        TileRegs r;
-        r.k0 = loadLane16(k_tile, k_off[0] & lane_mask);
-        r.k1 = loadLane16(k_tile, k_off[1] & lane_mask);
-        r.k2 = loadLane16(k_tile, k_off[2] & lane_mask);
-        r.k3 = loadLane16(k_tile, k_off[3] & lane_mask);
-        r.v0 = loadLane16(v_tile, v_off[0] & lane_mask);
-        r.v1 = loadLane16(v_tile, v_off[1] & lane_mask);
-        r.v2 = loadLane16(v_tile, v_off[2] & lane_mask);
-        r.v3 = loadLane16(v_tile, v_off[3] & lane_mask);
+        const TileRegs<HEAD> r = loadTileRegs<HEAD>(k_tile, v_tile, off, lane_mask);
         if (real && ++ld_t == ld_run.t1) {
             // next run: its page ids were requested one run ago
             ld_run = ld_next;
@@ -233,8 +220,8 @@ __global__ void __launch_bounds__(64) decodeBalancedKernel(DecodeArgs a, int wav
     };
 
     // ---- compute side ----
-    TileState st;
-    uint4 q_reg[4];
+    TileState<HEAD> st;
+    uint4 q_reg[G::kLoads];
     int c_seq = seq0, c_t = 0, c_t_begin = 0, c_seg_end = 0, c_seq_tiles = 0, c_len = 0;
 
     auto beginSegment = [&](int s, int flat) {
@@ -252,17 +239,17 @@ __global__ void __launch_bounds__(64) decodeBalancedKernel(DecodeArgs a, int wav
         c_len = __builtin_amdgcn_readfirstlane(static_cast<int>(len64 < max_len ? len64 : max_len));
         const S *q_ptr = static_cast<const S *>(a.q) + s * a.q_stride + (head_valid ? head : 0) * a.q_head_stride;
 #pragma unroll
-        for (int kk = 0; kk < 4; ++kk) {
+        for (int kk = 0; kk < G::kLoads; ++kk) {
             q_reg[kk] = head_valid ? *reinterpret_cast<const uint4 *>(q_ptr + 32 * kk + 8 * g) : make_uint4(0, 0, 0, 0);
         }
         // Use the query here, inside the rarely taken segment switch: the wait for it lands here and
         // the per-tile code keeps waiting for exactly its own tile, with the others still in flight.
 #pragma unroll
-        for (int kk = 0; kk < 4; ++kk) {
+        for (int kk = 0; kk < G::kLoads; ++kk) {
             asm volatile("" ::"v"(q_reg[kk].x), "v"(q_reg[kk].y), "v"(q_reg[kk].z), "v"(q_reg[kk].w));
         }
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
+        for (int e = 0; e < G::kCols; ++e) {
             st.o[e] = f32x4{0.f, 0.f, 0.f, 0.f};
         }
         st.m = -INFINITY;
@@ -283,19 +270,11 @@ __global__ void __launch_bounds__(64) decodeBalancedKernel(DecodeArgs a, int wav
             }
             const int out_head = kv_head * a.group + hg;
             if (whole) {
-                const float inv_l = 1.0f / (l_h + 1e-6f);
-                uint4 packed;
-                packed.x = T::pack2(st.o[0][rr] * inv_l, st.o[1][rr] * inv_l);
-                packed.y = T::pack2(st.o[2][rr] * inv_l, st.o[3][rr] * inv_l);
-                packed.z = T::pack2(st.o[4][rr] * inv_l, st.o[5][rr] * inv_l);
-                packed.w = T::pack2(st.o[6][rr] * inv_l, st.o[7][rr] * inv_l);
                 S *o_ptr = static_cast<S *>(a.out) + c_seq * a.o_stride + out_head * a.o_head_stride;
-                *reinterpret_cast<uint4 *>(o_ptr + 8 * c) = packed;
+                storeOutputRow<T, HEAD>(o_ptr + G::kCols * c, st, rr, 1.0f / (l_h + 1e-6f));
             } else {
                 const int64_t slot = static_cast<int64_t>(piece + c_seq) * a.num_heads + out_head;
-                float4 *pa = reinterpret_cast<float4 *>(a.part_acc + slot * kTiledHead + 8 * c);
-                pa[0] = make_float4(st.o[0][rr], st.o[1][rr], st.o[2][rr], st.o[3][rr]);
-                pa[1] = make_float4(st.o[4][rr], st.o[5][rr], st.o[6][rr], st.o[7][rr]);
+                storePartialRow<HEAD>(a.part_acc + slot * HEAD + G::kCols * c, st, rr);
                 if (c == 0) {
                     a.part_m[slot] = m_h;
                     a.part_l[slot] = l_h;
@@ -304,9 +283,10 @@ __global__ void __launch_bounds__(64) decodeBalancedKernel(DecodeArgs a, int wav
         }
     };
 
-    auto computeNextTile = [&](const TileRegs &r) {
+    auto computeNextTile = [&](const TileRegs<HEAD> &r) {
         const int tok0 = c_t * kTileTokens;
-        computeTile<T>(st, r, q_reg, k_lds, c, g, a.scale_log2, slope, tok0 - (c_len - 1), min(kTileTokens, c_len - tok0));
+        computeTile<T, HEAD>(st, r, q_reg, k_lds, lane, c, g, a.scale_log2, slope, tok0 - (c_len - 1),
+                             min(kTileTokens, c_len - tok0));
         if (++c_t == c_seg_end) {
             PA_STAMP(3);
             endSegment();
@@ -325,7 +305,7 @@ __global__ void __launch_bounds__(64) decodeBalancedKernel(DecodeArgs a, int wav
     // with theirs.
     PA_STAMP(2);
     const int n_flat = f1 - f0;
-    TileRegs buf[NBUF];
+    TileRegs<HEAD> buf[NBUF];
 #pragma unroll
     for (int i = 0; i < NBUF - 1; ++i) {
         buf[i] = loadNextTile();
@@ -345,13 +325,14 @@ __global__ void __launch_bounds__(64) decodeBalancedKernel(DecodeArgs a, int wav
 
 // Merge of the segment rows of one (query head, sequence); see decode_reduce.h for the arithmetic.
 // One wavefront per (head, sequence), four of them per workgroup. Lane = (row group g = lane / 16,
-// 8-column strip c = lane % 16): row group g merges rows g, g+4, ... of the sequence, the four
+// strip of HEAD/16 columns c = lane % 16): row group g merges rows g, g+4, ... of the sequence, the four
 // groups are then combined with lane swaps, and the lanes of group 0 store 16 bytes each. The piece
 // range of the sequence was left in seq_pieces by the decode kernel, so the only dependent memory
 // round trips are {length, piece range} -> rows.
-template <typename T, typename Tindex>
+template <typename T, typename Tindex, int HEAD>
 __global__ void __launch_bounds__(256) decodeBalancedMergeKernel(DecodeArgs a) {
     using S = typename T::storage;
+    constexpr int kCols = TileGeometry<HEAD>::kCols;
     const int head = blockIdx.x * 4 + (threadIdx.x >> 6);
     const int seq = blockIdx.y;
     const int lane = threadIdx.x & 63;
@@ -369,42 +350,49 @@ __global__ void __launch_bounds__(256) decodeBalancedMergeKernel(DecodeArgs a) {
     const int parts = pieces.y;
 
     float m_loc = -INFINITY, l_loc = 0.0f;
-    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    float acc[kCols];
+#pragma unroll
+    for (int i = 0; i < kCols; ++i) {
+        acc[i] = 0.0f;
+    }
     for (int p = g; p < parts; p += 4) {
         const int64_t slot = static_cast<int64_t>(piece_first + p + seq) * a.num_heads + head;
         const float m_p = a.part_m[slot];
         const float l_p = a.part_l[slot];
-        const float4 *row = reinterpret_cast<const float4 *>(a.part_acc + slot * kTiledHead + 8 * c);
-        const float4 v0 = row[0], v1 = row[1];
+        const float4 *row = reinterpret_cast<const float4 *>(a.part_acc + slot * HEAD + kCols * c);
+        float4 v[kCols / 4];
+#pragma unroll
+        for (int i = 0; i < kCols / 4; ++i) {
+            v[i] = row[i];
+        }
         const float m_new = fmaxf(m_loc, m_p);
         const float w_old = mergeWeight(m_loc, m_new), w_p = mergeWeight(m_p, m_new);
         l_loc = l_loc * w_old + l_p * w_p;
-        acc[0] = acc[0] * w_old + v0.x * w_p;
-        acc[1] = acc[1] * w_old + v0.y * w_p;
-        acc[2] = acc[2] * w_old + v0.z * w_p;
-        acc[3] = acc[3] * w_old + v0.w * w_p;
-        acc[4] = acc[4] * w_old + v1.x * w_p;
-        acc[5] = acc[5] * w_old + v1.y * w_p;
-        acc[6] = acc[6] * w_old + v1.z * w_p;
-        acc[7] = acc[7] * w_old + v1.w * w_p;
+#pragma unroll
+        for (int i = 0; i < kCols / 4; ++i) {
+            acc[4 * i + 0] = acc[4 * i + 0] * w_old + v[i].x * w_p;
+            acc[4 * i + 1] = acc[4 * i + 1] * w_old + v[i].y * w_p;
+            acc[4 * i + 2] = acc[4 * i + 2] * w_old + v[i].z * w_p;
+            acc[4 * i + 3] = acc[4 * i + 3] * w_old + v[i].w * w_p;
+        }
         m_loc = m_new;
     }
     const float m_all = swapMax(m_loc);
     const float f = mergeWeight(m_loc, m_all);
     const float l_all = swapSum(l_loc * f);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
+    for (int i = 0; i < kCols; ++i) {
         acc[i] = swapSum(acc[i] * f);
     }
     if (g == 0) {
         const float inv_l = 1.0f / (l_all + 1e-6f);
-        uint4 packed;
-        packed.x = T::pack2(acc[0] * inv_l, acc[1] * inv_l);
-        packed.y = T::pack2(acc[2] * inv_l, acc[3] * inv_l);
-        packed.z = T::pack2(acc[4] * inv_l, acc[5] * inv_l);
-        packed.w = T::pack2(acc[6] * inv_l, acc[7] * inv_l);
+        uint32_t w[kCols / 2];
+#pragma unroll
+        for (int i = 0; i < kCols / 2; ++i) {
+            w[i] = T::pack2(acc[2 * i] * inv_l, acc[2 * i + 1] * inv_l);
+        }
         S *o_ptr = static_cast<S *>(a.out) + seq * a.o_stride + head * a.o_head_stride;
-        *reinterpret_cast<uint4 *>(o_ptr + 8 * c) = packed;
+        storeStrip<HEAD>(o_ptr + kCols * c, w);
     }
 }
 

@@ -81,13 +81,39 @@ struct TileF16 : Half {
 };
 
 constexpr int kTileTokens = 16;     // tokens per tile = rows of one matrix instruction
-constexpr int kTiledHead = 128;     // head_size = value_size handled by this kernel
+constexpr int kTiledHead = 128;     // the head size the kernels were tuned on (others: 64, 192, 256)
 constexpr int kHeadsPerWave = 16;   // query heads of one KV head packed into one wavefront
 
+// Geometry of a 16-token tile for head_size = value_size = HEAD (64, 128, 192 or 256).
+//   K: 16 rows of HEAD/8 16-byte chunks; the wavefront fetches them in kLoads = HEAD/32 instructions,
+//      lane i of instruction j taking flat chunk 64 j + i (so every instruction covers whole rows when
+//      rows are packed). In LDS row r keeps its chunks XOR-swizzled by (r mod kSwizzle).
+//   V: lane (g, c) fetches rows 4g..4g+3, columns c*kCols .. c*kCols + kCols - 1 (kCols = HEAD/16, so
+//      2*kCols bytes per row): the lane that loads a strip is the lane that feeds it to the matrix unit
+//      and the lane that later owns those output columns.
+template <int HEAD>
+struct TileGeometry {
+    static_assert(HEAD == 64 || HEAD == 128 || HEAD == 192 || HEAD == 256, "head sizes of the tiled kernels");
+    static constexpr int kLoads = HEAD / 32;          // K load instructions per tile = K-steps of K.Q^T
+    static constexpr int kChunksPerRow = HEAD / 8;    // 16-byte chunks in one K row
+    static constexpr int kSwizzle = (HEAD == 64 || HEAD == 192) ? 8 : 16;
+    static constexpr int kCols = HEAD / 16;           // V / output columns per lane
+    static constexpr int kWords = kCols / 2;          // dwords of one V row strip
+    // register sets in flight: about 16 KiB of requests per wavefront whatever the head size
+    static constexpr int kBuffers = HEAD == 64 ? 5 : (HEAD == 256 ? 2 : 3);
+    static __device__ __forceinline__ int kRow(int j, int lane) { return (64 * j + lane) / kChunksPerRow; }
+    static __device__ __forceinline__ int kChunk(int j, int lane) { return (64 * j + lane) % kChunksPerRow; }
+    // position (in 16-byte units) of chunk `chunk` of row `row` in the LDS tile
+    static __device__ __forceinline__ int ldsIndex(int row, int chunk) {
+        return row * kChunksPerRow + (chunk ^ (row & (kSwizzle - 1)));
+    }
+};
+
 // K and V rows of one 16-token tile as they come out of the global loads; kept in registers.
+template <int HEAD>
 struct TileRegs {
-    uint4 k0, k1, k2, k3; // k<j>: token row 4j+g, columns 8c..8c+7
-    uint4 v0, v1, v2, v3; // v<j>: token row 4g+j, columns 8c..8c+7
+    uint4 k[TileGeometry<HEAD>::kLoads];        // k[j]: flat chunk 64 j + lane of the tile
+    uint32_t v[4][TileGeometry<HEAD>::kWords];  // v[j]: token row 4g+j, columns c*kCols ..
 };
 
 // 16-byte load from (wave-uniform base) + (32-bit per-lane byte offset). The empty asm keeps the
@@ -120,28 +146,97 @@ __device__ __forceinline__ float sumAcrossTokenGroups(float x) {
     return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
-// Softmax state of one wavefront. o[e][r] = O[head 4g+r of the chunk][column 8c+e].
+// 8-byte flavour of loadLane16, for row strips that are not a multiple of 16 bytes
+__device__ __forceinline__ uint2 loadLane8(const char *uniform_base, uint32_t lane_offset) {
+    asm volatile("" : "+v"(lane_offset));
+    typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+    const u32x2 v = __builtin_nontemporal_load(reinterpret_cast<const u32x2 *>(uniform_base + lane_offset));
+    return make_uint2(v[0], v[1]);
+}
+
+// This lane's strip of one V row: 2 * kCols bytes at uniform_base + lane_offset
+template <int HEAD>
+__device__ __forceinline__ void loadStrip(const char *uniform_base, uint32_t lane_offset,
+                                          uint32_t (&w)[TileGeometry<HEAD>::kWords]) {
+    constexpr int kWords = TileGeometry<HEAD>::kWords;
+    if constexpr (kWords % 4 == 0) {
+#pragma unroll
+        for (int i = 0; i < kWords / 4; ++i) {
+            const uint4 x = loadLane16(uniform_base, lane_offset + 16 * i);
+            w[4 * i] = x.x, w[4 * i + 1] = x.y, w[4 * i + 2] = x.z, w[4 * i + 3] = x.w;
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < kWords / 2; ++i) {
+            const uint2 x = loadLane8(uniform_base, lane_offset + 8 * i);
+            w[2 * i] = x.x, w[2 * i + 1] = x.y;
+        }
+    }
+}
+
+// kCols consecutive output values of one row, packed two per dword, to dst (2 * kCols bytes; 16-byte
+// stores when the strip is a multiple of 16 bytes, else 8-byte stores)
+template <int HEAD>
+__device__ __forceinline__ void storeStrip(void *dst, const uint32_t (&w)[TileGeometry<HEAD>::kWords]) {
+    constexpr int kWords = TileGeometry<HEAD>::kWords;
+    if constexpr (kWords % 4 == 0) {
+#pragma unroll
+        for (int i = 0; i < kWords / 4; ++i) {
+            reinterpret_cast<uint4 *>(dst)[i] = make_uint4(w[4 * i], w[4 * i + 1], w[4 * i + 2], w[4 * i + 3]);
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < kWords / 2; ++i) {
+            reinterpret_cast<uint2 *>(dst)[i] = make_uint2(w[2 * i], w[2 * i + 1]);
+        }
+    }
+}
+
+// Softmax state of one wavefront. o[e][r] = O[head 4g+r of the chunk][column c*kCols + e].
+template <int HEAD>
 struct TileState {
-    f32x4 o[8];
+    f32x4 o[TileGeometry<HEAD>::kCols];
     float m; // running maximum of head c (same value in the four lanes g = 0..3)
     float l; // sum of rounded probabilities of head c over this lane's tokens only
 };
 
+// Row rr of the accumulators, scaled, rounded to the storage dtype and written to dst
+template <typename T, int HEAD>
+__device__ __forceinline__ void storeOutputRow(void *dst, const TileState<HEAD> &st, int rr, float factor) {
+    uint32_t w[TileGeometry<HEAD>::kWords];
+#pragma unroll
+    for (int i = 0; i < TileGeometry<HEAD>::kWords; ++i) {
+        w[i] = T::pack2(st.o[2 * i][rr] * factor, st.o[2 * i + 1][rr] * factor);
+    }
+    storeStrip<HEAD>(dst, w);
+}
+
+// Row rr of the accumulators as fp32 partial result (kCols floats, 16-byte aligned)
+template <int HEAD>
+__device__ __forceinline__ void storePartialRow(float *dst, const TileState<HEAD> &st, int rr) {
+#pragma unroll
+    for (int i = 0; i < TileGeometry<HEAD>::kCols / 4; ++i) {
+        reinterpret_cast<float4 *>(dst)[i] = make_float4(st.o[4 * i][rr], st.o[4 * i + 1][rr], st.o[4 * i + 2][rr], st.o[4 * i + 3][rr]);
+    }
+}
+
 // One tile: scores, online softmax, accumulate. `valid` = tokens of the tile that belong to the
 // sequence (16 except possibly in the last tile).
-template <typename T>
-__device__ __forceinline__ void computeTile(TileState &st, const TileRegs r, const uint4 (&q_reg)[4], uint4 *k_lds,
+template <typename T, int HEAD>
+__device__ __forceinline__ void computeTile(TileState<HEAD> &st, const TileRegs<HEAD> r,
+                                            const uint4 (&q_reg)[TileGeometry<HEAD>::kLoads], uint4 *k_lds, int lane,
                                             int c, int g, float scale_log2, float slope, int rel_pos0, int valid) {
+    using G = TileGeometry<HEAD>;
     // K: registers -> swizzled LDS -> matrix-operand layout (token c, columns 32*kk + 8g .. +7)
-    k_lds[(g) * 16 + (c ^ (g))] = r.k0;
-    k_lds[(4 + g) * 16 + (c ^ (4 + g))] = r.k1;
-    k_lds[(8 + g) * 16 + (c ^ (8 + g))] = r.k2;
-    k_lds[(12 + g) * 16 + (c ^ (12 + g))] = r.k3;
+#pragma unroll
+    for (int j = 0; j < G::kLoads; ++j) {
+        k_lds[G::ldsIndex(G::kRow(j, lane), G::kChunk(j, lane))] = r.k[j];
+    }
     __builtin_amdgcn_wave_barrier();
     f32x4 s = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int kk = 0; kk < 4; ++kk) {
-        s = T::mfmaK32(k_lds[c * 16 + ((4 * kk + g) ^ c)], q_reg[kk], s);
+    for (int kk = 0; kk < G::kLoads; ++kk) {
+        s = T::mfmaK32(k_lds[G::ldsIndex(c, 4 * kk + g)], q_reg[kk], s);
     }
     __builtin_amdgcn_wave_barrier();
 
@@ -167,7 +262,7 @@ __device__ __forceinline__ void computeTile(TileState &st, const TileRegs r, con
         for (int rr = 0; rr < 4; ++rr) {
             const float alpha_r = __shfl(alpha, 4 * g + rr, 64);
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
+            for (int e = 0; e < G::kCols; ++e) {
                 st.o[e][rr] *= alpha_r;
             }
         }
@@ -191,26 +286,22 @@ __device__ __forceinline__ void computeTile(TileState &st, const TileRegs r, con
     }
     st.l += p_used;
 
-    // V rows beyond the sequence may hold anything (NaN included) and 0 * NaN is NaN: zero them.
-    typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
-    u32x4 v0 = __builtin_bit_cast(u32x4, r.v0), v1 = __builtin_bit_cast(u32x4, r.v1);
-    u32x4 v2 = __builtin_bit_cast(u32x4, r.v2), v3 = __builtin_bit_cast(u32x4, r.v3);
-    if (tail) {
-        const u32x4 zero = {0u, 0u, 0u, 0u};
-        v0 = (4 * g + 0 >= valid) ? zero : v0;
-        v1 = (4 * g + 1 >= valid) ? zero : v1;
-        v2 = (4 * g + 2 >= valid) ? zero : v2;
-        v3 = (4 * g + 3 >= valid) ? zero : v3;
-    }
-
-    // O += P . V, one 16-column output tile per e: column 8c+e of rows 4g..4g+3
+    // O += P . V, one 16-column output tile per e: column c*kCols + e of rows 4g..4g+3. V rows beyond
+    // the sequence may hold anything (NaN included) and 0 * NaN is NaN: they are zeroed.
 #pragma unroll
-    for (int w = 0; w < 4; ++w) {
+    for (int w = 0; w < G::kWords; ++w) {
+        uint32_t v0 = r.v[0][w], v1 = r.v[1][w], v2 = r.v[2][w], v3 = r.v[3][w];
+        if (tail) {
+            v0 = (4 * g + 0 >= valid) ? 0u : v0;
+            v1 = (4 * g + 1 >= valid) ? 0u : v1;
+            v2 = (4 * g + 2 >= valid) ? 0u : v2;
+            v3 = (4 * g + 3 >= valid) ? 0u : v3;
+        }
         uint2 even, odd;
-        even.x = __builtin_amdgcn_perm(v1[w], v0[w], 0x05040100u);
-        even.y = __builtin_amdgcn_perm(v3[w], v2[w], 0x05040100u);
-        odd.x = __builtin_amdgcn_perm(v1[w], v0[w], 0x07060302u);
-        odd.y = __builtin_amdgcn_perm(v3[w], v2[w], 0x07060302u);
+        even.x = __builtin_amdgcn_perm(v1, v0, 0x05040100u);
+        even.y = __builtin_amdgcn_perm(v3, v2, 0x05040100u);
+        odd.x = __builtin_amdgcn_perm(v1, v0, 0x07060302u);
+        odd.y = __builtin_amdgcn_perm(v3, v2, 0x07060302u);
         st.o[2 * w] = T::mfmaK16(p_op, even, st.o[2 * w]);
         st.o[2 * w + 1] = T::mfmaK16(p_op, odd, st.o[2 * w + 1]);
         if constexpr (T::kSplitProbabilities) {
@@ -226,7 +317,7 @@ __device__ __forceinline__ void computeTile(TileState &st, const TileRegs r, con
 // index (it neutralises indices past the end); compute() is skipped for those.
 template <int NBUF, typename Load, typename Compute>
 __device__ __forceinline__ void streamTiles(int n_tiles, Load loadTile, Compute compute) {
-    TileRegs buf[NBUF];
+    decltype(loadTile(0)) buf[NBUF];
 #pragma unroll
     for (int i = 0; i < NBUF - 1; ++i) {
         buf[i] = loadTile(i);
@@ -242,17 +333,48 @@ __device__ __forceinline__ void streamTiles(int n_tiles, Load loadTile, Compute 
     }
 }
 
-#ifndef INFINIOP_AMD_PA_GRID_BUFFERS
-#define INFINIOP_AMD_PA_GRID_BUFFERS 3
-#endif
-#ifndef INFINIOP_AMD_PA_BALANCED_BUFFERS
-#define INFINIOP_AMD_PA_BALANCED_BUFFERS 3
-#endif
+// Byte offsets of a lane's pieces inside a tile. They do not change from tile to tile, so a tile's
+// loads are "wave-uniform tile address + constant lane offset" and need no per-tile vector address
+// arithmetic.
+template <int HEAD>
+struct LaneOffsets {
+    uint32_t k[TileGeometry<HEAD>::kLoads];
+    uint32_t v[4];
+    __device__ __forceinline__ LaneOffsets(int lane, uint32_t k_row_bytes, uint32_t v_row_bytes) {
+        using G = TileGeometry<HEAD>;
+#pragma unroll
+        for (int j = 0; j < G::kLoads; ++j) {
+            k[j] = G::kRow(j, lane) * k_row_bytes + 16 * G::kChunk(j, lane);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            v[j] = (4 * (lane >> 4) + j) * v_row_bytes + 2 * G::kCols * (lane & 15);
+        }
+    }
+};
 
-template <typename T, typename Tindex>
+// The eight-plus loads of one tile. lane_mask = 0 turns them into harmless reads of the first bytes
+// of the tile (all lanes the same address: one request instead of a tile's worth).
+template <int HEAD>
+__device__ __forceinline__ TileRegs<HEAD> loadTileRegs(const char *k_tile, const char *v_tile, const LaneOffsets<HEAD> &off,
+                                                       uint32_t lane_mask) {
+    TileRegs<HEAD> r;
+#pragma unroll
+    for (int j = 0; j < TileGeometry<HEAD>::kLoads; ++j) {
+        r.k[j] = loadLane16(k_tile, off.k[j] & lane_mask);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        loadStrip<HEAD>(v_tile, off.v[j] & lane_mask, r.v[j]);
+    }
+    return r;
+}
+
+template <typename T, typename Tindex, int HEAD>
 __global__ void __launch_bounds__(64) decodeTiledKernel(DecodeArgs a) {
     using S = typename T::storage;
-    __shared__ uint4 k_lds[kTileTokens * kTiledHead / 8]; // one K tile, 4 KiB
+    using G = TileGeometry<HEAD>;
+    __shared__ uint4 k_lds[kTileTokens * G::kChunksPerRow]; // one K tile
 
     const int part = blockIdx.x;
     const int head_chunks = (a.group + kHeadsPerWave - 1) / kHeadsPerWave;
@@ -285,15 +407,15 @@ __global__ void __launch_bounds__(64) decodeTiledKernel(DecodeArgs a) {
             loadIndex<Tindex>(a.block_tables, seq * a.block_table_batch_stride + first_entry + lane), a.num_blocks);
     }
 
-    // Query of head (chunk*16 + c), as the B operand of the four K-steps: columns 32*kk + 8g .. +7.
+    // Query of head (chunk*16 + c), as the B operand of the K-steps: columns 32*kk + 8g .. +7.
     const int head_in_group = chunk * kHeadsPerWave + c;
     const bool head_valid = head_in_group < a.group;
     const int head = kv_head * a.group + head_in_group;
-    uint4 q_reg[4];
+    uint4 q_reg[G::kLoads];
     {
         const S *q_ptr = static_cast<const S *>(a.q) + seq * a.q_stride + (head_valid ? head : 0) * a.q_head_stride;
 #pragma unroll
-        for (int kk = 0; kk < 4; ++kk) {
+        for (int kk = 0; kk < G::kLoads; ++kk) {
             q_reg[kk] = head_valid ? *reinterpret_cast<const uint4 *>(q_ptr + 32 * kk + 8 * g) : make_uint4(0, 0, 0, 0);
         }
     }
@@ -302,22 +424,13 @@ __global__ void __launch_bounds__(64) decodeTiledKernel(DecodeArgs a) {
     const char *k_head = reinterpret_cast<const char *>(static_cast<const S *>(a.k_cache) + kv_head * a.k_head_stride);
     const char *v_head = reinterpret_cast<const char *>(static_cast<const S *>(a.v_cache) + kv_head * a.v_head_stride);
     const int block_mask = a.block_size - 1;
-    // Byte offsets of this lane's eight 16-byte pieces inside a tile. They do not change from tile
-    // to tile, so a tile's loads are "wave-uniform tile address + constant lane offset" and need no
-    // per-tile vector address arithmetic.
-    const uint32_t k_row_bytes = static_cast<uint32_t>(a.k_row_stride) * sizeof(S);
-    const uint32_t v_row_bytes = static_cast<uint32_t>(a.v_row_stride) * sizeof(S);
-    uint32_t k_off[4], v_off[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        k_off[j] = (4 * j + g) * k_row_bytes + 16 * c;
-        v_off[j] = (4 * g + j) * v_row_bytes + 16 * c;
-    }
+    const LaneOffsets<HEAD> off(lane, static_cast<uint32_t>(a.k_row_stride) * sizeof(S),
+                                static_cast<uint32_t>(a.v_row_stride) * sizeof(S));
 
     // The loop body is branch-free with a fixed number of loads in flight, so it also issues loads
     // for tile indices past the end of the partition. Those are made harmless: every lane reads the
-    // same 16 bytes (the start of the partition's first tile), one request instead of eight KiB.
-    auto loadTile = [&](int t) -> TileRegs {
+    // same few bytes (the start of the partition's first tile).
+    auto loadTile = [&](int t) -> TileRegs<HEAD> {
         const bool real = t < n_tiles;
         const uint32_t lane_mask = real ? 0xffffffffu : 0u;
         const int tok0 = start + (real ? t : 0) * kTileTokens;
@@ -325,32 +438,24 @@ __global__ void __launch_bounds__(64) decodeTiledKernel(DecodeArgs a) {
         const int row0 = tok0 & block_mask;
         const char *k_tile = k_head + (page * a.k_batch_stride + row0 * a.k_row_stride) * static_cast<int64_t>(sizeof(S));
         const char *v_tile = v_head + (page * a.v_batch_stride + row0 * a.v_row_stride) * static_cast<int64_t>(sizeof(S));
-        TileRegs r;
-        r.k0 = loadLane16(k_tile, k_off[0] & lane_mask);
-        r.k1 = loadLane16(k_tile, k_off[1] & lane_mask);
-        r.k2 = loadLane16(k_tile, k_off[2] & lane_mask);
-        r.k3 = loadLane16(k_tile, k_off[3] & lane_mask);
-        r.v0 = loadLane16(v_tile, v_off[0] & lane_mask);
-        r.v1 = loadLane16(v_tile, v_off[1] & lane_mask);
-        r.v2 = loadLane16(v_tile, v_off[2] & lane_mask);
-        r.v3 = loadLane16(v_tile, v_off[3] & lane_mask);
-        return r;
+        return loadTileRegs<HEAD>(k_tile, v_tile, off, lane_mask);
     };
 
-    TileState st;
+    TileState<HEAD> st;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
+    for (int e = 0; e < G::kCols; ++e) {
         st.o[e] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
     st.m = -INFINITY;
     st.l = 0.0f;
 
-    auto compute = [&](int t, const TileRegs &r) {
+    auto compute = [&](int t, const TileRegs<HEAD> &r) {
         const int tok0 = start + t * kTileTokens;
-        computeTile<T>(st, r, q_reg, k_lds, c, g, a.scale_log2, slope, tok0 - (len - 1), min(kTileTokens, end - tok0));
+        computeTile<T, HEAD>(st, r, q_reg, k_lds, lane, c, g, a.scale_log2, slope, tok0 - (len - 1),
+                             min(kTileTokens, end - tok0));
     };
 
-    streamTiles<INFINIOP_AMD_PA_GRID_BUFFERS>(n_tiles, loadTile, compute);
+    streamTiles<G::kBuffers>(n_tiles, loadTile, compute);
 
     // Epilogue. Denominator of head c over all 16 token slots, then move per-head scalars to the
     // lanes that hold that head's accumulators.
@@ -368,19 +473,11 @@ __global__ void __launch_bounds__(64) decodeTiledKernel(DecodeArgs a) {
         }
         const int out_head = kv_head * a.group + hg;
         if (single) {
-            const float inv_l = 1.0f / (l_h + 1e-6f);
-            uint4 packed;
-            packed.x = T::pack2(st.o[0][rr] * inv_l, st.o[1][rr] * inv_l);
-            packed.y = T::pack2(st.o[2][rr] * inv_l, st.o[3][rr] * inv_l);
-            packed.z = T::pack2(st.o[4][rr] * inv_l, st.o[5][rr] * inv_l);
-            packed.w = T::pack2(st.o[6][rr] * inv_l, st.o[7][rr] * inv_l);
             S *o_ptr = static_cast<S *>(a.out) + seq * a.o_stride + out_head * a.o_head_stride;
-            *reinterpret_cast<uint4 *>(o_ptr + 8 * c) = packed;
+            storeOutputRow<T, HEAD>(o_ptr + G::kCols * c, st, rr, 1.0f / (l_h + 1e-6f));
         } else {
             const int64_t slot = (static_cast<int64_t>(seq) * a.num_heads + out_head) * a.max_partitions + part;
-            float4 *pa = reinterpret_cast<float4 *>(a.part_acc + slot * kTiledHead + 8 * c);
-            pa[0] = make_float4(st.o[0][rr], st.o[1][rr], st.o[2][rr], st.o[3][rr]);
-            pa[1] = make_float4(st.o[4][rr], st.o[5][rr], st.o[6][rr], st.o[7][rr]);
+            storePartialRow<HEAD>(a.part_acc + slot * HEAD + G::kCols * c, st, rr);
             if (c == 0) {
                 a.part_m[slot] = m_h;
                 a.part_l[slot] = l_h;

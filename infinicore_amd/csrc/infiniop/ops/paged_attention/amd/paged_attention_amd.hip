@@ -21,7 +21,7 @@ namespace {
 // Decided once, at descriptor creation, from shapes and the device alone (sequence lengths live in
 // device memory and are never read on the host).
 struct Plan {
-    bool tiled;            // tiled matrix-core kernel (head 128, power-of-two pages >= 16, 16-byte aligned strides)
+    bool tiled;            // tiled matrix-core kernel (head 64 / 128 / 192 / 256, power-of-two pages >= 16, 16-byte aligned strides)
     bool balanced;         // tiled kernel under the work-equalising schedule (decode_balanced.h)
     int partition_tokens;  // grid schedule: tokens per unit of work
     int max_partitions;    // grid schedule: partitions the longest representable sequence needs
@@ -52,7 +52,8 @@ Plan makePlan(const PagedAttentionInfo &in, const device::amd::DeviceInfo &dev) 
     const long long max_tokens = static_cast<long long>(in.max_num_blocks_per_seq) * bs;
     const bool pow2_page = bs >= 16 && (bs & (bs - 1)) == 0;
 
-    plan.tiled = in.head_size == kTiledHead && in.value_size == kTiledHead && pow2_page
+    const bool tiled_head = in.head_size == 64 || in.head_size == 128 || in.head_size == 192 || in.head_size == 256;
+    plan.tiled = tiled_head && in.value_size == in.head_size && pow2_page
               && multipleOf8(in.q_stride) && multipleOf8(in.q_head_stride) && multipleOf8(in.o_stride)
               && multipleOf8(in.o_head_stride) && multipleOf8(in.k_batch_stride) && multipleOf8(in.k_head_stride)
               && multipleOf8(in.k_row_stride) && multipleOf8(in.v_batch_stride) && multipleOf8(in.v_head_stride)
@@ -152,18 +153,32 @@ void launchReduce(const DecodeArgs &a, hipStream_t stream) {
     }
 }
 
+// The tiled kernels of one head size: work-equalising schedule + merge, or fixed partitions.
+template <typename T, typename Tindex, int HEAD>
+void launchTiled(const DecodeArgs &a, const Plan &plan, hipStream_t stream) {
+    const int head_chunks = (a.group + kHeadsPerWave - 1) / kHeadsPerWave;
+    if (plan.balanced) {
+        const dim3 grid(plan.waves_per_stream, a.num_kv_heads * head_chunks);
+        decodeBalancedKernel<T, Tindex, HEAD><<<grid, 64, 0, stream>>>(a, plan.waves_per_stream);
+        decodeBalancedMergeKernel<T, Tindex, HEAD><<<dim3((a.num_heads + 3) / 4, a.num_seqs), 256, 0, stream>>>(a);
+    } else {
+        const dim3 grid(plan.max_partitions, a.num_kv_heads * head_chunks, a.num_seqs);
+        decodeTiledKernel<T, Tindex, HEAD><<<grid, 64, 0, stream>>>(a);
+    }
+}
+
 template <typename T, typename Tindex>
 void launchAll(const DecodeArgs &a, const Plan &plan, bool tiled, hipStream_t stream) {
-    const int head_chunks = (a.group + kHeadsPerWave - 1) / kHeadsPerWave;
-    if (tiled && plan.balanced) {
-        const dim3 grid(plan.waves_per_stream, a.num_kv_heads * head_chunks);
-        decodeBalancedKernel<T, Tindex><<<grid, 64, 0, stream>>>(a, plan.waves_per_stream);
-        decodeBalancedMergeKernel<T, Tindex><<<dim3((a.num_heads + 3) / 4, a.num_seqs), 256, 0, stream>>>(a);
-        return;
-    }
     if (tiled) {
-        const dim3 grid(plan.max_partitions, a.num_kv_heads * head_chunks, a.num_seqs);
-        decodeTiledKernel<T, Tindex><<<grid, 64, 0, stream>>>(a);
+        switch (a.head_size) {
+        case 64: launchTiled<T, Tindex, 64>(a, plan, stream); break;
+        case 128: launchTiled<T, Tindex, 128>(a, plan, stream); break;
+        case 192: launchTiled<T, Tindex, 192>(a, plan, stream); break;
+        default: launchTiled<T, Tindex, 256>(a, plan, stream); break;
+        }
+        if (plan.balanced) {
+            return; // merged by its own kernel
+        }
     } else {
         launchGeneric<typename T::Base, Tindex>(a, plan, stream);
     }
@@ -197,10 +212,10 @@ extern "C" __attribute__((visibility("default"))) int infiniopAmdPaTraceSet(void
 extern "C" __attribute__((visibility("default"))) int infiniopAmdPaOccupancy() {
     int blocks = -1;
     hipFuncAttributes attr{};
-    (void)hipFuncGetAttributes(&attr, reinterpret_cast<const void *>(&decodeBalancedKernel<TileBF16, IndexI64>));
+    (void)hipFuncGetAttributes(&attr, reinterpret_cast<const void *>(&decodeBalancedKernel<TileBF16, IndexI64, 128>));
     std::fprintf(stderr, "decodeBalancedKernel: numRegs=%d sharedSizeBytes=%zu localSizeBytes=%zu maxThreadsPerBlock=%d\n",
                  attr.numRegs, attr.sharedSizeBytes, attr.localSizeBytes, attr.maxThreadsPerBlock);
-    (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, decodeBalancedKernel<TileBF16, IndexI64>, 64, 0);
+    (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, decodeBalancedKernel<TileBF16, IndexI64, 128>, 64, 0);
     return blocks;
 }
 #endif

@@ -146,6 +146,62 @@ def test_mla_key_576_value_512(gpu_handle, oracle, dtype):
     assert_close(got, oracle.paged_attention(q, k, v, bt, sl, scale), "mla")
 
 
+# ---- head sizes of the tiled kernels -------------------------------------------------------------------
+
+@pytest.mark.parametrize("schedule", [None, "grid"])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("D", [64, 192, 256])
+def test_tiled_kernels_other_head_sizes(gpu_handle, oracle, monkeypatch, D, dtype, schedule):
+    """Head sizes 64 / 192 / 256 on the matrix-core kernels, both schedules: ragged lengths incl. 1 token and
+    exactly one page, GQA 4, long enough that sequences are split and merged."""
+    if schedule:
+        monkeypatch.setenv("INFINIOP_AMD_PA_SCHEDULE", schedule)
+    cfg = custom(f"head{D}_{schedule}", dtype, 6, 16, 4, D, 16, 1, 2500, seed=300 + D)
+    inp = workloads.make_decode_inputs(cfg)
+    inp.seq_lens[0], inp.seq_lens[1] = 1, 16
+    run_case(gpu_handle, oracle, inp)
+
+
+@pytest.mark.parametrize("D", [64, 192, 256])
+def test_other_head_sizes_match_the_elementwise_kernel_bit_for_bit_in_layout(gpu_handle, oracle, monkeypatch, D):
+    """Every output column lands where the element-wise kernel puts it: V with a distinct constant per
+    column makes the expected output that constant, whatever the softmax does."""
+    cfg = custom(f"cols{D}", torch.float16, 3, 8, 2, D, 16, 40, 700, seed=310 + D)
+    inp = workloads.make_decode_inputs(cfg)
+    ramp = (torch.arange(D, dtype=torch.float32) - D / 2) / 8
+    inp.v_cache[:] = ramp.to(torch.float16)
+    got = run_paged_attention(gpu_handle, *to_device(inp), inp.scale).float().cpu()
+    want = ramp.to(torch.float16).float().expand_as(got)
+    assert torch.allclose(got, want, atol=2e-3 * float(ramp.abs().max()), rtol=0), (got - want).abs().max()
+
+
+@pytest.mark.parametrize("D", [64, 256])
+def test_other_head_sizes_alibi_groups_pages_and_index_dtypes(gpu_handle, oracle, D):
+    cfg = custom(f"mix{D}", torch.bfloat16, 5, 40, 2, D, 64, 1, 1500, seed=320 + D)  # group of 20: two packs per KV head
+    inp = workloads.make_decode_inputs(cfg)
+    slopes = torch.tensor([2.0 ** (-(i % 8 + 1)) for i in range(40)], dtype=torch.float32)
+    q, k, v, bt, sl = to_device(inp)
+    got = run_paged_attention(gpu_handle, q, k, v, bt.to(torch.int32), sl.to(torch.int32), inp.scale, alibi=slopes.to(DEV))
+    want, want_f32 = oracle_of(oracle, inp, alibi_slopes=slopes, return_fp32=True)
+    assert_close(got, want, cfg.name, want_f32)
+
+
+@pytest.mark.parametrize("D", [64, 192, 256])
+def test_other_head_sizes_ignore_garbage_beyond_the_sequences(gpu_handle, oracle, D):
+    inp = workloads.make_decode_inputs(custom(f"poison{D}", torch.float16, 4, 8, 4, D, 16, 1, 600, seed=330 + D))
+    want = oracle_of(oracle, inp)
+    k, v = inp.k_cache.clone(), inp.v_cache.clone()
+    for s in range(4):
+        n = int(inp.seq_lens[s])
+        if n % 16:
+            page = inp.block_tables[s, (n - 1) // 16]
+            k[page, :, n % 16:, :] = float("nan")
+            v[page, :, n % 16:, :] = float("nan")
+    got = run_paged_attention(gpu_handle, inp.q.to(DEV), k.to(DEV), v.to(DEV), inp.block_tables.to(DEV),
+                              inp.seq_lens.to(DEV), inp.scale)
+    assert_close(got, want, f"poison{D}")
+
+
 # ---- every kernel and schedule against the same oracle ---------------------------------------------
 
 @pytest.mark.parametrize("kernel,schedule", [("generic", None), (None, "grid"), (None, None)])
