@@ -110,7 +110,8 @@ Plan makePlan(const PagedAttentionInfo &in, const device::amd::DeviceInfo &dev) 
         }
     }
     if (plan.balanced) {
-        int waves_per_cu = 4;
+        // head 64 moves half the bytes per tile with half the registers: two wavefronts per SIMD measured best there
+        int waves_per_cu = in.head_size == 64 ? 8 : 4;
         if (const char *env = std::getenv("INFINIOP_AMD_PA_WAVES_PER_CU")) {
             const int forced = std::atoi(env);
             waves_per_cu = forced >= 1 && forced <= 64 ? forced : waves_per_cu;

@@ -25,8 +25,8 @@ using op::paged_attention::amd::IndexU32;
 // Decided once, at descriptor creation, from shapes and the device alone (sequence lengths live in
 // device memory and are never read on the host).
 struct Plan {
-    bool tiled;          // matrix-core kernel (head 128, power-of-two pages >= 8, 16-byte aligned strides)
-    int groups_per_wave; // tiled: R = 1 or 2 column groups per wavefront -> 64 R rows per workgroup
+    bool tiled;          // matrix-core kernel (head 64 / 128 / 192 / 256, power-of-two pages >= 8, 16-byte aligned strides)
+    int groups_per_wave; // tiled: R = 1 or 2 column groups per wavefront -> 64 R rows per workgroup (heads above 128: always 1)
     int dims_per_lane;   // element-wise kernel: ceil(max(head_size, value_size) / 64)
 };
 
@@ -38,7 +38,8 @@ Plan makePlan(const PagedAttentionPrefillInfo &in, const device::amd::DeviceInfo
     const bool pow2_page = bs >= 8 && (bs & (bs - 1)) == 0;
     const long long group = static_cast<long long>(in.num_heads / in.num_kv_heads);
     const long long rows = static_cast<long long>(in.total_q_tokens) * group; // per KV head
-    plan.tiled = in.head_size == kPrefillHead && in.value_size == kPrefillHead && pow2_page
+    const bool tiled_head = in.head_size == 64 || in.head_size == 128 || in.head_size == 192 || in.head_size == 256;
+    plan.tiled = tiled_head && in.value_size == in.head_size && pow2_page
               && multipleOf8(in.q_stride) && multipleOf8(in.q_head_stride) && multipleOf8(in.o_stride)
               && multipleOf8(in.o_head_stride) && multipleOf8(in.k_batch_stride) && multipleOf8(in.k_head_stride)
               && multipleOf8(in.k_row_stride) && multipleOf8(in.v_batch_stride) && multipleOf8(in.v_head_stride)
@@ -85,24 +86,38 @@ void launchGeneric(const PrefillArgs &a, const Plan &plan, hipStream_t stream) {
     }
 }
 
-template <typename T, typename Tindex, bool PLAIN>
-void launchTiledGroups(const PrefillArgs &a, const Plan &plan, hipStream_t stream) {
+template <typename T, typename Tindex, int HEAD, bool PLAIN>
+void launchTiledHead(const PrefillArgs &a, const Plan &plan, hipStream_t stream) {
     // sum over sequences of ceil(rows / block_rows) is at most floor(total rows / block_rows) + num_seqs
     const long long rows = static_cast<long long>(a.total_q_tokens) * a.group;
-    const int block_rows = prefillBlockRows(plan.groups_per_wave);
+    const int groups = HEAD <= 128 ? plan.groups_per_wave : 1;
+    const int block_rows = prefillBlockRows(groups);
     const dim3 grid(static_cast<unsigned>((rows / block_rows + a.num_seqs) * a.num_kv_heads));
-    switch (plan.groups_per_wave) {
-    case 1: prefillTiledKernel<T, Tindex, 1, PLAIN><<<grid, kPrefillThreads, 0, stream>>>(a); break;
-    default: prefillTiledKernel<T, Tindex, 2, PLAIN><<<grid, kPrefillThreads, 0, stream>>>(a); break;
+    if constexpr (HEAD <= 128) {
+        if (groups == 2) {
+            prefillTiledKernel<T, Tindex, HEAD, 2, PLAIN><<<grid, kPrefillThreads, 0, stream>>>(a);
+            return;
+        }
+    }
+    prefillTiledKernel<T, Tindex, HEAD, 1, PLAIN><<<grid, kPrefillThreads, 0, stream>>>(a);
+}
+
+template <typename T, typename Tindex, bool PLAIN>
+void launchTiledPlain(const PrefillArgs &a, const Plan &plan, hipStream_t stream) {
+    switch (a.head_size) {
+    case 64: launchTiledHead<T, Tindex, 64, PLAIN>(a, plan, stream); break;
+    case 128: launchTiledHead<T, Tindex, 128, PLAIN>(a, plan, stream); break;
+    case 192: launchTiledHead<T, Tindex, 192, PLAIN>(a, plan, stream); break;
+    default: launchTiledHead<T, Tindex, 256, PLAIN>(a, plan, stream); break;
     }
 }
 
 template <typename T, typename Tindex>
 void launchTiled(const PrefillArgs &a, const Plan &plan, hipStream_t stream) {
     if (a.alibi_slopes == nullptr && a.scale_log2 > 0.0f) {
-        launchTiledGroups<T, Tindex, true>(a, plan, stream);
+        launchTiledPlain<T, Tindex, true>(a, plan, stream);
     } else {
-        launchTiledGroups<T, Tindex, false>(a, plan, stream);
+        launchTiledPlain<T, Tindex, false>(a, plan, stream);
     }
 }
 

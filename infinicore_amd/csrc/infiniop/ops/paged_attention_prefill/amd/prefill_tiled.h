@@ -1,20 +1,22 @@
-// Tiled prefill kernel for head_size = value_size = 128 on gfx950 (CDNA4, 64-lane wavefronts).
+// Tiled prefill kernel for head_size = value_size = 64, 128, 192 or 256 on gfx950 (CDNA4, 64-lane
+// wavefronts). Figures below are for head 128; tile geometry per head size is TileGeometry<HEAD> of
+// the decode kernels.
 //
 // Work unit: one 256-thread workgroup = 64*R "rows" of one (sequence, KV head). A row is a (new
 // token, query head of the KV head's group) pair, token-major: row = token * group + head_in_group.
 // Packing the heads of a group into the row dimension means a K/V tile fetched once serves all of
 // them, and short prompts still fill the matrix instructions. Each of the four wavefronts owns 16*R
-// consecutive rows (R = 1 or 2 column groups of 16).
+// consecutive rows (R = 1 or 2 column groups of 16; 1 only for heads above 128).
 //
-// The K/V tokens the rows may see are consumed in steps of 64. Per step the workgroup copies
-// 64 K rows and 64 V rows (16 KiB each) from the paged pool into LDS, every wavefront 16 tokens of
-// each, double-buffered: the global loads of step j+1 are in flight while step j is computed, and one
-// barrier per step separates writers and readers.
+// The K/V tokens the rows may see are consumed in steps of 64 (32 for heads above 128). Per step the
+// workgroup copies that many K rows and V rows (16 KiB each) from the paged pool into LDS, a wavefront
+// 16 tokens at a time, double-buffered: the global loads of step j+1 are in flight while step j is
+// computed, and one barrier per step separates writers and readers.
 //   * K is stored as it comes (16-byte chunks, XOR-swizzled so the later row-wise reads are
 //     conflict-free): the matrix instruction wants lane i to hold token i.
 //   * V is stored already transposed into matrix-operand order: the lane that loaded rows 4g..4g+3
-//     of an 8-column strip interleaves them per column with byte permutes and writes, for each of
-//     its 8 columns, the four tokens as one 8-byte word. A reader fetches two such words (tokens
+//     of a column strip interleaves them per column with byte permutes and writes, for each of its
+//     columns, the four tokens as one 8-byte word. A reader fetches two such words (tokens
 //     4g..4g+3 of two 16-token tiles) and has the 8-deep operand of one 16x16x32 instruction.
 //
 // Arithmetic per step and column group, lane = 16*g + c:
@@ -25,8 +27,9 @@
 //                             from the registers S came out in; B = V words from LDS; lane holds
 //                             O[row 4g + 0..3][8c + e], e = 0..7)
 //   l[row]      += P . 1       2 x v_mfma_f32_16x16x32: the denominator sums the rounded probabilities
-// K/V fragments read from LDS are shared by the R column groups of a wavefront. A step whose tokens lie beyond everything a wavefront's rows may see
-// is skipped by that wavefront (it still takes part in the copy).
+// K/V fragments read from LDS are shared by the R column groups of a wavefront. A step whose tokens
+// lie beyond everything a wavefront's rows may see is skipped by that wavefront (it still takes part
+// in the copy).
 //
 // The math follows the reference's prefill kernels (src/infiniop/ops/paged_attention_prefill/cuda/
 // kernel_v2.cuh:254-472: visible range, ALiBi distance, 1e-6 in the normaliser, rounding).
@@ -45,10 +48,11 @@ using op::paged_attention::amd::TileBF16;
 using op::paged_attention::amd::TileF16;
 
 using op::paged_attention::amd::kTileTokens;
+using op::paged_attention::amd::LaneOffsets;
+using op::paged_attention::amd::storeStrip;
+using op::paged_attention::amd::TileGeometry;
 
 constexpr int kPrefillThreads = 256;
-constexpr int kPrefillStepTokens = 64;
-constexpr int kPrefillHead = 128;
 
 // 16-byte load from (wave-uniform base) + (32-bit per-lane byte offset), through the caches: K/V tiles
 // are read again by the other row blocks of the sequence. The empty asm keeps the offset a value
@@ -98,14 +102,42 @@ __device__ __forceinline__ bool findRowBlock(const PrefillArgs &a, int lane, int
     return false;
 }
 
+// This lane's strip of one V row (2 * kCols bytes), through the caches
+template <int HEAD>
+__device__ __forceinline__ void loadStripCached(const char *src, uint32_t (&w)[TileGeometry<HEAD>::kWords]) {
+    constexpr int kWords = TileGeometry<HEAD>::kWords;
+    if constexpr (kWords % 4 == 0) {
+#pragma unroll
+        for (int i = 0; i < kWords / 4; ++i) {
+            const uint4 x = reinterpret_cast<const uint4 *>(src)[i];
+            w[4 * i] = x.x, w[4 * i + 1] = x.y, w[4 * i + 2] = x.z, w[4 * i + 3] = x.w;
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < kWords / 2; ++i) {
+            const uint2 x = reinterpret_cast<const uint2 *>(src)[i];
+            w[2 * i] = x.x, w[2 * i + 1] = x.y;
+        }
+    }
+}
+
+// Tokens per step: 64 for heads up to 128, 32 above (the two LDS buffers of K and V then stay within
+// 64 KiB and two workgroups share a compute unit).
+template <int HEAD>
+constexpr int prefillStepTokens() { return HEAD <= 128 ? 64 : 32; }
+
 // PLAIN: no ALiBi and scale > 0. The running maximum is then kept in units of the raw dot product
 // (a positive scale keeps the order) and each probability costs one fused multiply-add and one exp2.
-template <typename T, typename Tindex, int R, bool PLAIN>
-__global__ void __launch_bounds__(kPrefillThreads, 2) prefillTiledKernel(PrefillArgs a) {
+template <typename T, typename Tindex, int HEAD, int R, bool PLAIN>
+__global__ void __launch_bounds__(kPrefillThreads, HEAD <= 192 ? 2 : 1) prefillTiledKernel(PrefillArgs a) {
     using S = typename T::storage;
+    using G = TileGeometry<HEAD>;
     constexpr int BM = prefillBlockRows(R);
-    __shared__ uint4 k_lds[2][kPrefillStepTokens * 16];    // [token][16-byte chunk ^ (token & 15)]
-    __shared__ uint2 v_lds[2][8 * 4 * 4 * 16];             // [column e][16-token tile][token group g][strip c]
+    constexpr int BN = prefillStepTokens<HEAD>();
+    constexpr int TT = BN / kTileTokens;             // 16-token tiles per step: 4 or 2
+    constexpr int kTileChunks = kTileTokens * G::kChunksPerRow;
+    __shared__ uint4 k_lds[2][TT * kTileChunks];       // [tile][token][16-byte chunk, XOR-swizzled by the token]
+    __shared__ uint2 v_lds[2][G::kCols * TT * 64];     // [column e][tile][token group g][strip c]
 
     const int lane = threadIdx.x & 63;
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -134,10 +166,10 @@ __global__ void __launch_bounds__(kPrefillThreads, 2) prefillTiledKernel(Prefill
     kv_len64 = kv_len64 < 0 ? 0 : (kv_len64 > span.capacity ? span.capacity : kv_len64);
     // tokens that exist; rows beyond it are zeroed in V (they may hold anything, NaN included)
     const int kv_len = __builtin_amdgcn_readfirstlane(max(static_cast<int>(kv_len64), block_visible));
-    const int n_steps = (block_visible + kPrefillStepTokens - 1) / kPrefillStepTokens;
+    const int n_steps = (block_visible + BN - 1) / BN;
 
     // ---- this lane's columns: row c of each of the wavefront's R column groups ----
-    uint4 q_reg[R][4];
+    uint4 q_reg[R][G::kLoads];
     int visible[R];
     float slope[R];
     int wave_max_visible = 0, wave_min_visible = 0x7fffffff;
@@ -151,7 +183,7 @@ __global__ void __launch_bounds__(kPrefillThreads, 2) prefillTiledKernel(Prefill
         slope[r] = (a.alibi_slopes != nullptr && valid) ? a.alibi_slopes[head] * kLog2e : 0.0f;
         const S *q_ptr = static_cast<const S *>(a.q) + (span.q_start + token) * a.q_stride + head * a.q_head_stride;
 #pragma unroll
-        for (int kk = 0; kk < 4; ++kk) {
+        for (int kk = 0; kk < G::kLoads; ++kk) {
             q_reg[r][kk] = valid ? *reinterpret_cast<const uint4 *>(q_ptr + 32 * kk + 8 * g) : make_uint4(0, 0, 0, 0);
         }
         wave_max_visible = max(wave_max_visible, visible[r]);
@@ -165,7 +197,12 @@ __global__ void __launch_bounds__(kPrefillThreads, 2) prefillTiledKernel(Prefill
     wave_max_visible = __builtin_amdgcn_readfirstlane(wave_max_visible);
     wave_min_visible = __builtin_amdgcn_readfirstlane(wave_min_visible);
 
-    // ---- copy side: this wavefront moves tokens [64 j + 16 w, +16) of step j ----
+    // ---- copy side: per step this wavefront moves one 16-token tile of K and one of V (64-token
+    // steps: tile w of both), or one tile of either (32-token steps: wavefronts 0, 1 the K tiles,
+    // wavefronts 2, 3 the V tiles) ----
+    const bool copies_k = TT == 4 || w < 2;
+    const bool copies_v = TT == 4 || w >= 2;
+    const int copy_tile = TT == 4 ? w : (w & 1);
     const char *k_head = reinterpret_cast<const char *>(static_cast<const S *>(a.k_cache) + kv_head * a.k_head_stride);
     const char *v_head = reinterpret_cast<const char *>(static_cast<const S *>(a.v_cache) + kv_head * a.v_head_stride);
     const int64_t table_row = seq * a.block_table_batch_stride;
@@ -194,15 +231,14 @@ __global__ void __launch_bounds__(kPrefillThreads, 2) prefillTiledKernel(Prefill
         return clampPage(raw, a.num_blocks);
     };
 
-    uint32_t k_off[4], v_off[4]; // byte offsets of this lane's rows inside a 16-token tile (pages >= 16 tokens)
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        k_off[j] = static_cast<uint32_t>((4 * j + g) * a.k_row_stride * static_cast<int64_t>(sizeof(S))) + 16 * c;
-        v_off[j] = static_cast<uint32_t>((4 * g + j) * a.v_row_stride * static_cast<int64_t>(sizeof(S))) + 16 * c;
-    }
-    uint4 k_stage[4], v_stage[4];
-    auto loadStage = [&](int t) {
-        // K: rows 4 jj + g of the tile; V: rows 4 g + i. Tokens past kv_len are not fetched.
+    // byte offsets of this lane's pieces inside a 16-token tile (pages >= 16 tokens)
+    const LaneOffsets<HEAD> off(lane, static_cast<uint32_t>(a.k_row_stride) * sizeof(S),
+                                static_cast<uint32_t>(a.v_row_stride) * sizeof(S));
+    uint4 k_stage[G::kLoads];
+    uint32_t v_stage[4][G::kWords];
+    auto loadStage = [&](int step) {
+        // K: flat chunks 64 j + lane of the tile; V: rows 4 g + i. Tokens past kv_len are not fetched.
+        const int t = step * BN + kTileTokens * copy_tile;
         const int e0 = t >> a.block_shift;
         if ((min(e0, last_entry) >> 6) > id_batch) {
             ids_cur = ids_next;
@@ -212,15 +248,21 @@ __global__ void __launch_bounds__(kPrefillThreads, 2) prefillTiledKernel(Prefill
         if (t + kTileTokens <= kv_len && !small_pages) {
             const int page = pageOfEntry(e0);
             const int row0 = t & block_mask;
-            const char *k_tile = k_head + (page * a.k_batch_stride + row0 * a.k_row_stride) * static_cast<int64_t>(sizeof(S));
-            const char *v_tile = v_head + (page * a.v_batch_stride + row0 * a.v_row_stride) * static_cast<int64_t>(sizeof(S));
+            if (copies_k) {
+                const char *k_tile = k_head + (page * a.k_batch_stride + row0 * a.k_row_stride) * static_cast<int64_t>(sizeof(S));
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                k_stage[j] = loadLane16Cached(k_tile, k_off[j]);
+                for (int j = 0; j < G::kLoads; ++j) {
+                    k_stage[j] = loadLane16Cached(k_tile, off.k[j]);
+                }
             }
+            if (copies_v) {
+                const char *v_tile = v_head + (page * a.v_batch_stride + row0 * a.v_row_stride) * static_cast<int64_t>(sizeof(S));
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                v_stage[j] = loadLane16Cached(v_tile, v_off[j]);
+                for (int j = 0; j < 4; ++j) {
+                    uint32_t lane_off = off.v[j];
+                    asm volatile("" : "+v"(lane_off));
+                    loadStripCached<HEAD>(v_tile + lane_off, v_stage[j]);
+                }
             }
             return;
         }
@@ -228,55 +270,68 @@ __global__ void __launch_bounds__(kPrefillThreads, 2) prefillTiledKernel(Prefill
         const int id0 = t < kv_len ? pageOfEntry(e0) : 0;
         const int id1 = (small_pages && t < kv_len) ? pageOfEntry(e0 + 1) : id0;
         const int row0 = small_pages ? 0 : (t & block_mask);
+        if (copies_k) {
 #pragma unroll
-        for (int jj = 0; jj < 4; ++jj) {
-            const int o = 4 * jj + g;
-            const int page = (small_pages && jj >= 2) ? id1 : id0;
-            const int page_row = small_pages ? (o & 7) : row0 + o;
-            const char *src = k_head + (page * a.k_batch_stride + page_row * a.k_row_stride) * static_cast<int64_t>(sizeof(S)) + 16 * c;
-            k_stage[jj] = (t + o < kv_len) ? *reinterpret_cast<const uint4 *>(src) : make_uint4(0, 0, 0, 0);
+            for (int j = 0; j < G::kLoads; ++j) {
+                const int o = G::kRow(j, lane);
+                const int page = (small_pages && o >= 8) ? id1 : id0;
+                const int page_row = small_pages ? (o & 7) : row0 + o;
+                const char *src = k_head + (page * a.k_batch_stride + page_row * a.k_row_stride) * static_cast<int64_t>(sizeof(S))
+                                + 16 * G::kChunk(j, lane);
+                k_stage[j] = (t + o < kv_len) ? *reinterpret_cast<const uint4 *>(src) : make_uint4(0, 0, 0, 0);
+            }
         }
+        if (copies_v) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int o = 4 * g + i;
-            const int page = (small_pages && g >= 2) ? id1 : id0;
-            const int page_row = small_pages ? (o & 7) : row0 + o;
-            const char *src = v_head + (page * a.v_batch_stride + page_row * a.v_row_stride) * static_cast<int64_t>(sizeof(S)) + 16 * c;
-            v_stage[i] = (t + o < kv_len) ? *reinterpret_cast<const uint4 *>(src) : make_uint4(0, 0, 0, 0);
+            for (int i = 0; i < 4; ++i) {
+                const int o = 4 * g + i;
+                const int page = (small_pages && g >= 2) ? id1 : id0;
+                const int page_row = small_pages ? (o & 7) : row0 + o;
+                const char *src = v_head + (page * a.v_batch_stride + page_row * a.v_row_stride) * static_cast<int64_t>(sizeof(S))
+                                + 2 * G::kCols * c;
+                if (t + o < kv_len) {
+                    loadStripCached<HEAD>(src, v_stage[i]);
+                } else {
+#pragma unroll
+                    for (int wd = 0; wd < G::kWords; ++wd) {
+                        v_stage[i][wd] = 0u;
+                    }
+                }
+            }
         }
     };
     auto storeStage = [&](int buf) {
+        if (copies_k) {
 #pragma unroll
-        for (int jj = 0; jj < 4; ++jj) {
-            const int o = 4 * jj + g;
-            k_lds[buf][(16 * w + o) * 16 + (c ^ o)] = k_stage[jj];
+            for (int j = 0; j < G::kLoads; ++j) {
+                k_lds[buf][copy_tile * kTileChunks + G::ldsIndex(G::kRow(j, lane), G::kChunk(j, lane))] = k_stage[j];
+            }
         }
-        typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
-        const u32x4 v0 = __builtin_bit_cast(u32x4, v_stage[0]), v1 = __builtin_bit_cast(u32x4, v_stage[1]);
-        const u32x4 v2 = __builtin_bit_cast(u32x4, v_stage[2]), v3 = __builtin_bit_cast(u32x4, v_stage[3]);
+        if (copies_v) {
 #pragma unroll
-        for (int wd = 0; wd < 4; ++wd) {
-            uint2 even, odd;
-            even.x = __builtin_amdgcn_perm(v1[wd], v0[wd], 0x05040100u);
-            even.y = __builtin_amdgcn_perm(v3[wd], v2[wd], 0x05040100u);
-            odd.x = __builtin_amdgcn_perm(v1[wd], v0[wd], 0x07060302u);
-            odd.y = __builtin_amdgcn_perm(v3[wd], v2[wd], 0x07060302u);
-            v_lds[buf][(((2 * wd) * 4 + w) * 4 + g) * 16 + c] = even;
-            v_lds[buf][(((2 * wd + 1) * 4 + w) * 4 + g) * 16 + c] = odd;
+            for (int wd = 0; wd < G::kWords; ++wd) {
+                uint2 even, odd;
+                even.x = __builtin_amdgcn_perm(v_stage[1][wd], v_stage[0][wd], 0x05040100u);
+                even.y = __builtin_amdgcn_perm(v_stage[3][wd], v_stage[2][wd], 0x05040100u);
+                odd.x = __builtin_amdgcn_perm(v_stage[1][wd], v_stage[0][wd], 0x07060302u);
+                odd.y = __builtin_amdgcn_perm(v_stage[3][wd], v_stage[2][wd], 0x07060302u);
+                v_lds[buf][(((2 * wd) * TT + copy_tile) * 4 + g) * 16 + c] = even;
+                v_lds[buf][(((2 * wd + 1) * TT + copy_tile) * 4 + g) * 16 + c] = odd;
+            }
         }
     };
 
     // ---- softmax state ----
-    // o[r][e][rr] = O[row 4g+rr of group r][column 8c+e]; ol[r][rr] = sum of that row's probabilities
+    // o[r][e][rr] = O[row 4g+rr of group r][column c*kCols+e]; ol[r][rr] = sum of that row's probabilities
     // (computed by the matrix unit as P . 1, so it sums exactly the rounded probabilities the numerator
     // used and already sits in the accumulators' row layout); m[r] = running maximum of row c, in units
     // of the raw dot product when there is no ALiBi (scale > 0 keeps the order), else of the scaled score.
-    f32x4 o[R][8], ol[R];
+    f32x4 o[R][G::kCols], ol[R];
     float m[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
+        for (int e = 0; e < G::kCols; ++e) {
             o[r][e] = f32x4{0.f, 0.f, 0.f, 0.f};
         }
         ol[r] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -286,26 +341,26 @@ __global__ void __launch_bounds__(kPrefillThreads, 2) prefillTiledKernel(Prefill
     const uint4 ones = make_uint4(one2, one2, one2, one2);
     const float unit = PLAIN ? a.scale_log2 : 1.0f; // log2-domain size of one unit of m
 
-    // One step over the 64 tokens in LDS buffer `buf`. masked: some score of the step lies beyond
+    // One step over the BN tokens in LDS buffer `buf`. masked: some score of the step lies beyond
     // what its row may see (steps on the causal diagonal); the other steps skip the comparison.
     auto computeStep = [&](int buf, int t0, bool masked) {
-        f32x4 s[R][4];
+        f32x4 s[R][TT];
 #pragma unroll
         for (int r = 0; r < R; ++r) {
 #pragma unroll
-            for (int tt = 0; tt < 4; ++tt) {
+            for (int tt = 0; tt < TT; ++tt) {
                 s[r][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
             }
         }
 #pragma unroll
-        for (int tt = 0; tt < 4; ++tt) {
-            uint4 kf[4];
+        for (int tt = 0; tt < TT; ++tt) {
+            uint4 kf[G::kLoads];
 #pragma unroll
-            for (int kk = 0; kk < 4; ++kk) {
-                kf[kk] = k_lds[buf][(16 * tt + c) * 16 + ((4 * kk + g) ^ c)];
+            for (int kk = 0; kk < G::kLoads; ++kk) {
+                kf[kk] = k_lds[buf][tt * kTileChunks + G::ldsIndex(c, 4 * kk + g)];
             }
 #pragma unroll
-            for (int kk = 0; kk < 4; ++kk) {
+            for (int kk = 0; kk < G::kLoads; ++kk) {
 #pragma unroll
                 for (int r = 0; r < R; ++r) {
                     s[r][tt] = T::mfmaK32(kf[kk], q_reg[r][kk], s[r][tt]);
@@ -313,13 +368,13 @@ __global__ void __launch_bounds__(kPrefillThreads, 2) prefillTiledKernel(Prefill
             }
         }
 
-        uint4 p_op[R][2];
+        uint4 p_op[R][TT / 2];
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             // scores in the units m[r] is kept in
             if constexpr (!PLAIN) {
 #pragma unroll
-                for (int tt = 0; tt < 4; ++tt) {
+                for (int tt = 0; tt < TT; ++tt) {
 #pragma unroll
                     for (int rr = 0; rr < 4; ++rr) {
                         const int tok = t0 + 16 * tt + 4 * g + rr;
@@ -329,7 +384,7 @@ __global__ void __launch_bounds__(kPrefillThreads, 2) prefillTiledKernel(Prefill
             }
             if (masked) {
 #pragma unroll
-                for (int tt = 0; tt < 4; ++tt) {
+                for (int tt = 0; tt < TT; ++tt) {
 #pragma unroll
                     for (int rr = 0; rr < 4; ++rr) {
                         const int tok = t0 + 16 * tt + 4 * g + rr;
@@ -339,7 +394,7 @@ __global__ void __launch_bounds__(kPrefillThreads, 2) prefillTiledKernel(Prefill
             }
             float mx = fmaxf(fmaxf(s[r][0][0], s[r][0][1]), fmaxf(s[r][0][2], s[r][0][3]));
 #pragma unroll
-            for (int tt = 1; tt < 4; ++tt) {
+            for (int tt = 1; tt < TT; ++tt) {
                 mx = fmaxf(mx, fmaxf(fmaxf(s[r][tt][0], s[r][tt][1]), fmaxf(s[r][tt][2], s[r][tt][3])));
             }
             mx = maxAcrossTokenGroups(mx);
@@ -354,7 +409,7 @@ __global__ void __launch_bounds__(kPrefillThreads, 2) prefillTiledKernel(Prefill
                     const float alpha_r = __shfl(alpha, 4 * g + rr, 64);
                     ol[r][rr] *= alpha_r;
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) {
+                    for (int e = 0; e < G::kCols; ++e) {
                         o[r][e][rr] *= alpha_r;
                     }
                 }
@@ -362,7 +417,7 @@ __global__ void __launch_bounds__(kPrefillThreads, 2) prefillTiledKernel(Prefill
             // a row that has seen nothing yet keeps m = -inf: subtract 0, p = 2^-inf = 0
             const float shift = m[r] == -INFINITY ? 0.0f : -m[r] * unit;
 #pragma unroll
-            for (int u = 0; u < 2; ++u) {
+            for (int u = 0; u < TT / 2; ++u) {
                 uint32_t wds[4];
 #pragma unroll
                 for (int h = 0; h < 2; ++h) {
@@ -375,15 +430,15 @@ __global__ void __launch_bounds__(kPrefillThreads, 2) prefillTiledKernel(Prefill
         }
 
 #pragma unroll
-        for (int u = 0; u < 2; ++u) {
+        for (int u = 0; u < TT / 2; ++u) {
 #pragma unroll
             for (int r = 0; r < R; ++r) {
                 ol[r] = T::mfmaK32(p_op[r][u], ones, ol[r]);
             }
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const uint2 lo = v_lds[buf][((e * 4 + 2 * u) * 4 + g) * 16 + c];
-                const uint2 hi = v_lds[buf][((e * 4 + 2 * u + 1) * 4 + g) * 16 + c];
+            for (int e = 0; e < G::kCols; ++e) {
+                const uint2 lo = v_lds[buf][((e * TT + 2 * u) * 4 + g) * 16 + c];
+                const uint2 hi = v_lds[buf][((e * TT + 2 * u + 1) * 4 + g) * 16 + c];
                 const uint4 vf = make_uint4(lo.x, lo.y, hi.x, hi.y);
 #pragma unroll
                 for (int r = 0; r < R; ++r) {
@@ -394,27 +449,27 @@ __global__ void __launch_bounds__(kPrefillThreads, 2) prefillTiledKernel(Prefill
     };
 
     // ---- pipeline ----
-    loadStage(16 * w);
+    loadStage(0);
     storeStage(0);
     __syncthreads();
     if (n_steps > 1) {
-        loadStage(kPrefillStepTokens + 16 * w);
+        loadStage(1);
     }
     for (int j = 0; j < n_steps; ++j) {
-        const int t0 = j * kPrefillStepTokens;
+        const int t0 = j * BN;
         if (t0 < wave_max_visible) {
-            computeStep(j & 1, t0, t0 + kPrefillStepTokens > wave_min_visible);
+            computeStep(j & 1, t0, t0 + BN > wave_min_visible);
         }
         if (j + 1 < n_steps) {
             storeStage((j + 1) & 1);
         }
         __syncthreads();
         if (j + 2 < n_steps) {
-            loadStage((j + 2) * kPrefillStepTokens + 16 * w);
+            loadStage(j + 2);
         }
     }
 
-    // ---- normalise and store: lane writes columns 8c..8c+7 of rows 4g..4g+3 of each group ----
+    // ---- normalise and store: lane writes columns c*kCols .. of rows 4g..4g+3 of each group ----
 #pragma unroll
     for (int r = 0; r < R; ++r) {
 #pragma unroll
@@ -428,13 +483,13 @@ __global__ void __launch_bounds__(kPrefillThreads, 2) prefillTiledKernel(Prefill
             const int token = row / a.group;
             const int head = kv_head * a.group + (row - token * a.group);
             const float inv_l = 1.0f / (ol[r][rr] + 1e-6f);
-            uint4 packed;
-            packed.x = T::pack2(o[r][0][rr] * inv_l, o[r][1][rr] * inv_l);
-            packed.y = T::pack2(o[r][2][rr] * inv_l, o[r][3][rr] * inv_l);
-            packed.z = T::pack2(o[r][4][rr] * inv_l, o[r][5][rr] * inv_l);
-            packed.w = T::pack2(o[r][6][rr] * inv_l, o[r][7][rr] * inv_l);
+            uint32_t packed[G::kWords];
+#pragma unroll
+            for (int i = 0; i < G::kWords; ++i) {
+                packed[i] = T::pack2(o[r][2 * i][rr] * inv_l, o[r][2 * i + 1][rr] * inv_l);
+            }
             S *o_ptr = static_cast<S *>(a.out) + (span.q_start + token) * a.o_stride + head * a.o_head_stride;
-            *reinterpret_cast<uint4 *>(o_ptr + 8 * c) = packed;
+            storeStrip<HEAD>(o_ptr + G::kCols * c, packed);
         }
     }
 }

@@ -131,10 +131,45 @@ def test_element_wise_kernel_on_a_tiled_shape(gpu_handle, oracle, monkeypatch, d
     run_case(gpu_handle, oracle, workloads.make_prefill_inputs(cfg))
 
 
+@pytest.mark.parametrize("kernel", ["tiled", "generic"])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("D", [64, 192, 256])
-def test_other_head_sizes(gpu_handle, oracle, D):
-    cfg = prefill_config(f"head{D}", torch.float16, 3, 8, 4, D, 16, (1, 40), (0, 100), seed=41 + D)
+def test_other_head_sizes(gpu_handle, oracle, monkeypatch, D, dtype, kernel):
+    """Head sizes 64 / 192 / 256 on the matrix-core kernel (steps of 32 tokens above 128) and on the element-wise one."""
+    if kernel == "generic":
+        monkeypatch.setenv("INFINIOP_AMD_PREFILL_KERNEL", "generic")
+    small = kernel == "generic"
+    cfg = prefill_config(f"head{D}_{kernel}", dtype, 4, 8, 4, D, 16, (1, 40 if small else 260), (0, 100 if small else 400),
+                         seed=41 + D)
     run_case(gpu_handle, oracle, workloads.make_prefill_inputs(cfg))
+
+
+@pytest.mark.parametrize("D,groups", [(64, "1"), (64, "2"), (192, "1"), (256, "1")])
+def test_other_head_sizes_pages_of_8_alibi_and_int32(gpu_handle, oracle, monkeypatch, D, groups):
+    monkeypatch.setenv("INFINIOP_AMD_PREFILL_GROUPS", groups)
+    cfg = prefill_config(f"mix{D}", torch.bfloat16, 3, 12, 2, D, 8, (1, 150), (0, 300), seed=91 + D)
+    slopes = torch.tensor([2.0 ** -(i % 6 + 1) for i in range(12)], dtype=torch.float32)
+    run_case(gpu_handle, oracle, workloads.make_prefill_inputs(cfg), alibi=slopes, index_dtype=torch.int32)
+
+
+@pytest.mark.parametrize("D", [64, 192, 256])
+def test_other_head_sizes_column_layout_and_garbage(gpu_handle, oracle, D):
+    """V with a distinct constant per column makes the expected output that constant (every output column
+    lands where it belongs); NaN beyond the sequences must not leak in."""
+    cfg = prefill_config(f"cols{D}", torch.float16, 3, 8, 2, D, 16, (5, 90), (3, 200), seed=97 + D)
+    inp = workloads.make_prefill_inputs(cfg)
+    ramp = ((torch.arange(D, dtype=torch.float32) - D / 2) / 8).to(torch.float16)
+    inp.v_cache[:] = ramp
+    for s in range(cfg.num_seqs):
+        L = int(inp.seq_lens[s])
+        if L % 16:
+            page = int(inp.block_tables[s, (L - 1) // 16])
+            inp.k_cache[page, :, L % 16:, :] = float("nan")
+            inp.v_cache[page, :, L % 16:, :] = float("nan")
+    dev = [t.to(DEV) for t in (inp.q, inp.k_cache, inp.v_cache, inp.block_tables, inp.seq_lens, inp.cum_seq_lens_q)]
+    got = run_paged_attention_prefill(gpu_handle, *dev, inp.scale).float().cpu()
+    want = ramp.float().expand_as(got)
+    assert torch.allclose(got, want, atol=2e-3 * float(ramp.float().abs().max()), rtol=0), (got - want).abs().max()
 
 
 @pytest.mark.parametrize("bs", [4, 8, 32, 128, 24])
