@@ -21,6 +21,7 @@ from __future__ import annotations
 
 import argparse
 import ctypes
+import dataclasses
 import json
 import os
 import sys
@@ -47,6 +48,9 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=None, help="default 400 (decode) / 50 (prefill)")
     ap.add_argument("--warmup", type=int, default=None, help="default 40 (decode) / 5 (prefill)")
     ap.add_argument("--workload", default="c2_llama3_8b_b32")
+    ap.add_argument("--head-size", type=int, default=0,
+                    help="run the workload's shape with this head size (64 / 192 / 256) instead of its own; the "
+                         "workload name in the output gets a _d<head> suffix")
     ap.add_argument("--pools", type=int, default=4, help="distinct KV pools the steps rotate over")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-check", action="store_true", help="skip the oracle check of the output")
@@ -61,6 +65,8 @@ def run_prefill(args, torch, L, workloads, dev):
     import numpy as np
 
     cfg = workloads.PREFILL_CONFIGS[args.workload]
+    if args.head_size:
+        cfg = dataclasses.replace(cfg, head_size=args.head_size, name=f"{cfg.name}_d{args.head_size}")
     inp = workloads.make_prefill_inputs(cfg)
     new, history = workloads.draw_prefill_lens(cfg)
     flops = workloads.prefill_flops(cfg, new, history)
@@ -226,6 +232,8 @@ def main():
     args.steps = 400 if args.steps is None else args.steps
     args.warmup = 40 if args.warmup is None else args.warmup
     cfg = workloads.DECODE_CONFIGS[args.workload]
+    if args.head_size:
+        cfg = dataclasses.replace(cfg, head_size=args.head_size, name=f"{cfg.name}_d{args.head_size}")
     inp = workloads.make_decode_inputs(cfg)
     algo_bytes = workloads.decode_algorithmic_bytes(cfg, inp.seq_lens.numpy())
 
@@ -301,7 +309,8 @@ def main():
     gbps_dev = algo_bytes / (us_dev * 1e-6) / 1e9
 
     result = {
-        "metric": "PagedAttn decode achieved HBM GB/s (algorithmic bytes / time per call), 8B-GQA b=32, 1 GPU",
+        "metric": "PagedAttn decode achieved HBM GB/s (algorithmic bytes / time per call), 8B-GQA b=32, 1 GPU"
+                  if cfg.name == "c2_llama3_8b_b32" else f"PagedAttn decode achieved HBM GB/s, {cfg.name}, 1 GPU",
         "value": round(gbps_wall, 1),
         "unit": "GB/s",
         "n_gpus": 1,
@@ -342,10 +351,12 @@ def main():
 
         step(0)
         L.check_error(L.LIBINFINIRT.infinirtStreamSynchronize(stream))
-        want = paged_oracle.paged_attention(inp.q, inp.k_cache, inp.v_cache, inp.block_tables, inp.seq_lens,
-                                            inp.scale, num_threads=min(16, os.cpu_count() or 1))
-        err = (out.float().cpu() - want.float()).abs()
-        ok = bool((err <= 1e-2 + 2e-3 * want.float().abs()).all())
+        # against the oracle's value before its final rounding to the storage dtype: two correctly rounded
+        # results can sit one bf16 step apart, which above |x| = 2.44 is already more than the tolerance
+        _, want = paged_oracle.paged_attention(inp.q, inp.k_cache, inp.v_cache, inp.block_tables, inp.seq_lens,
+                                               inp.scale, num_threads=min(16, os.cpu_count() or 1), return_fp32=True)
+        err = (out.float().cpu() - want).abs()
+        ok = bool((err <= 1e-2 + 2e-3 * want.abs()).all())
         result["parity"] = {"max_abs_err": float(err.max()), "within_atol1e-2_rtol2e-3": ok}
         if not ok:
             print(json.dumps(result))
