@@ -84,6 +84,18 @@ __device__ __forceinline__ int uniformRead(const int *lds_word) {
     return __builtin_amdgcn_readfirstlane(*lds_word);
 }
 
+// Moves a loop-carried value that a load produced into the register of its consumer with an explicit
+// instruction. Written as a plain assignment the move is left to the end of the block, after the
+// load that refills the source has been issued; that load then cannot write the source register,
+// arrives in a temporary, and the copy out of the temporary waits for every load in flight - a full
+// drain of the tile pipeline at every run and segment change.
+__device__ __forceinline__ unsigned handOver(unsigned v) {
+    unsigned r;
+    asm volatile("v_mov_b32 %0, %1" : "=v"(r) : "v"(v));
+    return r;
+}
+__device__ __forceinline__ int handOver(int v) { return static_cast<int>(handOver(static_cast<unsigned>(v))); }
+
 // A run = consecutive tiles of one sequence whose pages fit one page-id register (64 block-table
 // entries, one per lane). All members are wave-uniform.
 struct TileRun {
@@ -101,6 +113,9 @@ __global__ void __launch_bounds__(64) decodeBalancedKernel(DecodeArgs a, int wav
     constexpr int NBUF = G::kBuffers;
     __shared__ uint4 k_lds[kTileTokens * G::kChunksPerRow];
     __shared__ int pre_incl[kBalancedMaxSeqs];
+    // one finished segment's state (accumulators, denominator, maximum), word-major so that lane i
+    // always touches bank i: written and read back by the same lane
+    __shared__ float stash[(4 * G::kCols + 2) * 64];
 
     const int piece = blockIdx.x;
     const int head_chunks = (a.group + kHeadsPerWave - 1) / kHeadsPerWave;
@@ -181,15 +196,15 @@ __global__ void __launch_bounds__(64) decodeBalancedKernel(DecodeArgs a, int wav
         }
         return runAtFlat(s, flat);
     };
+    // Page ids of a run: table entries first_entry .. first_entry + 63, one per lane. The load is
+    // unconditional (lanes past the run's last entry re-read that entry, a run past the end of the
+    // piece re-reads its predecessor's): a predicated load reaches its loop-carried register through a
+    // copy, and that copy waits for every load in flight. Low 32 bits, untouched: the value is
+    // clamped where it is used, so that nothing waits for this load while tiles are in flight.
     auto loadPageIds = [&](const TileRun &r) {
-        int ids = 0;
         const int last_entry = (r.t1 - 1) >> tiles_per_entry_shift;
-        if (r.valid && r.first_entry + lane <= last_entry) {
-            // low 32 bits, untouched: the value is clamped where it is used, so that nothing waits
-            // for this load while tiles are in flight
-            ids = static_cast<int>(loadIndex<Tindex>(a.block_tables, r.seq * a.block_table_batch_stride + r.first_entry + lane));
-        }
-        return ids;
+        const int entry = min(r.first_entry + lane, last_entry);
+        return static_cast<int>(loadIndex<Tindex>(a.block_tables, r.seq * a.block_table_batch_stride + entry));
     };
 
     // ---- load side: runs NBUF-1 tiles ahead of the compute side, across runs and sequences ----
@@ -211,7 +226,7 @@ __global__ void __launch_bounds__(64) decodeBalancedKernel(DecodeArgs a, int wav
         if (real && ++ld_t == ld_run.t1) {
             // next run: its page ids were requested one run ago
             ld_run = ld_next;
-            ld_ids = ld_next_ids;
+            ld_ids = handOver(ld_next_ids);
             ld_t = ld_run.t0;
             ld_next = nextRun(ld_run);
             ld_next_ids = loadPageIds(ld_next);
@@ -224,57 +239,86 @@ __global__ void __launch_bounds__(64) decodeBalancedKernel(DecodeArgs a, int wav
     uint4 q_reg[G::kLoads];
     int c_seq = seq0, c_t = 0, c_t_begin = 0, c_seg_end = 0, c_seq_tiles = 0, c_len = 0;
 
-    auto beginSegment = [&](int s, int flat) {
+    // Query and length of the sequence that follows the current one in this piece, requested when the
+    // current segment begins. A piece that crosses a sequence boundary would otherwise stop at the
+    // boundary for a full memory round trip with no tile requests going out, and such pieces are the
+    // last to finish.
+    uint4 q_next[G::kLoads];
+    int64_t len_next = 0;
+    int next_seq = -1; // -1: the piece ends inside the current sequence
+
+    // (a wavefront whose 16 lanes-heads are not all real reads head 0 for the others: valid memory,
+    // and their columns are never stored - a predicated load would come back through a copy that
+    // waits for every load in flight)
+    auto requestQuery = [&](int s, uint4(&dst)[G::kLoads]) {
+        const S *q_ptr = static_cast<const S *>(a.q) + s * a.q_stride + (head_valid ? head : 0) * a.q_head_stride;
+#pragma unroll
+        for (int kk = 0; kk < G::kLoads; ++kk) {
+            dst[kk] = *reinterpret_cast<const uint4 *>(q_ptr + 32 * kk + 8 * g);
+        }
+    };
+    // ask for the query and length of the sequence after segment [.., flat_end) of sequence s, if the piece reaches it
+    auto requestNext = [&](int s, int flat_end) {
+        next_seq = -1;
+        if (flat_end < f1) {
+            int n = s + 1;
+            while (seqLastTile(n) <= flat_end) { // sequences without tokens
+                ++n;
+            }
+            next_seq = n;
+            len_next = loadIndex<Tindex>(a.seq_lens, n);
+            requestQuery(n, q_next);
+        }
+    };
+
+    auto clampLength = [&](int64_t len64) {
+        return __builtin_amdgcn_readfirstlane(static_cast<int>(len64 < max_len ? len64 : max_len));
+    };
+    // bookkeeping of a new segment: tiles [flat - first, ..) of sequence s, which has `len` tokens
+    auto beginSegment = [&](int s, int flat, int len) {
         const int first = seqFirstTile(s);
         c_seq = s;
         c_seq_tiles = seqLastTile(s) - first;
         c_t_begin = flat - first;
         c_t = c_t_begin;
         c_seg_end = min(c_seq_tiles, f1 - first);
-        if (c_t_begin == 0 && blockIdx.y == 0 && lane == 0) {
-            // tell the merge kernel which pieces hold this sequence (one writer per sequence)
-            a.seq_pieces[s] = make_int2(piece, (first + c_seq_tiles - 1) / q - piece + 1);
-        }
-        const int64_t len64 = loadIndex<Tindex>(a.seq_lens, s);
-        c_len = __builtin_amdgcn_readfirstlane(static_cast<int>(len64 < max_len ? len64 : max_len));
-        const S *q_ptr = static_cast<const S *>(a.q) + s * a.q_stride + (head_valid ? head : 0) * a.q_head_stride;
-#pragma unroll
-        for (int kk = 0; kk < G::kLoads; ++kk) {
-            q_reg[kk] = head_valid ? *reinterpret_cast<const uint4 *>(q_ptr + 32 * kk + 8 * g) : make_uint4(0, 0, 0, 0);
-        }
-        // Use the query here, inside the rarely taken segment switch: the wait for it lands here and
-        // the per-tile code keeps waiting for exactly its own tile, with the others still in flight.
-#pragma unroll
-        for (int kk = 0; kk < G::kLoads; ++kk) {
-            asm volatile("" ::"v"(q_reg[kk].x), "v"(q_reg[kk].y), "v"(q_reg[kk].z), "v"(q_reg[kk].w));
-        }
+        c_len = len;
 #pragma unroll
         for (int e = 0; e < G::kCols; ++e) {
             st.o[e] = f32x4{0.f, 0.f, 0.f, 0.f};
         }
         st.m = -INFINITY;
         st.l = 0.0f;
+        requestNext(s, first + c_seg_end);
+    };
+    // Use the query inside the rarely taken segment switch: the wait for it lands there and the
+    // per-tile code keeps waiting for exactly its own tile, with the others still in flight.
+    auto pinQuery = [&]() {
+#pragma unroll
+        for (int kk = 0; kk < G::kLoads; ++kk) {
+            asm volatile("" ::"v"(q_reg[kk].x), "v"(q_reg[kk].y), "v"(q_reg[kk].z), "v"(q_reg[kk].w));
+        }
     };
 
-    auto endSegment = [&]() {
-        const float l_tot = sumAcrossTokenGroups(st.l);
-        const bool whole = c_t_begin == 0 && c_seg_end == c_seq_tiles;
+    // Stores the result of a finished segment of sequence `seq`: normalised output rows if the segment
+    // covered the whole sequence, else the partial (acc, m, l) rows for the merge kernel.
+    auto writeResult = [&](const TileState<HEAD> &state, float l_tot, int seq, bool whole) {
 #pragma unroll
         for (int rr = 0; rr < 4; ++rr) {
             const int hl = 4 * g + rr;
             const float l_h = __shfl(l_tot, hl, 64);
-            const float m_h = __shfl(st.m, hl, 64);
+            const float m_h = __shfl(state.m, hl, 64);
             const int hg = chunk * kHeadsPerWave + hl;
             if (hg >= a.group) {
                 continue;
             }
             const int out_head = kv_head * a.group + hg;
             if (whole) {
-                S *o_ptr = static_cast<S *>(a.out) + c_seq * a.o_stride + out_head * a.o_head_stride;
-                storeOutputRow<T, HEAD>(o_ptr + G::kCols * c, st, rr, 1.0f / (l_h + 1e-6f));
+                S *o_ptr = static_cast<S *>(a.out) + seq * a.o_stride + out_head * a.o_head_stride;
+                storeOutputRow<T, HEAD>(o_ptr + G::kCols * c, state, rr, 1.0f / (l_h + 1e-6f));
             } else {
-                const int64_t slot = static_cast<int64_t>(piece + c_seq) * a.num_heads + out_head;
-                storePartialRow<HEAD>(a.part_acc + slot * HEAD + G::kCols * c, st, rr);
+                const int64_t slot = static_cast<int64_t>(piece + seq) * a.num_heads + out_head;
+                storePartialRow<HEAD>(a.part_acc + slot * HEAD + G::kCols * c, state, rr);
                 if (c == 0) {
                     a.part_m[slot] = m_h;
                     a.part_l[slot] = l_h;
@@ -283,24 +327,91 @@ __global__ void __launch_bounds__(64) decodeBalancedKernel(DecodeArgs a, int wav
         }
     };
 
+    // A segment that ends in the middle of the piece is not stored at once: stores count as outstanding
+    // memory operations like the tile loads, the waits of the tile loop are fixed counts, and with a
+    // few dozen stores in front of them they would wait for the stores' round trip while no tile
+    // request goes out. Its state is parked in LDS instead and stored when the piece is done (or when
+    // the next segment ends, if the piece holds several).
+    int stash_seq = -1;
+    bool stash_whole = false;
+    auto flushStash = [&]() {
+        TileState<HEAD> parked;
+#pragma unroll
+        for (int e = 0; e < G::kCols; ++e) {
+#pragma unroll
+            for (int rr = 0; rr < 4; ++rr) {
+                parked.o[e][rr] = stash[(4 * e + rr) * 64 + lane];
+            }
+        }
+        const float l_tot = stash[(4 * G::kCols) * 64 + lane];
+        parked.m = stash[(4 * G::kCols + 1) * 64 + lane];
+        parked.l = 0.0f;
+        writeResult(parked, l_tot, stash_seq, stash_whole);
+        stash_seq = -1;
+    };
+    auto parkSegment = [&]() {
+        if (stash_seq >= 0) {
+            flushStash();
+        }
+        const float l_tot = sumAcrossTokenGroups(st.l);
+#pragma unroll
+        for (int e = 0; e < G::kCols; ++e) {
+#pragma unroll
+            for (int rr = 0; rr < 4; ++rr) {
+                stash[(4 * e + rr) * 64 + lane] = st.o[e][rr];
+            }
+        }
+        stash[(4 * G::kCols) * 64 + lane] = l_tot;
+        stash[(4 * G::kCols + 1) * 64 + lane] = st.m;
+        stash_seq = c_seq;
+        stash_whole = c_t_begin == 0 && c_seg_end == c_seq_tiles;
+    };
+
     auto computeNextTile = [&](const TileRegs<HEAD> &r) {
         const int tok0 = c_t * kTileTokens;
         computeTile<T, HEAD>(st, r, q_reg, k_lds, lane, c, g, a.scale_log2, slope, tok0 - (c_len - 1),
                              min(kTileTokens, c_len - tok0));
         if (++c_t == c_seg_end) {
-            PA_STAMP(3);
-            endSegment();
-            const int flat = seqFirstTile(c_seq) + c_seg_end;
-            if (flat < f1) {
-                int s = c_seq + 1;
-                while (seqLastTile(s) <= flat) {
-                    ++s;
+            if (next_seq >= 0) {
+                PA_STAMP(3);
+                // The next sequence's query and length were asked for when this segment began.
+                const int next_len = clampLength(len_next);
+#pragma unroll
+                for (int kk = 0; kk < G::kLoads; ++kk) {
+                    q_reg[kk].x = handOver(q_next[kk].x);
+                    q_reg[kk].y = handOver(q_next[kk].y);
+                    q_reg[kk].z = handOver(q_next[kk].z);
+                    q_reg[kk].w = handOver(q_next[kk].w);
                 }
-                beginSegment(s, flat);
+                __builtin_amdgcn_sched_barrier(0);
+                const int flat = seqFirstTile(c_seq) + c_seg_end;
+                parkSegment();
+                beginSegment(next_seq, flat, next_len);
+                PA_STAMP(5);
             }
         }
     };
 
+    // Tell the merge kernel which pieces hold each sequence that starts in this piece (one writer per
+    // sequence: the wavefront of the first stream whose piece contains the sequence's first tile).
+    // Done before the first tile is requested, for the reason given at parkSegment.
+    if (blockIdx.y == 0) {
+        for (int base = seq0; base < a.num_seqs; base += 64) {
+            const int s = base + lane;
+            bool more = false;
+            if (s < a.num_seqs) {
+                const int first = s == 0 ? 0 : pre_incl[s - 1];
+                const int last = pre_incl[s];
+                more = first < f1;
+                if (last > first && first >= f0 && first < f1) {
+                    a.seq_pieces[s] = make_int2(piece, (last - 1) / q - piece + 1);
+                }
+            }
+            if (__builtin_amdgcn_ballot_w64(more) == 0) {
+                break;
+            }
+        }
+    }
     // The first tiles are requested before the first query: the query's round trip then overlaps
     // with theirs.
     PA_STAMP(2);
@@ -310,7 +421,12 @@ __global__ void __launch_bounds__(64) decodeBalancedKernel(DecodeArgs a, int wav
     for (int i = 0; i < NBUF - 1; ++i) {
         buf[i] = loadNextTile();
     }
-    beginSegment(seq0, f0);
+    {
+        const int64_t len64 = loadIndex<Tindex>(a.seq_lens, seq0);
+        requestQuery(seq0, q_reg);
+        pinQuery();
+        beginSegment(seq0, f0, clampLength(len64));
+    }
     for (int t = 0; t < n_flat; t += NBUF) {
 #pragma unroll
         for (int i = 0; i < NBUF; ++i) {
@@ -319,6 +435,11 @@ __global__ void __launch_bounds__(64) decodeBalancedKernel(DecodeArgs a, int wav
                 computeNextTile(buf[i]);
             }
         }
+    }
+    // the piece's last segment, then the parked one
+    writeResult(st, sumAcrossTokenGroups(st.l), c_seq, c_t_begin == 0 && c_seg_end == c_seq_tiles);
+    if (stash_seq >= 0) {
+        flushStash();
     }
     PA_STAMP(4);
 }
