@@ -248,7 +248,7 @@ def main():
     for _ in range(1, max(1, args.pools)):
         k_pools.append(k_pools[0].clone())
         v_pools.append(v_pools[0].clone())
-    out = torch.zeros_like(q)
+    out = torch.zeros((*q.shape[:-1], v_pools[0].shape[-1]), dtype=q.dtype, device=dev)
 
     # descriptor + workspace, exactly as a caller of the C API does it
     def describe(t):

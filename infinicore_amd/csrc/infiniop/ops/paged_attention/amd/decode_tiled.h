@@ -220,8 +220,85 @@ __device__ __forceinline__ void storePartialRow(float *dst, const TileState<HEAD
     }
 }
 
-// One tile: scores, online softmax, accumulate. `valid` = tokens of the tile that belong to the
-// sequence (16 except possibly in the last tile).
+// Online-softmax step of one tile. s = raw scores of head c for tokens 4g..4g+3 of the tile; rel_pos0 =
+// position of the tile's first token relative to the last token of the sequence (ALiBi distance);
+// `valid` = tokens of the tile that belong to the sequence (16 except possibly in the last tile).
+// Updates the running maximum m, the denominator l and rescales the accumulators o when some head's
+// maximum moved; returns the probabilities as the A operand of P.V.
+//
+// The matrix instruction takes the probabilities in the storage dtype; fp16 keeps 11 significant bits
+// of a value in [0, 1], bf16 only 8. For bf16 the probability is therefore fed as two terms,
+// p = hi + lo with lo = bf16(p - hi), and P.V takes two matrix instructions per output tile: the
+// product then carries ~16 bits of p, close to the fp32 probabilities of the reference kernel. The
+// denominator sums exactly what the numerator used.
+template <typename T, int COLS>
+__device__ __forceinline__ void softmaxStep(f32x4 (&o)[COLS], float &m, float &l, const f32x4 s, int g, float scale_log2,
+                                            float slope, int rel_pos0, int valid, uint2 &p_op, uint2 &p_lo) {
+    const bool tail = valid < kTileTokens;
+    float sc[4];
+#pragma unroll
+    for (int rr = 0; rr < 4; ++rr) {
+        sc[rr] = s[rr] * scale_log2 + slope * static_cast<float>(rel_pos0 + 4 * g + rr);
+        sc[rr] = (tail && 4 * g + rr >= valid) ? -INFINITY : sc[rr];
+    }
+    const float mx = maxAcrossTokenGroups(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])));
+    const float m_new = fmaxf(m, mx);
+
+    if (__builtin_amdgcn_ballot_w64(m_new > m) != 0) {
+        // some head's maximum moved: rescale. Lane holds accumulators of heads 4g..4g+3, whose
+        // factors live in lanes 4g..4g+3.
+        const float alpha = fastExp2(m - m_new);
+        l *= alpha;
+        m = m_new;
+#pragma unroll
+        for (int rr = 0; rr < 4; ++rr) {
+            const float alpha_r = __shfl(alpha, 4 * g + rr, 64);
+#pragma unroll
+            for (int e = 0; e < COLS; ++e) {
+                o[e][rr] *= alpha_r;
+            }
+        }
+    }
+
+    const float p0 = fastExp2(sc[0] - m), p1 = fastExp2(sc[1] - m);
+    const float p2 = fastExp2(sc[2] - m), p3 = fastExp2(sc[3] - m);
+    p_op.x = T::pack2(p0, p1);
+    p_op.y = T::pack2(p2, p3);
+    float p_used = (T::unpackLo(p_op.x) + T::unpackHi(p_op.x)) + (T::unpackLo(p_op.y) + T::unpackHi(p_op.y));
+    if constexpr (T::kSplitProbabilities) {
+        p_lo.x = T::pack2(p0 - T::unpackLo(p_op.x), p1 - T::unpackHi(p_op.x));
+        p_lo.y = T::pack2(p2 - T::unpackLo(p_op.y), p3 - T::unpackHi(p_op.y));
+        p_used += (T::unpackLo(p_lo.x) + T::unpackHi(p_lo.x)) + (T::unpackLo(p_lo.y) + T::unpackHi(p_lo.y));
+    }
+    l += p_used;
+}
+
+// O += P . V for two adjacent output columns: v0..v3 hold those two columns of token rows 4g..4g+3
+// (one dword per row). V rows beyond the sequence may hold anything (NaN included) and 0 * NaN is
+// NaN: they are zeroed.
+template <typename T>
+__device__ __forceinline__ void accumulatePair(f32x4 &o_even, f32x4 &o_odd, uint32_t v0, uint32_t v1, uint32_t v2,
+                                               uint32_t v3, const uint2 p_op, const uint2 p_lo, int g, int valid) {
+    if (valid < kTileTokens) {
+        v0 = (4 * g + 0 >= valid) ? 0u : v0;
+        v1 = (4 * g + 1 >= valid) ? 0u : v1;
+        v2 = (4 * g + 2 >= valid) ? 0u : v2;
+        v3 = (4 * g + 3 >= valid) ? 0u : v3;
+    }
+    uint2 even, odd;
+    even.x = __builtin_amdgcn_perm(v1, v0, 0x05040100u);
+    even.y = __builtin_amdgcn_perm(v3, v2, 0x05040100u);
+    odd.x = __builtin_amdgcn_perm(v1, v0, 0x07060302u);
+    odd.y = __builtin_amdgcn_perm(v3, v2, 0x07060302u);
+    o_even = T::mfmaK16(p_op, even, o_even);
+    o_odd = T::mfmaK16(p_op, odd, o_odd);
+    if constexpr (T::kSplitProbabilities) {
+        o_even = T::mfmaK16(p_lo, even, o_even);
+        o_odd = T::mfmaK16(p_lo, odd, o_odd);
+    }
+}
+
+// One tile: scores, online softmax, accumulate.
 template <typename T, int HEAD>
 __device__ __forceinline__ void computeTile(TileState<HEAD> &st, const TileRegs<HEAD> r,
                                             const uint4 (&q_reg)[TileGeometry<HEAD>::kLoads], uint4 *k_lds, int lane,
@@ -240,74 +317,13 @@ __device__ __forceinline__ void computeTile(TileState<HEAD> &st, const TileRegs<
     }
     __builtin_amdgcn_wave_barrier();
 
-    // scores of head c for tokens 4g + rr of the tile, log2 domain; rel_pos0 = position of the
-    // tile's first token relative to the last token of the sequence (ALiBi distance)
-    const bool tail = valid < kTileTokens;
-    float sc[4];
-#pragma unroll
-    for (int rr = 0; rr < 4; ++rr) {
-        sc[rr] = s[rr] * scale_log2 + slope * static_cast<float>(rel_pos0 + 4 * g + rr);
-        sc[rr] = (tail && 4 * g + rr >= valid) ? -INFINITY : sc[rr];
-    }
-    const float mx = maxAcrossTokenGroups(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])));
-    const float m_new = fmaxf(st.m, mx);
+    uint2 p_op, p_lo = make_uint2(0, 0);
+    softmaxStep<T, G::kCols>(st.o, st.m, st.l, s, g, scale_log2, slope, rel_pos0, valid, p_op, p_lo);
 
-    if (__builtin_amdgcn_ballot_w64(m_new > st.m) != 0) {
-        // some head's maximum moved: rescale. Lane holds accumulators of heads 4g..4g+3, whose
-        // factors live in lanes 4g..4g+3.
-        const float alpha = fastExp2(st.m - m_new);
-        st.l *= alpha;
-        st.m = m_new;
-#pragma unroll
-        for (int rr = 0; rr < 4; ++rr) {
-            const float alpha_r = __shfl(alpha, 4 * g + rr, 64);
-#pragma unroll
-            for (int e = 0; e < G::kCols; ++e) {
-                st.o[e][rr] *= alpha_r;
-            }
-        }
-    }
-
-    // Probabilities as the A operand of P.V. The matrix instruction takes them in the storage dtype;
-    // fp16 keeps 11 significant bits of a value in [0, 1], bf16 only 8. For bf16 the probability is
-    // therefore fed as two terms, p = hi + lo with lo = bf16(p - hi), and P.V takes two matrix
-    // instructions per output tile: the product then carries ~16 bits of p, close to the fp32
-    // probabilities of the reference kernel. The denominator sums exactly what the numerator used.
-    const float p0 = fastExp2(sc[0] - st.m), p1 = fastExp2(sc[1] - st.m);
-    const float p2 = fastExp2(sc[2] - st.m), p3 = fastExp2(sc[3] - st.m);
-    uint2 p_op, p_lo;
-    p_op.x = T::pack2(p0, p1);
-    p_op.y = T::pack2(p2, p3);
-    float p_used = (T::unpackLo(p_op.x) + T::unpackHi(p_op.x)) + (T::unpackLo(p_op.y) + T::unpackHi(p_op.y));
-    if constexpr (T::kSplitProbabilities) {
-        p_lo.x = T::pack2(p0 - T::unpackLo(p_op.x), p1 - T::unpackHi(p_op.x));
-        p_lo.y = T::pack2(p2 - T::unpackLo(p_op.y), p3 - T::unpackHi(p_op.y));
-        p_used += (T::unpackLo(p_lo.x) + T::unpackHi(p_lo.x)) + (T::unpackLo(p_lo.y) + T::unpackHi(p_lo.y));
-    }
-    st.l += p_used;
-
-    // O += P . V, one 16-column output tile per e: column c*kCols + e of rows 4g..4g+3. V rows beyond
-    // the sequence may hold anything (NaN included) and 0 * NaN is NaN: they are zeroed.
+    // one 16-column output tile per e: column c*kCols + e of rows 4g..4g+3
 #pragma unroll
     for (int w = 0; w < G::kWords; ++w) {
-        uint32_t v0 = r.v[0][w], v1 = r.v[1][w], v2 = r.v[2][w], v3 = r.v[3][w];
-        if (tail) {
-            v0 = (4 * g + 0 >= valid) ? 0u : v0;
-            v1 = (4 * g + 1 >= valid) ? 0u : v1;
-            v2 = (4 * g + 2 >= valid) ? 0u : v2;
-            v3 = (4 * g + 3 >= valid) ? 0u : v3;
-        }
-        uint2 even, odd;
-        even.x = __builtin_amdgcn_perm(v1, v0, 0x05040100u);
-        even.y = __builtin_amdgcn_perm(v3, v2, 0x05040100u);
-        odd.x = __builtin_amdgcn_perm(v1, v0, 0x07060302u);
-        odd.y = __builtin_amdgcn_perm(v3, v2, 0x07060302u);
-        st.o[2 * w] = T::mfmaK16(p_op, even, st.o[2 * w]);
-        st.o[2 * w + 1] = T::mfmaK16(p_op, odd, st.o[2 * w + 1]);
-        if constexpr (T::kSplitProbabilities) {
-            st.o[2 * w] = T::mfmaK16(p_lo, even, st.o[2 * w]);
-            st.o[2 * w + 1] = T::mfmaK16(p_lo, odd, st.o[2 * w + 1]);
-        }
+        accumulatePair<T>(st.o[2 * w], st.o[2 * w + 1], r.v[0][w], r.v[1][w], r.v[2][w], r.v[3][w], p_op, p_lo, g, valid);
     }
 }
 

@@ -8,6 +8,7 @@
 #include "../../../devices/amd/amd_device.h"
 #include "decode_common.h"
 #include "decode_generic.h"
+#include "decode_mla.h"
 #include "decode_reduce.h"
 #include "decode_balanced.h"
 #include "decode_tiled.h"
@@ -21,7 +22,7 @@ namespace {
 // Decided once, at descriptor creation, from shapes and the device alone (sequence lengths live in
 // device memory and are never read on the host).
 struct Plan {
-    bool tiled;            // tiled matrix-core kernel (head 64 / 128 / 192 / 256, power-of-two pages >= 16, 16-byte aligned strides)
+    bool tiled;            // tiled matrix-core kernel (head 64 / 128 / 192 / 256 or 576 with values of 512, power-of-two pages >= 16, 16-byte aligned strides)
     bool balanced;         // tiled kernel under the work-equalising schedule (decode_balanced.h)
     int partition_tokens;  // grid schedule: tokens per unit of work
     int max_partitions;    // grid schedule: partitions the longest representable sequence needs
@@ -53,7 +54,8 @@ Plan makePlan(const PagedAttentionInfo &in, const device::amd::DeviceInfo &dev) 
     const bool pow2_page = bs >= 16 && (bs & (bs - 1)) == 0;
 
     const bool tiled_head = in.head_size == 64 || in.head_size == 128 || in.head_size == 192 || in.head_size == 256;
-    plan.tiled = tiled_head && in.value_size == in.head_size && pow2_page
+    const bool latent_head = in.head_size == kMlaKeySize && in.value_size == kMlaValueSize;
+    plan.tiled = ((tiled_head && in.value_size == in.head_size) || latent_head) && pow2_page
               && multipleOf8(in.q_stride) && multipleOf8(in.q_head_stride) && multipleOf8(in.o_stride)
               && multipleOf8(in.o_head_stride) && multipleOf8(in.k_batch_stride) && multipleOf8(in.k_head_stride)
               && multipleOf8(in.k_row_stride) && multipleOf8(in.v_batch_stride) && multipleOf8(in.v_head_stride)
@@ -73,9 +75,12 @@ Plan makePlan(const PagedAttentionInfo &in, const device::amd::DeviceInfo &dev) 
     const long long group = static_cast<long long>(in.num_heads / in.num_kv_heads);
     const long long stream_count = static_cast<long long>(in.num_kv_heads) * ((group + kHeadsPerWave - 1) / kHeadsPerWave);
     const long long units = static_cast<long long>(in.num_seqs) * (plan.tiled ? stream_count : static_cast<long long>(in.num_heads));
-    long long want = units * max_tokens / (16LL * dev.compute_units);
+    // The latent-attention kernel runs one wavefront per SIMD and leaves 32 KiB of partial results per
+    // unit: half as many, twice as long units measured best there.
+    long long want = units * max_tokens / ((latent_head ? 8LL : 16LL) * dev.compute_units);
     int p = floorPow2(want < 1 ? 1 : want);
-    p = p < 64 ? 64 : (p > 512 ? 512 : p);
+    const int p_min = latent_head ? 128 : 64;
+    p = p < p_min ? p_min : (p > 512 ? 512 : p);
     if (const char *env = std::getenv("INFINIOP_AMD_PA_PARTITION")) {
         const int forced = std::atoi(env);
         if (forced >= 16) {
@@ -103,7 +108,7 @@ Plan makePlan(const PagedAttentionInfo &in, const device::amd::DeviceInfo &dev) 
     // with as many wavefronts as fill the device once at one wavefront per SIMD (4 per compute unit,
     // the setting that measured best: every compute unit gets the same number, each wavefront streams
     // as long as possible), each with an equal share of the tiles.
-    plan.balanced = plan.tiled && in.num_seqs <= static_cast<size_t>(kBalancedMaxSeqs);
+    plan.balanced = plan.tiled && !latent_head && in.num_seqs <= static_cast<size_t>(kBalancedMaxSeqs);
     if (const char *env = std::getenv("INFINIOP_AMD_PA_SCHEDULE")) {
         if (std::strcmp(env, "grid") == 0) {
             plan.balanced = false;
@@ -175,7 +180,13 @@ void launchAll(const DecodeArgs &a, const Plan &plan, bool tiled, hipStream_t st
         case 64: launchTiled<T, Tindex, 64>(a, plan, stream); break;
         case 128: launchTiled<T, Tindex, 128>(a, plan, stream); break;
         case 192: launchTiled<T, Tindex, 192>(a, plan, stream); break;
-        default: launchTiled<T, Tindex, 256>(a, plan, stream); break;
+        case 256: launchTiled<T, Tindex, 256>(a, plan, stream); break;
+        default: {
+            const int head_chunks = (a.group + kHeadsPerWave - 1) / kHeadsPerWave;
+            const dim3 grid(plan.max_partitions, a.num_kv_heads * head_chunks, a.num_seqs);
+            decodeMlaKernel<T, Tindex><<<grid, 64, 0, stream>>>(a);
+            break;
+        }
         }
         if (plan.balanced) {
             return; // merged by its own kernel

@@ -29,10 +29,15 @@ class DecodeConfig:
     peaked_fraction: float = 0.0       # fraction of token positions whose K row is scaled
     peaked_scale: float = 8.0
     seed: int = 0
+    value_size: int = 0                # width of a V row; 0 = head_size (latent-attention caches: 576 / 512)
 
     @property
     def scale(self) -> float:
         return 1.0 / float(self.head_size) ** 0.5
+
+    @property
+    def v_size(self) -> int:
+        return self.value_size or self.head_size
 
 
 @dataclass
@@ -76,6 +81,12 @@ DECODE_CONFIGS = {
     "c3_long_context": DecodeConfig("c3_long_context", torch.bfloat16, 8, 32, 8, 128, 16, 16384, 32768,
                                     peaked_fraction=0.01, seed=103),
     "c4_70b_share_b128": DecodeConfig("c4_70b_share_b128", torch.float16, 128, 64, 8, 128, 16, 1024, 8192, seed=104),
+    # latent-attention cache (one KV head, 576-wide keys, 512-wide values): a tensor-parallel share of 16 query
+    # heads, and all 128 heads of the model on one GPU
+    "m1_mla_16_heads_b32": DecodeConfig("m1_mla_16_heads_b32", torch.bfloat16, 32, 16, 1, 576, 16, 512, 4096,
+                                        spare_block_fraction=0.10, seed=106, value_size=512),
+    "m2_mla_128_heads_b32": DecodeConfig("m2_mla_128_heads_b32", torch.bfloat16, 32, 128, 1, 576, 16, 512, 4096,
+                                         spare_block_fraction=0.10, seed=107, value_size=512),
 }
 CACHING_CONFIGS = {
     "c5_prefill_scatter": CachingConfig("c5_prefill_scatter", torch.bfloat16, 4096, 8, 128, 16, 65536, 0.05, seed=105),
@@ -117,8 +128,8 @@ def decode_algorithmic_bytes(cfg: DecodeConfig, seq_lens) -> int:
     entries actually needed (int64) and the lengths."""
     e = 2
     lens = np.asarray(seq_lens, dtype=np.int64)
-    kv = int(lens.sum()) * cfg.num_kv_heads * 2 * cfg.head_size * e
-    qo = 2 * cfg.num_seqs * cfg.num_heads * cfg.head_size * e
+    kv = int(lens.sum()) * cfg.num_kv_heads * (cfg.head_size + cfg.v_size) * e
+    qo = cfg.num_seqs * cfg.num_heads * (cfg.head_size + cfg.v_size) * e
     idx = int(((lens + cfg.block_size - 1) // cfg.block_size).sum()) * 8 + cfg.num_seqs * 8
     return kv + qo + idx
 
@@ -147,7 +158,7 @@ def make_decode_inputs(cfg: DecodeConfig, seed_offset: int = 0) -> DecodeInputs:
         hot = rng.random((num_blocks, 1, cfg.block_size, 1)) < cfg.peaked_fraction
         k_cache = k_cache * torch.from_numpy(np.where(hot, cfg.peaked_scale, 1.0).astype(np.float32))
     k_cache = k_cache.to(cfg.dtype)
-    v_cache = _normal(rng, cache_shape, cfg.dtype)
+    v_cache = _normal(rng, cache_shape[:3] + (cfg.v_size,), cfg.dtype)
     return DecodeInputs(cfg, q, k_cache, v_cache, torch.from_numpy(table), torch.from_numpy(lens), cfg.scale)
 
 

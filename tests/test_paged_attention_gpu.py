@@ -202,6 +202,84 @@ def test_other_head_sizes_ignore_garbage_beyond_the_sequences(gpu_handle, oracle
     assert_close(got, want, f"poison{D}")
 
 
+# ---- latent-attention caches: keys of 576, values of 512 (tiled kernel of its own) -------------------------
+
+def mla(name, dtype, B, H, bs, lo, hi, seed, **kw):
+    return workloads.DecodeConfig(name, dtype, B, H, 1, 576, bs, lo, hi, seed=seed, value_size=512, **kw)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("H", [16, 128, 20])
+def test_mla_ragged_batches(gpu_handle, oracle, dtype, H):
+    """Ragged lengths incl. 1 token and exactly one page, long enough that sequences are split into
+    partitions and merged; 16 heads (one wavefront per unit), 128 (eight) and 20 (a partly filled one)."""
+    inp = workloads.make_decode_inputs(mla(f"mla_h{H}", dtype, 5, H, 16, 1, 2500, seed=400 + H))
+    inp.seq_lens[0], inp.seq_lens[1] = 1, 16
+    got, _ = run_case(gpu_handle, oracle, inp)
+    assert got.shape == (5, H, 512)
+
+
+@pytest.mark.parametrize("partition", [16, 48, 1024])
+def test_mla_partition_sizes(gpu_handle, oracle, monkeypatch, partition):
+    monkeypatch.setenv("INFINIOP_AMD_PA_PARTITION", str(partition))
+    run_case(gpu_handle, oracle, workloads.make_decode_inputs(mla(f"mla_p{partition}", torch.bfloat16, 3, 16, 16, 1, 1200, seed=410)))
+
+
+def test_mla_matches_the_elementwise_kernel_in_layout(gpu_handle):
+    """Every output column lands where the element-wise kernel puts it: V with a distinct constant per
+    column makes the expected output that constant, whatever the softmax does. Short sequences (written by the
+    decode kernel) and long ones (merged from partitions)."""
+    inp = workloads.make_decode_inputs(mla("mla_cols", torch.float16, 4, 16, 16, 40, 1500, seed=420))
+    inp.seq_lens[0] = 33
+    ramp = (torch.arange(512, dtype=torch.float32) - 256) / 16
+    inp.v_cache[:] = ramp.to(torch.float16)
+    got = run_paged_attention(gpu_handle, *to_device(inp), inp.scale).float().cpu()
+    want = ramp.to(torch.float16).float().expand_as(got)
+    assert torch.allclose(got, want, atol=2e-3 * float(ramp.abs().max()), rtol=0), (got - want).abs().max()
+
+
+def test_mla_alibi_pages_of_64_and_int32_indices(gpu_handle, oracle):
+    inp = workloads.make_decode_inputs(mla("mla_mix", torch.bfloat16, 4, 32, 64, 1, 1500, seed=430))
+    slopes = torch.tensor([2.0 ** (-(i % 8 + 1)) for i in range(32)], dtype=torch.float32)
+    q, k, v, bt, sl = to_device(inp)
+    got = run_paged_attention(gpu_handle, q, k, v, bt.to(torch.int32), sl.to(torch.int32), inp.scale, alibi=slopes.to(DEV))
+    want, want_f32 = oracle_of(oracle, inp, alibi_slopes=slopes, return_fp32=True)
+    assert_close(got, want, "mla_mix", want_f32)
+
+
+def test_mla_ignores_garbage_beyond_the_sequences(gpu_handle, oracle):
+    inp = workloads.make_decode_inputs(mla("mla_poison", torch.float16, 4, 16, 16, 1, 600, seed=440))
+    want = oracle_of(oracle, inp)
+    k, v = inp.k_cache.clone(), inp.v_cache.clone()
+    for s in range(4):
+        n = int(inp.seq_lens[s])
+        if n % 16:
+            page = inp.block_tables[s, (n - 1) // 16]
+            k[page, :, n % 16:, :] = float("nan")
+            v[page, :, n % 16:, :] = float("nan")
+    got = run_paged_attention(gpu_handle, inp.q.to(DEV), k.to(DEV), v.to(DEV), inp.block_tables.to(DEV),
+                              inp.seq_lens.to(DEV), inp.scale)
+    assert_close(got, want, "mla_poison")
+
+
+def test_mla_padded_cache_rows(gpu_handle, oracle):
+    """K and V rows that are not packed (views into wider pools): row strides of 640 and 576 elements."""
+    inp = workloads.make_decode_inputs(mla("mla_strided", torch.bfloat16, 3, 16, 16, 1, 900, seed=450))
+    nb = inp.k_cache.shape[0]
+    k_pool = torch.full((nb, 1, 16, 640), float("nan"), dtype=torch.bfloat16)
+    v_pool = torch.full((nb, 1, 16, 576), float("nan"), dtype=torch.bfloat16)
+    k_pool[..., :576] = inp.k_cache
+    v_pool[..., :512] = inp.v_cache
+    got = run_paged_attention(gpu_handle, inp.q.to(DEV), k_pool.to(DEV)[..., :576], v_pool.to(DEV)[..., :512],
+                              inp.block_tables.to(DEV), inp.seq_lens.to(DEV), inp.scale)
+    want, want_f32 = oracle_of(oracle, inp, return_fp32=True)
+    assert_close(got, want, "mla_strided", want_f32)
+
+
+def test_mla_full_size_against_oracle(gpu_handle, oracle):
+    run_case(gpu_handle, oracle, workloads.make_decode_inputs(workloads.DECODE_CONFIGS["m1_mla_16_heads_b32"]))
+
+
 # ---- every kernel and schedule against the same oracle ---------------------------------------------
 
 @pytest.mark.parametrize("kernel,schedule", [("generic", None), (None, "grid"), (None, None)])
