@@ -326,7 +326,7 @@ def main():
         "config": {
             "workload": cfg.name,
             "num_seqs": cfg.num_seqs, "num_heads": cfg.num_heads, "num_kv_heads": cfg.num_kv_heads,
-            "head_size": cfg.head_size, "block_size": cfg.block_size,
+            "head_size": cfg.head_size, "value_size": cfg.v_size, "block_size": cfg.block_size,
             "seq_lens": f"uniform[{cfg.min_len},{cfg.max_len}] sum={int(inp.seq_lens.sum())}",
             "kv_pools_rotated": len(k_pools),
             "algorithmic_bytes_per_call": algo_bytes,

@@ -392,11 +392,14 @@ __global__ void __launch_bounds__(64) decodeTiledKernel(DecodeArgs a) {
     using G = TileGeometry<HEAD>;
     __shared__ uint4 k_lds[kTileTokens * G::kChunksPerRow]; // one K tile
 
-    const int part = blockIdx.x;
     const int head_chunks = (a.group + kHeadsPerWave - 1) / kHeadsPerWave;
     const int kv_head = blockIdx.y / head_chunks;
     const int chunk = blockIdx.y - kv_head * head_chunks;
     const int seq = blockIdx.z;
+    // Workgroups are dealt to the eight XCDs round-robin by linear index, which follows blockIdx.x when the
+    // grid's x extent is a multiple of eight. Partition p of every sequence on the same XCD would load the
+    // XCDs by how many sequences reach partition p, so the partitions of sequence s are rotated by s.
+    const int part = static_cast<int>((blockIdx.x + blockIdx.z) % gridDim.x);
     const int lane = threadIdx.x;
     const int c = lane & 15; // column strip / head within the chunk / token for the K operand
     const int g = lane >> 4; // group of four tokens

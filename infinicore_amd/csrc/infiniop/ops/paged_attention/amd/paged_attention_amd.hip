@@ -8,10 +8,10 @@
 #include "../../../devices/amd/amd_device.h"
 #include "decode_common.h"
 #include "decode_generic.h"
-#include "decode_mla.h"
 #include "decode_reduce.h"
 #include "decode_balanced.h"
 #include "decode_tiled.h"
+#include "decode_mla.h" // after decode_balanced.h: shares its diagnostic timestamp buffer
 #include <cstdlib>
 #include <cstring>
 
@@ -75,11 +75,12 @@ Plan makePlan(const PagedAttentionInfo &in, const device::amd::DeviceInfo &dev) 
     const long long group = static_cast<long long>(in.num_heads / in.num_kv_heads);
     const long long stream_count = static_cast<long long>(in.num_kv_heads) * ((group + kHeadsPerWave - 1) / kHeadsPerWave);
     const long long units = static_cast<long long>(in.num_seqs) * (plan.tiled ? stream_count : static_cast<long long>(in.num_heads));
-    // The latent-attention kernel runs one wavefront per SIMD and leaves 32 KiB of partial results per
-    // unit: half as many, twice as long units measured best there.
-    long long want = units * max_tokens / ((latent_head ? 8LL : 16LL) * dev.compute_units);
+    // A unit of the latent-attention kernel leaves 32 KiB of partial results and advances one tile per
+    // memory latency however many units there are: fewer, longer units measured best there.
+    long long want = latent_head ? units * max_tokens * 3 / (16LL * dev.compute_units)
+                                 : units * max_tokens / (16LL * dev.compute_units);
     int p = floorPow2(want < 1 ? 1 : want);
-    const int p_min = latent_head ? 128 : 64;
+    const int p_min = latent_head ? 256 : 64;
     p = p < p_min ? p_min : (p > 512 ? 512 : p);
     if (const char *env = std::getenv("INFINIOP_AMD_PA_PARTITION")) {
         const int forced = std::atoi(env);
@@ -184,7 +185,7 @@ void launchAll(const DecodeArgs &a, const Plan &plan, bool tiled, hipStream_t st
         default: {
             const int head_chunks = (a.group + kHeadsPerWave - 1) / kHeadsPerWave;
             const dim3 grid(plan.max_partitions, a.num_kv_heads * head_chunks, a.num_seqs);
-            decodeMlaKernel<T, Tindex><<<grid, 64, 0, stream>>>(a);
+            decodeMlaKernel<T, Tindex><<<grid, kMlaThreads, 0, stream>>>(a);
             break;
         }
         }
