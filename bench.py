@@ -60,6 +60,17 @@ def parse_args():
     return ap.parse_args()
 
 
+def pmc_calibration_copies(torch, dev):
+    """Three plain 256 MiB device-to-device copies: a kernel of known traffic that gives hardware byte
+    counters their scale when the same run is collected with rocprofv3 --pmc."""
+    src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(3)
+    dst = torch.empty_like(src)
+    for _ in range(3):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+    del src, dst
+
+
 def run_prefill(args, torch, L, workloads, dev):
     """One step = one infiniopPagedAttentionPrefill call; inputs resident in HBM."""
     import numpy as np
@@ -100,6 +111,8 @@ def run_prefill(args, torch, L, workloads, dev):
             c_void_p(k_cache.data_ptr()), c_void_p(v_cache.data_ptr()), c_void_p(bt.data_ptr()), c_void_p(sl.data_ptr()),
             c_void_p(cu.data_ptr()), c_void_p(0), stream))
 
+    if args.pmc_calibration:
+        pmc_calibration_copies(torch, dev)
     torch.cuda.synchronize()
     for _ in range(args.warmup):
         step()
@@ -210,6 +223,124 @@ def run_prefill(args, torch, L, workloads, dev):
     L.destroy_handle(handle)
 
 
+def run_caching(args, torch, L, workloads, dev):
+    """One step = one infiniopPagedCaching call (scatter of a chunk of new K/V rows into the pools);
+    inputs resident in HBM, several source / pool sets rotated so that the rows are not served from cache."""
+    cfg = workloads.CACHING_CONFIGS[args.workload]
+    inp = workloads.make_caching_inputs(cfg)
+    algo_bytes = workloads.caching_algorithmic_bytes(cfg, inp.slot_mapping.numpy())
+
+    L.set_device(L.InfiniDevice.AMD, 0)
+    handle = L.create_handle()
+    slots = inp.slot_mapping.to(dev)
+    sets = []
+    for _ in range(max(1, args.pools)):
+        sets.append((inp.k_cache.to(dev), inp.v_cache.to(dev), inp.k.to(dev), inp.v.to(dev)))
+    DTYPES = {torch.float16: L.InfiniDtype.F16, torch.bfloat16: L.InfiniDtype.BF16, torch.int64: L.InfiniDtype.I64}
+    descs = [L.create_tensor_descriptor(tuple(t.shape), tuple(t.stride()), DTYPES[t.dtype]) for t in (*sets[0], slots)]
+    op = L.infiniopOperatorDescriptor_t()
+    L.check_error(L.LIBINFINIOP.infiniopCreatePagedCachingDescriptor(handle, ctypes.byref(op), *descs))
+    for d in descs:
+        L.destroy_tensor_descriptor(d)
+    ws_size = c_size_t(0)
+    L.check_error(L.LIBINFINIOP.infiniopGetPagedCachingWorkspaceSize(op, ctypes.byref(ws_size)))
+
+    stream = c_void_p()
+    L.check_error(L.LIBINFINIRT.infinirtStreamCreate(ctypes.byref(stream)))
+    ev0, ev1 = c_void_p(), c_void_p()
+    L.check_error(L.LIBINFINIRT.infinirtEventCreate(ctypes.byref(ev0)))
+    L.check_error(L.LIBINFINIRT.infinirtEventCreate(ctypes.byref(ev1)))
+
+    def step(i):
+        kc, vc, k, v = sets[i % len(sets)]
+        L.check_error(L.LIBINFINIOP.infiniopPagedCaching(
+            op, c_void_p(0), 0, c_void_p(kc.data_ptr()), c_void_p(vc.data_ptr()), c_void_p(k.data_ptr()),
+            c_void_p(v.data_ptr()), c_void_p(slots.data_ptr()), stream))
+
+    if args.pmc_calibration:
+        pmc_calibration_copies(torch, dev)
+    torch.cuda.synchronize()
+    for i in range(args.warmup):
+        step(i)
+    L.check_error(L.LIBINFINIRT.infinirtStreamSynchronize(stream))
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    L.check_error(L.LIBINFINIRT.infinirtEventRecord(ev0, stream))
+    for i in range(args.steps):
+        step(i)
+    L.check_error(L.LIBINFINIRT.infinirtEventRecord(ev1, stream))
+    L.check_error(L.LIBINFINIRT.infinirtStreamSynchronize(stream))
+    torch.cuda.synchronize()
+    wall_s = time.perf_counter() - t0
+    ms = c_float(0)
+    L.check_error(L.LIBINFINIRT.infinirtEventElapsedTime(ctypes.byref(ms), ev0, ev1))
+    us_wall = wall_s / args.steps * 1e6
+    us_dev = ms.value / args.steps * 1e3
+    valid = int((inp.slot_mapping >= 0).sum())
+
+    result = {
+        "metric": "paged_caching scatter achieved HBM GB/s (rows read + rows written + slot ids / time per call), 1 GPU",
+        "value": round(algo_bytes / (us_wall * 1e-6) / 1e9, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(us_wall / 1e3, 6),
+        "us_per_call": round(us_wall, 2),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "u8",
+        "data": "synthetic",
+        "config": {
+            "workload": cfg.name, "num_tokens": cfg.num_tokens, "valid_tokens": valid, "num_kv_heads": cfg.num_kv_heads,
+            "head_size": cfg.head_size, "block_size": cfg.block_size, "num_slots": cfg.num_slots,
+            "sets_rotated": len(sets), "algorithmic_bytes_per_call": algo_bytes,
+        },
+        "roofline": {
+            "bound": "hbm",
+            "achieved": round(algo_bytes / (us_dev * 1e-6) / 1e9, 1),
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": round(algo_bytes / (us_dev * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
+            "traffic": None,
+            "us_per_call_device": round(us_dev, 2),
+            "note": "achieved = algorithmic bytes / device time per call (events on the kernel's stream, back-to-back "
+                    "launches); a call moves 32 MB, which at 8 TB/s is 4 us: the size of a kernel launch",
+        },
+    }
+
+    from oracle import paged_oracle
+
+    if not args.no_check:
+        kc, vc, k, v = sets[0]
+        want_k, want_v = paged_oracle.paged_caching(inp.k_cache.clone(), inp.v_cache.clone(), inp.k, inp.v, inp.slot_mapping)
+        ok = bool(torch.equal(kc.cpu().view(torch.int16), want_k.view(torch.int16))
+                  and torch.equal(vc.cpu().view(torch.int16), want_v.view(torch.int16)))
+        result["parity"] = {"bit_exact": ok}
+        if not ok:
+            print(json.dumps(result))
+            print("bench.py: pools differ from the oracle's", file=sys.stderr)
+            sys.exit(4)
+    if not args.no_cpu_baseline:
+        kc, vc = inp.k_cache.clone(), inp.v_cache.clone()
+        reps, t0 = 0, time.perf_counter()
+        while reps < 2000 and time.perf_counter() - t0 < 10.0:
+            paged_oracle.paged_caching(kc, vc, inp.k, inp.v, inp.slot_mapping)
+            reps += 1
+        cpu_s = (time.perf_counter() - t0) / reps
+        result["cpu_baseline"] = {
+            "value": round(algo_bytes / cpu_s / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"{reps} full calls of the same workload through the C oracle (one thread), {cpu_s * 1e6:.0f} us per call",
+        }
+    print(json.dumps(result))
+    L.check_error(L.LIBINFINIOP.infiniopDestroyPagedCachingDescriptor(op))
+    L.check_error(L.LIBINFINIRT.infinirtEventDestroy(ev0))
+    L.check_error(L.LIBINFINIRT.infinirtEventDestroy(ev1))
+    L.check_error(L.LIBINFINIRT.infinirtStreamDestroy(stream))
+    L.destroy_handle(handle)
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -225,6 +356,10 @@ def main():
         print("bench.py: no GPU visible; the HIP path has no CPU fallback", file=sys.stderr)
         sys.exit(3)
     dev = torch.device("cuda:0")
+    if args.workload in workloads.CACHING_CONFIGS:
+        args.steps = 400 if args.steps is None else args.steps
+        args.warmup = 40 if args.warmup is None else args.warmup
+        return run_caching(args, torch, L, workloads, dev)
     if args.workload in workloads.PREFILL_CONFIGS:
         args.steps = 50 if args.steps is None else args.steps
         args.warmup = 5 if args.warmup is None else args.warmup
@@ -279,12 +414,7 @@ def main():
             c_void_p(sl.data_ptr()), c_void_p(0), stream))
 
     if args.pmc_calibration:
-        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(3)
-        dst = torch.empty_like(src)
-        for _ in range(3):
-            dst.copy_(src)
-        torch.cuda.synchronize()
-        del src, dst
+        pmc_calibration_copies(torch, dev)
 
     torch.cuda.synchronize()
     for i in range(args.warmup):
