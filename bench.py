@@ -35,11 +35,15 @@ sys.path.insert(0, str(ROOT))
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E
 MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 / fp16 matrix peak
 
-# HBM bytes per launch of the decode kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
-# file, each scaled by what the same counter reads for a 256 MiB copy (summary and commands:
-# profiles/decode_balanced_c2_llama3_8b_b32_hbm_traffic.md). Counters cannot be read from inside this
-# process, so the figure is recorded here; it belongs to the default workload only.
-MEASURED_TRAFFIC_BYTES = {"c2_llama3_8b_b32": 322_300_000}
+# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
+# file, each scaled by what the same counter reads for a 256 MiB copy (summaries and commands: profiles/).
+# Counters cannot be read from inside this process, so the figures are recorded here, per workload.
+MEASURED_TRAFFIC_BYTES = {
+    "c2_llama3_8b_b32": 322_400_000,       # decodeBalancedKernel: 319.8 MB fetched + 2.6 MB written
+    "m1_mla_16_heads_b32": 146_500_000,    # decodeMlaKernel: 137.9 MB fetched + 8.6 MB written
+    "c5_prefill_scatter": 32_100_000,      # pagedCachingScatterKernel: 16.2 MB fetched + 15.9 MB written
+    "p3_llama3_8b_chunked": 451_500_000,   # prefillTiledKernel: fetched (writes: the 44 MB output)
+}
 
 
 def parse_args():
@@ -163,7 +167,7 @@ def run_prefill(args, torch, L, workloads, dev):
             "peak": MFMA_PEAK_TFLOPS,
             "unit": "TFLOP/s",
             "frac": round(tflops_dev / MFMA_PEAK_TFLOPS, 4),
-            "traffic": None,
+            "traffic": MEASURED_TRAFFIC_BYTES.get(cfg.name),
             "us_per_call_device": round(us_dev, 2),
             "note": "achieved = flops per call / device time per call (events on the kernel's stream); one kernel per call",
         },
@@ -303,7 +307,7 @@ def run_caching(args, torch, L, workloads, dev):
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": round(algo_bytes / (us_dev * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
-            "traffic": None,
+            "traffic": MEASURED_TRAFFIC_BYTES.get(cfg.name),
             "us_per_call_device": round(us_dev, 2),
             "note": "achieved = algorithmic bytes / device time per call (events on the kernel's stream, back-to-back "
                     "launches); a call moves 32 MB, which at 8 TB/s is 4 us: the size of a kernel launch",
