@@ -135,19 +135,53 @@ __global__ void __launch_bounds__(64) decodeBalancedKernel(DecodeArgs a, int wav
 #endif
     const int total_tiles = tilePrefixSums<Tindex>(a, lane, pre_incl);
     PA_STAMP(1);
-    const int q = tilesPerPiece(total_tiles, waves_per_stream);
-    const int f0 = piece * q;
-    const int f1 = min(total_tiles, f0 + q);
+    // The flat range is not cut into equal tile counts but into equal COST: a sequence that begins inside
+    // a piece costs its wavefront about as much time as kStartCost more tiles would (measured: pieces with
+    // such a start finish level with the others when they hold three to four tiles fewer at head 128), and they were
+    // the last to finish. On a virtual axis every sequence is preceded by kStartCost empty slots; pieces are
+    // equal ranges of that axis, and a piece's tiles are the real tiles its range covers: tile i of
+    // sequence s sits at virtual position (tiles before s) + i + kStartCost * (s + 1).
+    constexpr int kStartCost = HEAD <= 128 ? 384 / HEAD : 2;
+    const int q = tilesPerPiece(total_tiles + kStartCost * a.num_seqs, waves_per_stream);
+    // Real tiles below virtual positions x0 = piece * q and x1 = x0 + q: count the sequences that lie
+    // entirely below each (one pass over the prefix sums for both), then add the part of the next one.
+    const int x0 = piece * q, x1 = x0 + q;
+    int s0 = 0, s1 = 0;
+    int first_64 = 0; // prefix sum of sequence `lane`: the first 64 are kept in a register as well
+    for (int base = 0; base < a.num_seqs; base += 64) {
+        const int b = base + lane;
+        const int mine = b < a.num_seqs ? pre_incl[b] : 0x3fffffff;
+        first_64 = base == 0 ? mine : first_64;
+        const int seq_end = mine + kStartCost * (b + 1);
+        s0 += __popcll(__builtin_amdgcn_ballot_w64(seq_end <= x0));
+        s1 += __popcll(__builtin_amdgcn_ballot_w64(seq_end <= x1));
+    }
+    s0 = __builtin_amdgcn_readfirstlane(s0);
+    s1 = __builtin_amdgcn_readfirstlane(s1);
+    // prefix sum of sequence s (wave-uniform s): a lane read for the first 64 sequences, which costs a few
+    // clocks where the LDS round trip costs a hundred, and these reads are chained at every piece start
+    // and segment switch
+    auto prefixAt = [&](int s) {
+        return s < 64 ? __builtin_amdgcn_readlane(first_64, s) : uniformRead(&pre_incl[s]);
+    };
+    auto tilesBelow = [&](int x, int s) {
+        if (s >= a.num_seqs) {
+            return total_tiles;
+        }
+        const int first = s == 0 ? 0 : prefixAt(s - 1);
+        const int inside = x - (first + kStartCost * s) - kStartCost; // tiles of sequence s below x
+        return first + max(0, min(inside, prefixAt(s) - first));
+    };
+    const int f0 = tilesBelow(x0, s0);
+    const int f1 = tilesBelow(x1, s1);
     if (f0 >= f1) {
         return;
     }
-    // first sequence whose tiles reach past f0
-    int seq0 = 0;
-    for (int base = 0; base < a.num_seqs; base += 64) {
-        const int b = base + lane;
-        seq0 += __popcll(__builtin_amdgcn_ballot_w64(b < a.num_seqs && pre_incl[b] <= f0));
+    // first sequence whose tiles reach past f0: s0, or a later one if s0 has no tile at or after f0
+    int seq0 = s0;
+    while (prefixAt(seq0) <= f0) {
+        ++seq0;
     }
-    seq0 = __builtin_amdgcn_readfirstlane(seq0);
 
     const int64_t max_len = static_cast<int64_t>(a.max_blocks_per_seq) << a.block_shift;
     const int head_in_group = chunk * kHeadsPerWave + c;
@@ -162,8 +196,8 @@ __global__ void __launch_bounds__(64) decodeBalancedKernel(DecodeArgs a, int wav
                                 static_cast<uint32_t>(a.v_row_stride) * sizeof(S));
 
     // ---- wave-uniform walk over the piece: sequences -> segments -> runs ----
-    auto seqFirstTile = [&](int s) { return s == 0 ? 0 : uniformRead(&pre_incl[s - 1]); };
-    auto seqLastTile = [&](int s) { return uniformRead(&pre_incl[s]); };
+    auto seqFirstTile = [&](int s) { return s == 0 ? 0 : prefixAt(s - 1); };
+    auto seqLastTile = [&](int s) { return prefixAt(s); };
     auto makeRun = [&](int s, int t0, int seg_end) {
         TileRun r;
         r.seq = s;
@@ -404,7 +438,7 @@ __global__ void __launch_bounds__(64) decodeBalancedKernel(DecodeArgs a, int wav
                 const int last = pre_incl[s];
                 more = first < f1;
                 if (last > first && first >= f0 && first < f1) {
-                    a.seq_pieces[s] = make_int2(piece, (last - 1) / q - piece + 1);
+                    a.seq_pieces[s] = make_int2(piece, (last - 1 + kStartCost * (s + 1)) / q - piece + 1);
                 }
             }
             if (__builtin_amdgcn_ballot_w64(more) == 0) {
