@@ -40,6 +40,19 @@ __device__ unsigned long long *g_pa_trace = nullptr;
 constexpr int kBalancedMaxSeqs = 1024; // prefix sums of the batch live in LDS
 constexpr int kBalancedMinTiles = 4;   // never cut pieces finer than 64 tokens
 
+// Inclusive prefix sum over the 64 lanes with data-parallel-primitive moves (no LDS-unit permutes: this
+// runs at the head of every wavefront, before its first memory request can go out). Rows of 16 lanes are
+// scanned with row shifts, then lane 15 of rows 0 and 2 is added to the next row, then lane 31 to rows 2, 3.
+__device__ __forceinline__ int waveInclusiveSum(int x) {
+    x += __builtin_amdgcn_update_dpp(0, x, 0x111, 0xf, 0xf, false); // row_shr:1
+    x += __builtin_amdgcn_update_dpp(0, x, 0x112, 0xf, 0xf, false); // row_shr:2
+    x += __builtin_amdgcn_update_dpp(0, x, 0x114, 0xf, 0xf, false); // row_shr:4
+    x += __builtin_amdgcn_update_dpp(0, x, 0x118, 0xf, 0xf, false); // row_shr:8
+    x += __builtin_amdgcn_update_dpp(0, x, 0x142, 0xa, 0xf, false); // row_bcast:15 into rows 1 and 3
+    x += __builtin_amdgcn_update_dpp(0, x, 0x143, 0xc, 0xf, false); // row_bcast:31 into rows 2 and 3
+    return x;
+}
+
 // Inclusive prefix sums of the per-sequence tile counts into LDS; returns the total. Executed by
 // one wavefront (lanes 0..63 of the caller).
 template <typename Tindex>
@@ -54,16 +67,11 @@ __device__ __forceinline__ int tilePrefixSums(const DecodeArgs &a, int lane, int
             len = len < max_len ? len : max_len;
             x = len > 0 ? static_cast<int>((len + kTileTokens - 1) / kTileTokens) : 0;
         }
-#pragma unroll
-        for (int off = 1; off < 64; off <<= 1) {
-            const int y = __shfl_up(x, off, 64);
-            x += lane >= off ? y : 0;
-        }
-        x += running;
+        x = waveInclusiveSum(x) + running;
         if (b < a.num_seqs) {
             pre_incl[b] = x;
         }
-        running = __shfl(x, 63, 64);
+        running = __builtin_amdgcn_readlane(x, 63);
     }
     __builtin_amdgcn_wave_barrier();
     // every lane holds the same total; say so, or all index arithmetic derived from it is
