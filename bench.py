@@ -42,6 +42,7 @@ MEASURED_TRAFFIC_BYTES = {
     "c2_llama3_8b_b32": 322_400_000,       # decodeBalancedKernel: 319.8 MB fetched + 2.6 MB written
     "m1_mla_16_heads_b32": 146_500_000,    # decodeMlaKernel: 137.9 MB fetched + 8.6 MB written
     "c5_prefill_scatter": 32_100_000,      # pagedCachingScatterKernel: 16.2 MB fetched + 15.9 MB written
+    "k2_append_prefill_chunk": 33_600_000, # kvCachingAppendKernel: 16.8 MB fetched + 16.8 MB written
     "p3_llama3_8b_chunked": 451_500_000,   # prefillTiledKernel: fetched (writes: the 44 MB output)
 }
 
@@ -228,26 +229,52 @@ def run_prefill(args, torch, L, workloads, dev):
 
 
 def run_caching(args, torch, L, workloads, dev):
-    """One step = one infiniopPagedCaching call (scatter of a chunk of new K/V rows into the pools);
-    inputs resident in HBM, several source / pool sets rotated so that the rows are not served from cache."""
-    cfg = workloads.CACHING_CONFIGS[args.workload]
-    inp = workloads.make_caching_inputs(cfg)
-    algo_bytes = workloads.caching_algorithmic_bytes(cfg, inp.slot_mapping.numpy())
+    """One step = one infiniopPagedCaching call (scatter of a chunk of new K/V rows into the paged pools) or one
+    infiniopKVCaching call (append to contiguous caches); inputs resident in HBM, several source / cache sets
+    rotated so that the rows are not served from cache."""
+    def oracle_fn(*operands):  # the checker and the CPU baseline; never on the timed path
+        from oracle import paged_oracle
+
+        return (paged_oracle.paged_caching if paged else paged_oracle.kv_caching)(*operands)
+
+    paged = args.workload in workloads.CACHING_CONFIGS
+    if paged:
+        cfg = workloads.CACHING_CONFIGS[args.workload]
+        inp = workloads.make_caching_inputs(cfg)
+        index = inp.slot_mapping
+        algo_bytes = workloads.caching_algorithmic_bytes(cfg, index.numpy())
+        create, size_of = L.LIBINFINIOP.infiniopCreatePagedCachingDescriptor, L.LIBINFINIOP.infiniopGetPagedCachingWorkspaceSize
+        call, destroy = L.LIBINFINIOP.infiniopPagedCaching, L.LIBINFINIOP.infiniopDestroyPagedCachingDescriptor
+        metric = "paged_caching scatter achieved HBM GB/s (rows read + rows written + slot ids / time per call), 1 GPU"
+        config = {"workload": cfg.name, "num_tokens": cfg.num_tokens, "valid_tokens": int((index >= 0).sum()),
+                  "num_kv_heads": cfg.num_kv_heads, "head_size": cfg.head_size, "block_size": cfg.block_size,
+                  "num_slots": cfg.num_slots}
+    else:
+        cfg = workloads.KV_CACHING_CONFIGS[args.workload]
+        inp = workloads.make_kv_caching_inputs(cfg)
+        index = inp.past_kv_lengths
+        algo_bytes = workloads.kv_caching_algorithmic_bytes(cfg)
+        create, size_of = L.LIBINFINIOP.infiniopCreateKVCachingDescriptor, L.LIBINFINIOP.infiniopGetKVCachingWorkspaceSize
+        call, destroy = L.LIBINFINIOP.infiniopKVCaching, L.LIBINFINIOP.infiniopDestroyKVCachingDescriptor
+        metric = "kv_caching append achieved HBM GB/s (rows read + rows written + lengths / time per call), 1 GPU"
+        config = {"workload": cfg.name, "batch": cfg.batch, "num_kv_heads": cfg.num_kv_heads, "max_seq_len": cfg.max_seq_len,
+                  "new_tokens_per_sequence": cfg.new_tokens, "head_size": cfg.head_size}
 
     L.set_device(L.InfiniDevice.AMD, 0)
     handle = L.create_handle()
-    slots = inp.slot_mapping.to(dev)
-    sets = []
-    for _ in range(max(1, args.pools)):
-        sets.append((inp.k_cache.to(dev), inp.v_cache.to(dev), inp.k.to(dev), inp.v.to(dev)))
+    index_dev = index.to(dev)
+    # bound the rotation by memory: a set of the append workload's caches is 2 GiB
+    set_bytes = 2 * inp.k_cache.numel() * inp.k_cache.element_size()
+    n_sets = max(1, min(args.pools, (8 << 30) // max(set_bytes, 1)))
+    sets = [(inp.k_cache.to(dev), inp.v_cache.to(dev), inp.k.to(dev), inp.v.to(dev)) for _ in range(n_sets)]
     DTYPES = {torch.float16: L.InfiniDtype.F16, torch.bfloat16: L.InfiniDtype.BF16, torch.int64: L.InfiniDtype.I64}
-    descs = [L.create_tensor_descriptor(tuple(t.shape), tuple(t.stride()), DTYPES[t.dtype]) for t in (*sets[0], slots)]
+    descs = [L.create_tensor_descriptor(tuple(t.shape), tuple(t.stride()), DTYPES[t.dtype]) for t in (*sets[0], index_dev)]
     op = L.infiniopOperatorDescriptor_t()
-    L.check_error(L.LIBINFINIOP.infiniopCreatePagedCachingDescriptor(handle, ctypes.byref(op), *descs))
+    L.check_error(create(handle, ctypes.byref(op), *descs))
     for d in descs:
         L.destroy_tensor_descriptor(d)
     ws_size = c_size_t(0)
-    L.check_error(L.LIBINFINIOP.infiniopGetPagedCachingWorkspaceSize(op, ctypes.byref(ws_size)))
+    L.check_error(size_of(op, ctypes.byref(ws_size)))
 
     stream = c_void_p()
     L.check_error(L.LIBINFINIRT.infinirtStreamCreate(ctypes.byref(stream)))
@@ -257,9 +284,8 @@ def run_caching(args, torch, L, workloads, dev):
 
     def step(i):
         kc, vc, k, v = sets[i % len(sets)]
-        L.check_error(L.LIBINFINIOP.infiniopPagedCaching(
-            op, c_void_p(0), 0, c_void_p(kc.data_ptr()), c_void_p(vc.data_ptr()), c_void_p(k.data_ptr()),
-            c_void_p(v.data_ptr()), c_void_p(slots.data_ptr()), stream))
+        L.check_error(call(op, c_void_p(0), 0, c_void_p(kc.data_ptr()), c_void_p(vc.data_ptr()), c_void_p(k.data_ptr()),
+                           c_void_p(v.data_ptr()), c_void_p(index_dev.data_ptr()), stream))
 
     if args.pmc_calibration:
         pmc_calibration_copies(torch, dev)
@@ -280,10 +306,10 @@ def run_caching(args, torch, L, workloads, dev):
     L.check_error(L.LIBINFINIRT.infinirtEventElapsedTime(ctypes.byref(ms), ev0, ev1))
     us_wall = wall_s / args.steps * 1e6
     us_dev = ms.value / args.steps * 1e3
-    valid = int((inp.slot_mapping >= 0).sum())
+    config.update({"sets_rotated": len(sets), "algorithmic_bytes_per_call": algo_bytes})
 
     result = {
-        "metric": "paged_caching scatter achieved HBM GB/s (rows read + rows written + slot ids / time per call), 1 GPU",
+        "metric": metric,
         "value": round(algo_bytes / (us_wall * 1e-6) / 1e9, 1),
         "unit": "GB/s",
         "n_gpus": 1,
@@ -296,11 +322,7 @@ def run_caching(args, torch, L, workloads, dev):
         "vs_baseline": None,
         "dtype": "u8",
         "data": "synthetic",
-        "config": {
-            "workload": cfg.name, "num_tokens": cfg.num_tokens, "valid_tokens": valid, "num_kv_heads": cfg.num_kv_heads,
-            "head_size": cfg.head_size, "block_size": cfg.block_size, "num_slots": cfg.num_slots,
-            "sets_rotated": len(sets), "algorithmic_bytes_per_call": algo_bytes,
-        },
+        "config": config,
         "roofline": {
             "bound": "hbm",
             "achieved": round(algo_bytes / (us_dev * 1e-6) / 1e9, 1),
@@ -310,27 +332,25 @@ def run_caching(args, torch, L, workloads, dev):
             "traffic": MEASURED_TRAFFIC_BYTES.get(cfg.name),
             "us_per_call_device": round(us_dev, 2),
             "note": "achieved = algorithmic bytes / device time per call (events on the kernel's stream, back-to-back "
-                    "launches); a call moves 32 MB, which at 8 TB/s is 4 us: the size of a kernel launch",
+                    "launches); 32 MB per call is 4 us of traffic at 8 TB/s, the size of a kernel launch",
         },
     }
 
-    from oracle import paged_oracle
-
     if not args.no_check:
         kc, vc, k, v = sets[0]
-        want_k, want_v = paged_oracle.paged_caching(inp.k_cache.clone(), inp.v_cache.clone(), inp.k, inp.v, inp.slot_mapping)
+        want_k, want_v = oracle_fn(inp.k_cache.clone(), inp.v_cache.clone(), inp.k, inp.v, index)
         ok = bool(torch.equal(kc.cpu().view(torch.int16), want_k.view(torch.int16))
                   and torch.equal(vc.cpu().view(torch.int16), want_v.view(torch.int16)))
         result["parity"] = {"bit_exact": ok}
         if not ok:
             print(json.dumps(result))
-            print("bench.py: pools differ from the oracle's", file=sys.stderr)
+            print("bench.py: caches differ from the oracle's", file=sys.stderr)
             sys.exit(4)
     if not args.no_cpu_baseline:
         kc, vc = inp.k_cache.clone(), inp.v_cache.clone()
         reps, t0 = 0, time.perf_counter()
         while reps < 2000 and time.perf_counter() - t0 < 10.0:
-            paged_oracle.paged_caching(kc, vc, inp.k, inp.v, inp.slot_mapping)
+            oracle_fn(kc, vc, inp.k, inp.v, index)
             reps += 1
         cpu_s = (time.perf_counter() - t0) / reps
         result["cpu_baseline"] = {
@@ -338,7 +358,7 @@ def run_caching(args, torch, L, workloads, dev):
             "sample": f"{reps} full calls of the same workload through the C oracle (one thread), {cpu_s * 1e6:.0f} us per call",
         }
     print(json.dumps(result))
-    L.check_error(L.LIBINFINIOP.infiniopDestroyPagedCachingDescriptor(op))
+    L.check_error(destroy(op))
     L.check_error(L.LIBINFINIRT.infinirtEventDestroy(ev0))
     L.check_error(L.LIBINFINIRT.infinirtEventDestroy(ev1))
     L.check_error(L.LIBINFINIRT.infinirtStreamDestroy(stream))
@@ -360,7 +380,7 @@ def main():
         print("bench.py: no GPU visible; the HIP path has no CPU fallback", file=sys.stderr)
         sys.exit(3)
     dev = torch.device("cuda:0")
-    if args.workload in workloads.CACHING_CONFIGS:
+    if args.workload in workloads.CACHING_CONFIGS or args.workload in workloads.KV_CACHING_CONFIGS:
         args.steps = 400 if args.steps is None else args.steps
         args.warmup = 40 if args.warmup is None else args.warmup
         return run_caching(args, torch, L, workloads, dev)

@@ -4,6 +4,7 @@
 
 #include "infiniop/handle.h"
 #include "infiniop/operator_descriptor.h"
+#include "infiniop/ops/kv_caching.h"
 #include "infiniop/ops/paged_attention.h"
 #include "infiniop/ops/paged_attention_prefill.h"
 #include "infiniop/ops/paged_caching.h"

@@ -16,7 +16,7 @@
 -- The sources are the ones under infinicore_amd/csrc of this repository, copied to the matching
 -- places of the reference tree (src/infinirt/amd, src/infiniop/devices/amd,
 -- src/infiniop/ops/paged_attention/amd, src/infiniop/ops/paged_attention_prefill/amd,
--- src/infiniop/ops/paged_caching/amd).
+-- src/infiniop/ops/paged_caching/amd, src/infiniop/ops/kv_caching/amd).
 -- xmake is not installed in the environment this file was written in; the Makefile next to it builds
 -- the same objects with the same flags and is what the tests use.
 
@@ -78,7 +78,8 @@ target("infiniop-amd")
     add_links("amdhip64")
     add_cxflags("-fPIC")
     add_files("../src/infiniop/devices/amd/*.cc")
-    add_files("../src/infiniop/ops/paged_attention/amd/*.hip", "../src/infiniop/ops/paged_caching/amd/*.hip")
+    add_files("../src/infiniop/ops/paged_attention/amd/*.hip", "../src/infiniop/ops/paged_caching/amd/*.hip",
+              "../src/infiniop/ops/kv_caching/amd/*.hip")
     -- the prefill kernel keeps its matrix-instruction accumulators in ordinary vector registers
     add_files("../src/infiniop/ops/paged_attention_prefill/amd/*.hip", {cxflags = {"-mllvm", "-amdgpu-mfma-vgpr-form=1"}})
 target_end()

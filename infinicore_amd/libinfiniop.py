@@ -163,6 +163,10 @@ def _open():
     _declare(op, "infiniopGetPagedCachingWorkspaceSize", [D, POINTER(c_size_t)])
     _declare(op, "infiniopPagedCaching", [D, vp, c_size_t, vp, vp, vp, vp, vp, vp])
     _declare(op, "infiniopDestroyPagedCachingDescriptor", [D])
+    _declare(op, "infiniopCreateKVCachingDescriptor", [infiniopHandle_t, POINTER(D), T, T, T, T, T])
+    _declare(op, "infiniopGetKVCachingWorkspaceSize", [D, POINTER(c_size_t)])
+    _declare(op, "infiniopKVCaching", [D, vp, c_size_t, vp, vp, vp, vp, vp, vp])
+    _declare(op, "infiniopDestroyKVCachingDescriptor", [D])
     return rt, op
 
 

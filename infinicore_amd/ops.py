@@ -220,3 +220,39 @@ def paged_caching(k_cache, v_cache, k, v, slot_mapping):
         "infiniopPagedCaching",
     )
     return k_cache, v_cache
+
+
+def kv_caching(k_cache, v_cache, k, v, past_kv_lengths):
+    """Append ``k`` / ``v`` [batch, num_kv_heads, seq_len, d] to the contiguous caches
+    [batch, num_kv_heads, max_seq_len, d] behind the first ``past_kv_lengths[b]`` positions, in place; returns
+    the caches (argument order of the reference's infiniopKVCaching, include/infiniop/ops/kv_caching.h:8-29)."""
+    index = _device_index(k)
+    tensors = (k_cache, v_cache, k, v, past_kv_lengths)
+    key = ("kv_caching", index, *(_meta(t) for t in tensors))
+
+    def make():
+        handle = _handle_for(index)
+        descs = [_describe(t) for t in tensors]
+        op = lib.infiniopOperatorDescriptor_t()
+        try:
+            check_error(
+                LIBINFINIOP.infiniopCreateKVCachingDescriptor(handle, ctypes.byref(op), *descs),
+                "infiniopCreateKVCachingDescriptor",
+            )
+        finally:
+            for d in descs:
+                lib.destroy_tensor_descriptor(d)
+        size = c_size_t(0)
+        check_error(LIBINFINIOP.infiniopGetKVCachingWorkspaceSize(op, ctypes.byref(size)))
+        return _Plan(op, LIBINFINIOP.infiniopDestroyKVCachingDescriptor, size.value, k.device)
+
+    plan = _cached_plan(key, make)
+    lib.set_device(InfiniDevice.AMD, index)
+    check_error(
+        LIBINFINIOP.infiniopKVCaching(
+            plan.descriptor, _ptr(plan.workspace), plan.workspace_bytes, _ptr(k_cache), _ptr(v_cache), _ptr(k),
+            _ptr(v), _ptr(past_kv_lengths), _stream_ptr(index),
+        ),
+        "infiniopKVCaching",
+    )
+    return k_cache, v_cache

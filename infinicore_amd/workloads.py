@@ -93,6 +93,25 @@ CACHING_CONFIGS = {
 }
 
 
+@dataclass
+class KVCachingConfig:
+    """Append to contiguous (non-paged) caches: ``new_tokens`` tokens per sequence behind random past lengths."""
+    name: str
+    dtype: torch.dtype
+    batch: int
+    num_kv_heads: int
+    max_seq_len: int
+    new_tokens: int
+    head_size: int
+    seed: int = 0
+
+
+KV_CACHING_CONFIGS = {
+    "k1_append_decode_step": KVCachingConfig("k1_append_decode_step", torch.bfloat16, 32, 8, 4096, 1, 128, seed=301),
+    "k2_append_prefill_chunk": KVCachingConfig("k2_append_prefill_chunk", torch.bfloat16, 8, 8, 8192, 512, 128, seed=302),
+}
+
+
 PREFILL_CONFIGS = {
     "p1_plumbing_mha": PrefillConfig("p1_plumbing_mha", torch.float16, 4, 8, 8, 128, 16, 1, 64, 0, 128, seed=201),
     "p2_llama3_8b_prompt": PrefillConfig("p2_llama3_8b_prompt", torch.bfloat16, 4, 32, 8, 128, 16, 1024, 4096, 0, 0,
@@ -254,3 +273,30 @@ def make_caching_inputs(cfg: CachingConfig) -> CachingInputs:
     k_cache = torch.full(shape, -777.0, dtype=cfg.dtype)
     v_cache = torch.full(shape, 555.0, dtype=cfg.dtype)
     return CachingInputs(cfg, k, v, k_cache, v_cache, torch.from_numpy(slots))
+
+
+@dataclass
+class KVCachingInputs:
+    config: KVCachingConfig
+    k: torch.Tensor                # [B, Hkv, new_tokens, D]
+    v: torch.Tensor
+    k_cache: torch.Tensor          # [B, Hkv, max_seq_len, D], pre-filled with a sentinel
+    v_cache: torch.Tensor
+    past_kv_lengths: torch.Tensor  # [B] int64
+
+
+def kv_caching_algorithmic_bytes(cfg: KVCachingConfig) -> int:
+    e = 2 if cfg.dtype in (torch.float16, torch.bfloat16) else 4
+    moved = cfg.batch * cfg.num_kv_heads * cfg.new_tokens * cfg.head_size * e * 2  # K and V
+    return 2 * moved + cfg.batch * 8  # read + write + lengths
+
+
+def make_kv_caching_inputs(cfg: KVCachingConfig) -> KVCachingInputs:
+    rng = np.random.default_rng([cfg.seed, 13])
+    new_shape = (cfg.batch, cfg.num_kv_heads, cfg.new_tokens, cfg.head_size)
+    cache_shape = (cfg.batch, cfg.num_kv_heads, cfg.max_seq_len, cfg.head_size)
+    k, v = _normal(rng, new_shape, cfg.dtype), _normal(rng, new_shape, cfg.dtype)
+    past = rng.integers(0, cfg.max_seq_len - cfg.new_tokens + 1, size=cfg.batch, dtype=np.int64)
+    k_cache = torch.full(cache_shape, -777.0, dtype=cfg.dtype)
+    v_cache = torch.full(cache_shape, 555.0, dtype=cfg.dtype)
+    return KVCachingInputs(cfg, k, v, k_cache, v_cache, torch.from_numpy(past))

@@ -1,5 +1,5 @@
 /*
- * CPU oracle for InfiniOP paged_attention (decode), paged_attention_prefill and paged_caching.
+ * CPU oracle for InfiniOP paged_attention (decode), paged_attention_prefill, paged_caching and kv_caching.
  *
  * TEST INFRASTRUCTURE ONLY. This file restates, in plain C, the algorithm of the reference's device
  * kernels so that the HIP kernels of this repository can be checked against it. Only tests/,
@@ -12,7 +12,7 @@
  * scaled_dot_product_attention on the gathered sequence, closed forms (length 1, equal V rows,
  * zero query, one dominant key), invariance under page permutation, GQA == MHA on repeated heads,
  * split == unsplit, prefill row j == decode over the first history + j + 1 tokens, prefill against an
- * fp64 masked softmax, and a byte-exact scatter model for paged_caching.
+ * fp64 masked softmax, and byte-exact copy models (numpy assignment) for paged_caching and kv_caching.
  *
  * Functions and the reference code each one follows:
  *   oracle_paged_attention         src/infiniop/ops/paged_attention/cuda/kernel_v2.cuh:134-336
@@ -26,6 +26,9 @@
  *   oracle_paged_caching           src/infiniop/ops/paged_caching/cuda/kernel.cuh:22-89
  *                                  (slot < 0 skipped, page = slot / block_size, row = slot % block_size,
  *                                  source heads packed, element-wise copy)
+ *   oracle_kv_caching              src/infiniop/ops/kv_caching/cuda/kernel.cuh:32-58
+ *                                  (element (b, h, s, d) of the new tensors goes to cache position
+ *                                  past_kv_lengths[b] + s; every dimension of every tensor strided)
  *
  * Build: make -C oracle   (gcc -O2 -fopenmp -shared)
  */
@@ -405,4 +408,45 @@ int oracle_paged_caching(void *k_cache_, void *v_cache_, const void *k_, const v
         }
     }
     return 0;
+}
+
+typedef struct {
+    int64_t elem_size; /* bytes per element: 2 or 4 */
+    int64_t batch_size, num_kv_heads, max_seq_len, seq_len, hidden_dim;
+    /* element strides of dims 0..3 */
+    int64_t k_cache_strides[4], v_cache_strides[4], k_strides[4], v_strides[4];
+} oracle_kv_caching_shape;
+
+/* Append to contiguous caches, kv_caching/cuda/kernel.cuh:32-58: one element at a time, position
+ * past_kv_lengths[b] + s. A position outside the cache is an out-of-bounds write in the reference and
+ * reported here (-2) without touching anything for that row. */
+int oracle_kv_caching(void *k_cache_, void *v_cache_, const void *k_, const void *v_, const int64_t *past_kv_lengths,
+                      const oracle_kv_caching_shape *s) {
+    if (s->elem_size != 2 && s->elem_size != 4) {
+        return -1;
+    }
+    char *k_cache = (char *)k_cache_, *v_cache = (char *)v_cache_;
+    const char *k = (const char *)k_, *v = (const char *)v_;
+    const int64_t es = s->elem_size;
+    int rc = 0;
+    for (int64_t b = 0; b < s->batch_size; ++b) {
+        for (int64_t h = 0; h < s->num_kv_heads; ++h) {
+            for (int64_t t = 0; t < s->seq_len; ++t) {
+                const int64_t pos = past_kv_lengths[b] + t; /* :48-50 */
+                if (pos < 0 || pos >= s->max_seq_len) {
+                    rc = -2;
+                    continue;
+                }
+                for (int64_t d = 0; d < s->hidden_dim; ++d) {
+                    const int64_t kc = b * s->k_cache_strides[0] + h * s->k_cache_strides[1] + pos * s->k_cache_strides[2] + d * s->k_cache_strides[3];
+                    const int64_t vc = b * s->v_cache_strides[0] + h * s->v_cache_strides[1] + pos * s->v_cache_strides[2] + d * s->v_cache_strides[3];
+                    const int64_t ks = b * s->k_strides[0] + h * s->k_strides[1] + t * s->k_strides[2] + d * s->k_strides[3];
+                    const int64_t vs = b * s->v_strides[0] + h * s->v_strides[1] + t * s->v_strides[2] + d * s->v_strides[3];
+                    memcpy(k_cache + kc * es, k + ks * es, (size_t)es); /* :51-57 */
+                    memcpy(v_cache + vc * es, v + vs * es, (size_t)es);
+                }
+            }
+        }
+    }
+    return rc;
 }

@@ -51,6 +51,12 @@ class CachingShape(Structure):
     ]
 
 
+class KVCachingShape(Structure):
+    _fields_ = [(name, c_int64) for name in ("elem_size", "batch_size", "num_kv_heads", "max_seq_len", "seq_len",
+                                             "hidden_dim")] + [
+        (name, c_int64 * 4) for name in ("k_cache_strides", "v_cache_strides", "k_strides", "v_strides")]
+
+
 def build() -> None:
     proc = subprocess.run(["make", "-C", str(_DIR)], capture_output=True, text=True)
     if proc.returncode != 0:
@@ -74,6 +80,8 @@ def load():
         lib.oracle_paged_attention_prefill.restype = c_int
         lib.oracle_paged_caching.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, POINTER(CachingShape)]
         lib.oracle_paged_caching.restype = c_int
+        lib.oracle_kv_caching.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, POINTER(KVCachingShape)]
+        lib.oracle_kv_caching.restype = c_int
         lib.oracle_to_float.argtypes = [ctypes.c_uint16, c_int]
         lib.oracle_to_float.restype = c_float
         lib.oracle_from_float.argtypes = [c_float, c_int]
@@ -180,6 +188,31 @@ def paged_caching(k_cache, v_cache, k, v, slot_mapping):
                                   _cpu(v).data_ptr(), slot_mapping.data_ptr(), ctypes.byref(s))
     if rc != 0:
         raise ValueError("oracle rejected the arguments")
+    return k_cache, v_cache
+
+
+def kv_caching(k_cache, v_cache, k, v, past_kv_lengths):
+    """C oracle append to contiguous caches; writes into ``k_cache`` / ``v_cache`` in place and returns them.
+    Raises if a new token would land outside the cache (an out-of-bounds write in the reference)."""
+    lib = load()
+    past = _cpu(past_kv_lengths).to(torch.int64).contiguous()
+    s = KVCachingShape(k.element_size(), k_cache.shape[0], k_cache.shape[1], k_cache.shape[2], k.shape[2], k_cache.shape[3],
+                       (c_int64 * 4)(*k_cache.stride()), (c_int64 * 4)(*v_cache.stride()),
+                       (c_int64 * 4)(*k.stride()), (c_int64 * 4)(*v.stride()))
+    rc = lib.oracle_kv_caching(_cpu(k_cache).data_ptr(), _cpu(v_cache).data_ptr(), _cpu(k).data_ptr(),
+                               _cpu(v).data_ptr(), past.data_ptr(), ctypes.byref(s))
+    if rc != 0:
+        raise ValueError("oracle rejected the arguments" if rc == -1 else "a new token lands outside the cache")
+    return k_cache, v_cache
+
+
+def torch_reference_kv_caching(k_cache, v_cache, k, v, past_kv_lengths):
+    """The expected-value function of the reference's test (test/infiniop/kv_caching.py:23-33), restated."""
+    seq_len = k.shape[2]
+    for b in range(k_cache.shape[0]):
+        past = int(past_kv_lengths[b])
+        k_cache[b, :, past:past + seq_len, :] = k[b]
+        v_cache[b, :, past:past + seq_len, :] = v[b]
     return k_cache, v_cache
 
 

@@ -133,3 +133,30 @@ def run_paged_caching(handle, k_cache, v_cache, k, v, slot_mapping, stream=None)
     torch.cuda.synchronize()
     L.check_error(L.LIBINFINIOP.infiniopDestroyPagedCachingDescriptor(op))
     return k_cache, v_cache
+
+
+def create_kv_caching(handle, k_cache, v_cache, k, v, past_kv_lengths):
+    descs = [describe(t) for t in (k_cache, v_cache, k, v, past_kv_lengths)]
+    op = L.infiniopOperatorDescriptor_t()
+    status = L.LIBINFINIOP.infiniopCreateKVCachingDescriptor(handle, ctypes.byref(op), *descs)
+    for d in descs:
+        L.destroy_tensor_descriptor(d)
+    return status, op
+
+
+def run_kv_caching(handle, k_cache, v_cache, k, v, past_kv_lengths, stream=None):
+    """In place on the device caches (the sequence of calls of test/infiniop/kv_caching.py:95-150); returns them."""
+    status, op = create_kv_caching(handle, k_cache, v_cache, k, v, past_kv_lengths)
+    L.check_error(status, "infiniopCreateKVCachingDescriptor")
+    size = c_size_t(123)
+    L.check_error(L.LIBINFINIOP.infiniopGetKVCachingWorkspaceSize(op, ctypes.byref(size)))
+    assert size.value == 0
+    torch.cuda.synchronize()
+    L.check_error(
+        L.LIBINFINIOP.infiniopKVCaching(op, c_void_p(0), 0, ptr(k_cache), ptr(v_cache), ptr(k), ptr(v),
+                                        ptr(past_kv_lengths), c_void_p(stream or 0)),
+        "infiniopKVCaching",
+    )
+    torch.cuda.synchronize()
+    L.check_error(L.LIBINFINIOP.infiniopDestroyKVCachingDescriptor(op))
+    return k_cache, v_cache

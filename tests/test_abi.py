@@ -25,6 +25,8 @@ def test_headers_declare_the_expected_entry_points():
         "infiniopGetPagedAttentionPrefillWorkspaceSize", "infiniopPagedAttentionPrefill",
         "infiniopDestroyPagedAttentionPrefillDescriptor", "infiniopCreatePagedCachingDescriptor",
         "infiniopGetPagedCachingWorkspaceSize", "infiniopPagedCaching", "infiniopDestroyPagedCachingDescriptor",
+        "infiniopCreateKVCachingDescriptor", "infiniopGetKVCachingWorkspaceSize", "infiniopKVCaching",
+        "infiniopDestroyKVCachingDescriptor",
         "infiniopCreateHandle", "infiniopDestroyHandle", "infiniopCreateTensorDescriptor",
         "infiniopDestroyTensorDescriptor", "infinirtSetDevice", "infinirtMalloc", "infinirtStreamCreate",
     ):
