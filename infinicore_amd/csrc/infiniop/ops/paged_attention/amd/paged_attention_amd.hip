@@ -75,9 +75,17 @@ Plan makePlan(const PagedAttentionInfo &in, const device::amd::DeviceInfo &dev) 
     const long long group = static_cast<long long>(in.num_heads / in.num_kv_heads);
     const long long stream_count = static_cast<long long>(in.num_kv_heads) * ((group + kHeadsPerWave - 1) / kHeadsPerWave);
     const long long units = static_cast<long long>(in.num_seqs) * (plan.tiled ? stream_count : static_cast<long long>(in.num_heads));
+    // A job whose block table cannot hold more than 16 tiles per wavefront of the work-equalising schedule
+    // (134 MB of K and V at head 128) is over in 10 - 30 us, and there the fixed partitions win: their
+    // wavefronts start with two round trips less and share a SIMD two at a time (one sequence of 2 100
+    // tokens: 10.4 vs 15.9 us; 4 ragged sequences: 14.2 vs 18.6; 8: 22.2 vs 22.0; 16: 34.6 vs 33.4).
+    const long long max_tiles = (max_tokens + kTileTokens - 1) / kTileTokens;
+    const bool small_job = plan.tiled && !latent_head
+                        && static_cast<long long>(in.num_seqs) * stream_count * max_tiles <= 64LL * dev.compute_units;
     // A unit of the latent-attention kernel leaves 32 KiB of partial results and advances one tile per
     // memory latency however many units there are: fewer, longer units measured best there.
     long long want = latent_head ? units * max_tokens * 3 / (16LL * dev.compute_units)
+                   : small_job   ? units * max_tokens / (8LL * dev.compute_units)
                                  : units * max_tokens / (16LL * dev.compute_units);
     int p = floorPow2(want < 1 ? 1 : want);
     const int p_min = latent_head ? 256 : 64;
@@ -109,10 +117,12 @@ Plan makePlan(const PagedAttentionInfo &in, const device::amd::DeviceInfo &dev) 
     // with as many wavefronts as fill the device once at one wavefront per SIMD (4 per compute unit,
     // the setting that measured best: every compute unit gets the same number, each wavefront streams
     // as long as possible), each with an equal share of the tiles.
-    plan.balanced = plan.tiled && !latent_head && in.num_seqs <= static_cast<size_t>(kBalancedMaxSeqs);
+    plan.balanced = plan.tiled && !latent_head && !small_job && in.num_seqs <= static_cast<size_t>(kBalancedMaxSeqs);
     if (const char *env = std::getenv("INFINIOP_AMD_PA_SCHEDULE")) {
         if (std::strcmp(env, "grid") == 0) {
             plan.balanced = false;
+        } else if (std::strcmp(env, "balanced") == 0) {
+            plan.balanced = plan.tiled && !latent_head && in.num_seqs <= static_cast<size_t>(kBalancedMaxSeqs);
         }
     }
     if (plan.balanced) {

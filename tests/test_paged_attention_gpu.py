@@ -23,6 +23,14 @@ ORACLE_THREADS = min(16, os.cpu_count() or 1)
 DEV = "cuda:0"
 
 
+@pytest.fixture(autouse=True)
+def balanced_schedule_unless_the_test_says_otherwise(monkeypatch):
+    """Small jobs are routed to the fixed-partition schedule by default; most cases here are small but are
+    meant to exercise the work-equalising kernels, so that schedule is forced (tests that set the variable
+    themselves override this; test_default_schedule_choice removes it)."""
+    monkeypatch.setenv("INFINIOP_AMD_PA_SCHEDULE", "balanced")
+
+
 def ulp_of(dtype, x):
     """Spacing of the storage dtype at |x|."""
     bits = 10 if dtype == torch.float16 else 7
@@ -278,6 +286,14 @@ def test_mla_padded_cache_rows(gpu_handle, oracle):
 
 def test_mla_full_size_against_oracle(gpu_handle, oracle):
     run_case(gpu_handle, oracle, workloads.make_decode_inputs(workloads.DECODE_CONFIGS["m1_mla_16_heads_b32"]))
+
+
+@pytest.mark.parametrize("B,lo,hi", [(1, 2100, 2100), (4, 512, 4096), (16, 512, 4096)])
+def test_default_schedule_choice(gpu_handle, oracle, monkeypatch, B, lo, hi):
+    """No knob set: one sequence and four ragged ones take the fixed partitions (small job), sixteen the
+    work-equalising schedule; all must agree with the oracle."""
+    monkeypatch.delenv("INFINIOP_AMD_PA_SCHEDULE", raising=False)
+    run_case(gpu_handle, oracle, workloads.make_decode_inputs(custom(f"default_b{B}", torch.bfloat16, B, 32, 8, 128, 16, lo, hi, seed=500 + B)))
 
 
 # ---- every kernel and schedule against the same oracle ---------------------------------------------
