@@ -4,17 +4,18 @@
 // partitions; with ragged lengths the number of units does not match the number of wavefronts the
 // device can hold, and the last, half-empty round costs as much as a full one. Here the device
 // does the split itself: for one KV head (and chunk of 16 query heads) all 16-token tiles of all
-// sequences form one flat range [0, T); it is cut into `waves_per_stream` equal pieces, one per
-// wavefront, so every wavefront streams the same number of bytes and they all finish together in a
-// single round. A piece may cover the end of one sequence and the start of the next; each
-// (piece, sequence) intersection is a segment with its own softmax state.
+// sequences form one flat range [0, T); it is cut into `waves_per_stream` pieces of equal cost (equal
+// tile counts, less a few tiles for every sequence that starts inside the piece), one per wavefront,
+// so they all finish together in a single round. A piece may cover the end of one sequence and the
+// start of the next; each (piece, sequence) intersection is a segment with its own softmax state.
 //
 // Every wavefront derives the split from seq_lens alone (a prefix sum over the batch, redone per
 // wavefront, kept in LDS), so nothing is read back to the host and no wavefront waits for another.
 //   * a segment that covers its whole sequence is normalised and written to `out` directly;
 //   * any other segment leaves (acc, m, l) in workspace row (piece + sequence), which is unique
 //     per segment because consecutive segments advance the piece, the sequence or both;
-//   * decodeBalancedMergeKernel recomputes the same split and merges the rows of each sequence.
+//   * the wavefront whose piece holds a sequence's first tile records which pieces the sequence spans
+//     (seq_pieces), and decodeBalancedMergeKernel merges the rows of each sequence from that.
 // Tile arithmetic is computeTile() of decode_tiled.h unchanged.
 #ifndef INFINICORE_AMD_PA_DECODE_BALANCED_H
 #define INFINICORE_AMD_PA_DECODE_BALANCED_H
@@ -79,8 +80,8 @@ __device__ __forceinline__ int tilePrefixSums(const DecodeArgs &a, int lane, int
     return __builtin_amdgcn_readfirstlane(running);
 }
 
-// Tiles per piece: the flat range split evenly over the wavefronts of a stream, but never finer
-// than kBalancedMinTiles. Decode and merge kernels must agree on this.
+// Slots (tiles plus start costs) per piece: the range split evenly over the wavefronts of a stream, but
+// never finer than kBalancedMinTiles.
 __device__ __forceinline__ int tilesPerPiece(int total_tiles, int waves_per_stream) {
     const int q = (total_tiles + waves_per_stream - 1) / waves_per_stream;
     return q < kBalancedMinTiles ? kBalancedMinTiles : q;
