@@ -217,10 +217,12 @@ def mla(name, dtype, B, H, bs, lo, hi, seed, **kw):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("H", [16, 128, 20])
+@pytest.mark.parametrize("H", [16, 128, 20, 48, 80])
 def test_mla_ragged_batches(gpu_handle, oracle, dtype, H):
     """Ragged lengths incl. 1 token and exactly one page, long enough that sequences are split into
-    partitions and merged; 16 heads (one wavefront per unit), 128 (eight) and 20 (a partly filled one)."""
+    partitions and merged; 16 heads (one chunk of 16 per workgroup), 20 (two chunks, one partly filled), 48
+    (three chunks in workgroups of two: one workgroup slot without heads), 80 (five in workgroups of four) and
+    128 (eight)."""
     inp = workloads.make_decode_inputs(mla(f"mla_h{H}", dtype, 5, H, 16, 1, 2500, seed=400 + H))
     inp.seq_lens[0], inp.seq_lens[1] = 1, 16
     got, _ = run_case(gpu_handle, oracle, inp)
