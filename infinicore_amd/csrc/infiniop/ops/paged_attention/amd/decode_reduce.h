@@ -6,7 +6,8 @@
 //
 // One 256-thread workgroup per (query head, sequence). Thread = (row group rg = tid / 16, strip
 // c = tid % 16): it merges partitions rg, rg+16, ... for the value_size/16 output columns of strip
-// c, so all partial rows of up to 16 partitions are fetched by one round of independent loads.
+// c (groups of four columns, 64 apart), so all partial rows of up to 16 partitions are fetched by
+// one round of independent, coalesced loads.
 // Row groups are then merged with the same associative rule: inside a wavefront with lane swaps,
 // across the four wavefronts through LDS.
 #ifndef INFINICORE_AMD_PA_DECODE_REDUCE_H
@@ -39,13 +40,16 @@ __device__ __forceinline__ float mergeWeight(float m, float m_ref) {
     return m == -INFINITY ? 0.0f : fastExp2(m - m_ref);
 }
 
-// COLS = value_size / 16 output columns per thread (a multiple of 4).
+// COLS = value_size / 16 output columns per thread (a multiple of 4): strip c owns the COLS/4 groups of
+// four columns 64 i + 4 c .. + 3, so the 16 threads of a row group read 256 contiguous bytes of a partial
+// row with every load instruction and write 128 contiguous bytes of the output row per group.
 template <typename T, typename Tindex, int COLS>
 __global__ void __launch_bounds__(kReduceThreads) decodeReduceKernel(DecodeArgs a) {
     using S = typename T::storage;
-    __shared__ float wave_acc[4][16][COLS];
-    __shared__ float wave_m[4][16];
-    __shared__ float wave_l[4][16];
+    constexpr int kGroups = COLS / 4;
+    __shared__ float4 wave_acc[4][kGroups][16];
+    __shared__ float wave_m[4];
+    __shared__ float wave_l[4];
 
     const int head = blockIdx.x;
     const int seq = blockIdx.y;
@@ -65,29 +69,29 @@ __global__ void __launch_bounds__(kReduceThreads) decodeReduceKernel(DecodeArgs 
 
     // this thread's partitions: running (m, l, acc) merge
     float m_loc = -INFINITY, l_loc = 0.0f;
-    float acc[COLS];
+    float4 acc[kGroups];
 #pragma unroll
-    for (int i = 0; i < COLS; ++i) {
-        acc[i] = 0.0f;
+    for (int i = 0; i < kGroups; ++i) {
+        acc[i] = make_float4(0.f, 0.f, 0.f, 0.f);
     }
     for (int p = rg; p < parts; p += kReduceRowGroups) {
         const float m_p = a.part_m[slot0 + p];
         const float l_p = a.part_l[slot0 + p];
-        const float4 *row = reinterpret_cast<const float4 *>(a.part_acc + (slot0 + p) * a.value_size + c * COLS);
-        float4 v[COLS / 4];
+        const float4 *row = reinterpret_cast<const float4 *>(a.part_acc + (slot0 + p) * a.value_size) + c;
+        float4 v[kGroups];
 #pragma unroll
-        for (int i = 0; i < COLS / 4; ++i) {
-            v[i] = row[i];
+        for (int i = 0; i < kGroups; ++i) {
+            v[i] = row[16 * i];
         }
         const float m_new = fmaxf(m_loc, m_p);
         const float w_old = mergeWeight(m_loc, m_new), w_p = mergeWeight(m_p, m_new);
         l_loc = l_loc * w_old + l_p * w_p;
 #pragma unroll
-        for (int i = 0; i < COLS / 4; ++i) {
-            acc[4 * i + 0] = acc[4 * i + 0] * w_old + v[i].x * w_p;
-            acc[4 * i + 1] = acc[4 * i + 1] * w_old + v[i].y * w_p;
-            acc[4 * i + 2] = acc[4 * i + 2] * w_old + v[i].z * w_p;
-            acc[4 * i + 3] = acc[4 * i + 3] * w_old + v[i].w * w_p;
+        for (int i = 0; i < kGroups; ++i) {
+            acc[i].x = acc[i].x * w_old + v[i].x * w_p;
+            acc[i].y = acc[i].y * w_old + v[i].y * w_p;
+            acc[i].z = acc[i].z * w_old + v[i].z * w_p;
+            acc[i].w = acc[i].w * w_old + v[i].w * w_p;
         }
         m_loc = m_new;
     }
@@ -97,46 +101,43 @@ __global__ void __launch_bounds__(kReduceThreads) decodeReduceKernel(DecodeArgs 
     const float f = mergeWeight(m_loc, m_w);
     const float l_w = swapSum(l_loc * f);
 #pragma unroll
-    for (int i = 0; i < COLS; ++i) {
-        acc[i] = swapSum(acc[i] * f);
+    for (int i = 0; i < kGroups; ++i) {
+        acc[i].x = swapSum(acc[i].x * f);
+        acc[i].y = swapSum(acc[i].y * f);
+        acc[i].z = swapSum(acc[i].z * f);
+        acc[i].w = swapSum(acc[i].w * f);
     }
     if ((tid & 63) < 16) {
-        wave_m[wave][c] = m_w;
-        wave_l[wave][c] = l_w;
+        if (c == 0) {
+            wave_m[wave] = m_w; // the 16 strips of a row group went through the same partitions
+            wave_l[wave] = l_w;
+        }
 #pragma unroll
-        for (int i = 0; i < COLS; ++i) {
-            wave_acc[wave][c][i] = acc[i];
+        for (int i = 0; i < kGroups; ++i) {
+            wave_acc[wave][i][c] = acc[i];
         }
     }
     __syncthreads();
 
-    // the first 16 threads merge the four wavefronts, normalise and store COLS columns each
-    if (tid < 16) {
-        float m = wave_m[0][c];
-#pragma unroll
-        for (int w = 1; w < 4; ++w) {
-            m = fmaxf(m, wave_m[w][c]);
-        }
-        float l = 0.0f, out_acc[COLS];
-#pragma unroll
-        for (int i = 0; i < COLS; ++i) {
-            out_acc[i] = 0.0f;
-        }
+    // one thread per group of four columns merges the four wavefronts, normalises and stores
+    for (int e = tid; e < 16 * kGroups; e += kReduceThreads) {
+        const int i = e >> 4, cc = e & 15;
+        const float m = fmaxf(fmaxf(wave_m[0], wave_m[1]), fmaxf(wave_m[2], wave_m[3]));
+        float l = 0.0f;
+        float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
         for (int w = 0; w < 4; ++w) {
-            const float fw = mergeWeight(wave_m[w][c], m);
-            l += wave_l[w][c] * fw;
-#pragma unroll
-            for (int i = 0; i < COLS; ++i) {
-                out_acc[i] += wave_acc[w][c][i] * fw;
-            }
+            const float fw = mergeWeight(wave_m[w], m);
+            const float4 x = wave_acc[w][i][cc];
+            l += wave_l[w] * fw;
+            sum.x += x.x * fw, sum.y += x.y * fw, sum.z += x.z * fw, sum.w += x.w * fw;
         }
         const float inv_l = 1.0f / (l + 1e-6f);
-        S *o_ptr = static_cast<S *>(a.out) + seq * a.o_stride + head * a.o_head_stride + c * COLS;
-#pragma unroll
-        for (int i = 0; i < COLS; ++i) {
-            o_ptr[i] = T::fromFloat(out_acc[i] * inv_l);
-        }
+        S *o_ptr = static_cast<S *>(a.out) + seq * a.o_stride + head * a.o_head_stride + 64 * i + 4 * cc;
+        o_ptr[0] = T::fromFloat(sum.x * inv_l);
+        o_ptr[1] = T::fromFloat(sum.y * inv_l);
+        o_ptr[2] = T::fromFloat(sum.z * inv_l);
+        o_ptr[3] = T::fromFloat(sum.w * inv_l);
     }
 }
 
