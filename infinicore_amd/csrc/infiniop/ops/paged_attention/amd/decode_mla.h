@@ -15,10 +15,12 @@
 //     tile of 32 registers, consumed in two strips of 128 columns; as soon as a strip of V(t) has been
 //     used the same strip of V(t+1) is requested into its registers;
 //   * the query rows sit in LDS next to the K tile and are read back K-step by K-step.
-// That fits 256 registers per wavefront (188 as compiled; a second register set for K or V does not fit
-// without spills inside the loop), so every SIMD holds two wavefronts. Every request has one step of
-// the loop to arrive, so a unit advances one tile per memory latency (2.1 - 2.8 us measured); throughput
-// comes from the four units a compute unit's LDS holds.
+// That fits 256 registers per wavefront (188 as compiled), so every SIMD holds two wavefronts and a compute
+// unit's LDS four units. A unit advances one tile per 1.9 - 2.5 us however many units run and whether or not
+// the pages sit in cache: its pace is set by the order-preserving return of one wavefront's loads (about
+// one 128-byte line per 10 - 15 ns, 136 lines per tile and wavefront) plus the part of the matrix and
+// vector work that does not overlap with it, so throughput comes from the number of units. A second
+// register set for K or V (two tiles in flight, one wavefront per SIMD) was measured and is slower.
 // (Direct global -> LDS loads would free the K registers as well, but with one of those outstanding this
 // compiler turns every wait on a vector-memory result into a wait for all of them, which serialises the
 // pipeline.)

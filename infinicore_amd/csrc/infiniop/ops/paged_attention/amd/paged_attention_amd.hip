@@ -83,7 +83,8 @@ Plan makePlan(const PagedAttentionInfo &in, const device::amd::DeviceInfo &dev) 
     const bool small_job = plan.tiled && !latent_head
                         && static_cast<long long>(in.num_seqs) * stream_count * max_tiles <= 64LL * dev.compute_units;
     // A unit of the latent-attention kernel leaves 32 KiB of partial results and advances one tile per
-    // memory latency however many units there are: fewer, longer units measured best there.
+    // ~2 us however many units there are: fewer, longer units measured best there (more units end the
+    // decode kernel sooner, but writing and merging their partial results costs more than that gains).
     long long want = latent_head ? units * max_tokens * 3 / (16LL * dev.compute_units)
                    : small_job   ? units * max_tokens / (8LL * dev.compute_units)
                                  : units * max_tokens / (16LL * dev.compute_units);
