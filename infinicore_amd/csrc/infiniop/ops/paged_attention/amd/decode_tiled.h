@@ -22,7 +22,7 @@
 //                              in the registers S came out in, B = V strip; lane holds
 //                              O[4g..4g+3][8c+e] for e = 0..7)
 // The softmax denominator sums the rounded probabilities, so numerator and denominator see the same
-// weights. Accumulators are rescaled only when some head's maximum actually moves.
+// weights. Accumulators are rescaled only when some head's maximum has outgrown the reference point by 2^8.
 // The math follows the reference's decode kernels (src/infiniop/ops/paged_attention/cuda/
 // kernel_v2.cuh:134-336 for the recurrence, :340-554 for per-shard partial results).
 #ifndef INFINICORE_AMD_PA_DECODE_TILED_H
@@ -83,6 +83,7 @@ struct TileF16 : Half {
 constexpr int kTileTokens = 16;     // tokens per tile = rows of one matrix instruction
 constexpr int kTiledHead = 128;     // the head size the kernels were tuned on (others: 64, 192, 256)
 constexpr int kHeadsPerWave = 16;   // query heads of one KV head packed into one wavefront
+constexpr float kLazyRescaleLog2 = 8.0f; // how far (in powers of two) a maximum may outgrow its reference point
 
 // Geometry of a 16-token tile for head_size = value_size = HEAD (64, 128, 192 or 256).
 //   K: 16 rows of HEAD/8 16-byte chunks; the wavefront fetches them in kLoads = HEAD/32 instructions,
@@ -244,9 +245,12 @@ __device__ __forceinline__ void softmaxStep(f32x4 (&o)[COLS], float &m, float &l
     const float mx = maxAcrossTokenGroups(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])));
     const float m_new = fmaxf(m, mx);
 
-    if (__builtin_amdgcn_ballot_w64(m_new > m) != 0) {
-        // some head's maximum moved: rescale. Lane holds accumulators of heads 4g..4g+3, whose
-        // factors live in lanes 4g..4g+3.
+    // m only has to keep the exponentials in range, it need not be the exact maximum: it is moved (and the
+    // accumulators rescaled) only when some head's maximum has outgrown it by more than 2^kLazyRescaleLog2,
+    // so a probability reaches at most that factor above 1. Numerator and denominator carry the same
+    // reference point, the quotient is unchanged, and the partial results stay mergeable as they are.
+    if (__builtin_amdgcn_ballot_w64(mx > m + kLazyRescaleLog2) != 0) {
+        // rescale. Lane holds accumulators of heads 4g..4g+3, whose factors live in lanes 4g..4g+3.
         const float alpha = fastExp2(m - m_new);
         l *= alpha;
         m = m_new;

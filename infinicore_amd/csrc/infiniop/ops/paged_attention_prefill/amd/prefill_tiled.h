@@ -53,6 +53,7 @@ using op::paged_attention::amd::storeStrip;
 using op::paged_attention::amd::TileGeometry;
 
 constexpr int kPrefillThreads = 256;
+constexpr float kLazyLog2 = 8.0f; // how far (in powers of two) a row maximum may outgrow its reference point
 
 // 16-byte load from (wave-uniform base) + (32-bit per-lane byte offset), through the caches: K/V tiles
 // are read again by the other row blocks of the sequence. The empty asm keeps the offset a value
@@ -399,9 +400,13 @@ __global__ void __launch_bounds__(kPrefillThreads, HEAD <= 192 ? 2 : 1) prefillT
             }
             mx = maxAcrossTokenGroups(mx);
             const float m_new = fmaxf(m[r], mx);
-            if (__builtin_amdgcn_ballot_w64(m_new > m[r]) != 0) {
-                // some row's maximum moved: rescale. Lane holds accumulators of rows 4g..4g+3, whose
-                // factors live in lanes 4g..4g+3.
+            // The reference point m[r] only has to keep the exponentials in range, it need not be the
+            // exact maximum: it is moved (and the accumulators rescaled, ~70 vector instructions) only
+            // when some row's maximum has grown by more than 2^kLazyLog2 since, so probabilities reach at
+            // most that factor above 1. Numerator and denominator carry the same reference, the quotient
+            // is unchanged.
+            if (__builtin_amdgcn_ballot_w64(mx * unit > m[r] * unit + kLazyLog2 || (m[r] == -INFINITY && mx > -INFINITY)) != 0) {
+                // rescale. Lane holds accumulators of rows 4g..4g+3, whose factors live in lanes 4g..4g+3.
                 const float alpha = m_new > m[r] ? fastExp2((m[r] - m_new) * unit) : 1.0f;
                 m[r] = m_new;
 #pragma unroll
