@@ -271,6 +271,337 @@ __global__ void __launch_bounds__(kMlaThreads, 2) decodeMlaKernel(DecodeArgs a) 
     MLA_STAMP(3);
 }
 
+// ---- many query heads per KV head ---------------------------------------------------------------------
+// With more than 32 query heads per KV head the kernel above fetches every K / V tile once per 16 heads
+// (from L2) and each pair of wavefronts moves a whole tile through its own registers. The kernel below
+// gives a workgroup of EIGHT wavefronts 64 query heads of one (partition, sequence): a K / V tile of 32
+// tokens (two halves of 16, each inside one page) is fetched once for all of them and shared through
+// LDS, double-buffered.
+//   * copy: wavefronts 0..3 fetch the V tile, one 128-column quarter each (lane (g, c): token rows
+//     4g..4g+3 of both halves, one 8-column strip), and store it already transposed into matrix-operand
+//     order (per column, the eight tokens of a lane as one 16-byte word); wavefronts 4..7 fetch the K
+//     tile as flat 16-byte chunks (nine load instructions each, every one inside one half) and store it
+//     row-major with a pitch of 73 chunks (conflict-free for both the row-major writes and the
+//     column-of-16-rows reads).
+//   * compute: wavefront w works for head chunk w % 4 (16 heads); the two wavefronts of a chunk split
+//     the 18 K-steps of K . Q^T (9 each, their query slice in registers) and exchange the partial
+//     scores through LDS, run the same softmax, and own 256 value columns each (64 accumulator
+//     registers; P . V as 32-deep matrix instructions). Two workgroup barriers per tile.
+// Partial results and their merge are those of the kernel above.
+constexpr int kMlaWideThreads = 512;
+constexpr int kMlaWideChunks = 4;      // head chunks of 16 per workgroup
+constexpr int kMlaWideTileTokens = 32; // two halves of 16
+
+// Online-softmax step of one 32-token tile. s0 / s1 = raw scores of head c for tokens 4g..4g+3 of the
+// first / second half; the rest as softmaxStep (decode_tiled.h). The probabilities come back as the A
+// operand of a 32-deep matrix instruction whose k index 8g + j stands for token 4g + j of the first
+// half (j < 4) or token 4g + j - 4 of the second.
+template <typename T, int COLS>
+__device__ __forceinline__ void softmaxStepPair(f32x4 (&o)[COLS], float &m, float &l, const f32x4 s0, const f32x4 s1, int g,
+                                                float scale_log2, float slope, int rel_pos0, int valid, uint4 &p_op,
+                                                uint4 &p_lo) {
+    const bool tail = valid < kMlaWideTileTokens;
+    float sc[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int idx = 16 * (i >> 2) + 4 * g + (i & 3);
+        const float raw = i < 4 ? s0[i & 3] : s1[i & 3];
+        sc[i] = raw * scale_log2 + slope * static_cast<float>(rel_pos0 + idx);
+        sc[i] = (tail && idx >= valid) ? -INFINITY : sc[i];
+    }
+    const float mx = maxAcrossTokenGroups(fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])),
+                                                fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7]))));
+    const float m_new = fmaxf(m, mx);
+    if (__builtin_amdgcn_ballot_w64(mx > m + kLazyRescaleLog2) != 0) {
+        // rescale (see softmaxStep). Lane holds accumulators of heads 4g..4g+3, whose factors live in
+        // lanes 4g..4g+3.
+        const float alpha = fastExp2(m - m_new);
+        l *= alpha;
+        m = m_new;
+#pragma unroll
+        for (int rr = 0; rr < 4; ++rr) {
+            const float alpha_r = __shfl(alpha, 4 * g + rr, 64);
+#pragma unroll
+            for (int e = 0; e < COLS; ++e) {
+                o[e][rr] *= alpha_r;
+            }
+        }
+    }
+    uint32_t hi[4], lo[4] = {0, 0, 0, 0};
+    float p_used = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const float pa = fastExp2(sc[2 * i] - m), pb = fastExp2(sc[2 * i + 1] - m);
+        hi[i] = T::pack2(pa, pb);
+        p_used += T::unpackLo(hi[i]) + T::unpackHi(hi[i]);
+        if constexpr (T::kSplitProbabilities) {
+            lo[i] = T::pack2(pa - T::unpackLo(hi[i]), pb - T::unpackHi(hi[i]));
+            p_used += T::unpackLo(lo[i]) + T::unpackHi(lo[i]);
+        }
+    }
+    p_op = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+    p_lo = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+    l += p_used;
+}
+
+template <typename T, typename Tindex>
+__global__ void __launch_bounds__(kMlaWideThreads, 2) decodeMlaWideKernel(DecodeArgs a) {
+    using S = typename T::storage;
+    constexpr int kSteps = kMlaKeySize / 32;        // 18
+    constexpr int kHalfSteps = kSteps / 2;          // K-steps per wavefront
+    constexpr int kChunksPerRow = kMlaKeySize / 8;  // 72 16-byte chunks in a K row
+    constexpr int kPitch = kChunksPerRow + 1;
+    constexpr int kHalfChunks = kTileTokens * kChunksPerRow; // 1152 chunks in a half
+    constexpr int kLoads = 2 * kHalfChunks / 256;            // 9 load instructions per copying wavefront
+    constexpr int kBlocks = kMlaValueSize / 16;              // 32 column blocks of 16
+    __shared__ uint4 k_lds[2][kMlaWideTileTokens * kPitch];
+    __shared__ uint4 v_lds[2][kBlocks * 64];  // [column block][token group g][lane c]: .xy first half, .zw second
+    __shared__ f32x4 s_lds[8][2][64];         // partial scores of every wavefront, both halves
+
+    const int head_chunks = (a.group + kHeadsPerWave - 1) / kHeadsPerWave;
+    const int groups_of_chunks = (head_chunks + kMlaWideChunks - 1) / kMlaWideChunks;
+    const int kv_head = blockIdx.y / groups_of_chunks;
+    const int chunk_group = blockIdx.y - kv_head * groups_of_chunks;
+    const int seq = blockIdx.z;
+    const int part = static_cast<int>((blockIdx.x + blockIdx.z) % gridDim.x); // see decodeMlaKernel
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    const int c = lane & 15;
+    const int g = lane >> 4;
+    const int chunk = chunk_group * kMlaWideChunks + (wave & 3); // may lie beyond the last chunk: no heads
+    const int kh = wave >> 2; // half of the K-steps and half of the value columns
+
+    // Everything up to the first barrier depends on the workgroup only, so all wavefronts leave together.
+    const int64_t len64 = loadIndex<Tindex>(a.seq_lens, seq);
+    if (len64 <= 0) {
+        return;
+    }
+    const int64_t max_len = static_cast<int64_t>(a.max_blocks_per_seq) << a.block_shift;
+    const int len = static_cast<int>(len64 < max_len ? len64 : max_len);
+    const int start = part * a.partition_tokens;
+    if (start >= len) {
+        return;
+    }
+    const int end = min(len, start + a.partition_tokens);
+    const int n_tiles = (end - start + kMlaWideTileTokens - 1) / kMlaWideTileTokens;
+
+    const int first_entry = start >> a.block_shift;
+    const int last_entry = (end - 1) >> a.block_shift;
+    int page_ids = 0;
+    if (first_entry + lane <= last_entry) {
+        page_ids = clampPage(
+            loadIndex<Tindex>(a.block_tables, seq * a.block_table_batch_stride + first_entry + lane), a.num_blocks);
+    }
+
+    // Query of head (chunk*16 + c): columns 288 kh + 32 i + 8g .. +7, the B operand of this wavefront's K-steps
+    const int head_in_group = chunk * kHeadsPerWave + c;
+    const bool head_valid = head_in_group < a.group;
+    const int head = kv_head * a.group + head_in_group;
+    uint4 q_reg[kHalfSteps];
+    {
+        const S *q_ptr = static_cast<const S *>(a.q) + seq * a.q_stride + (head_valid ? head : 0) * a.q_head_stride
+                       + kh * (kMlaKeySize / 2);
+        const uint32_t keep = head_valid ? 0xffffffffu : 0u;
+#pragma unroll
+        for (int i = 0; i < kHalfSteps; ++i) {
+            uint4 x = *reinterpret_cast<const uint4 *>(q_ptr + 32 * i + 8 * g);
+            x.x &= keep, x.y &= keep, x.z &= keep, x.w &= keep;
+            q_reg[i] = x;
+        }
+    }
+    const float slope = (a.alibi_slopes != nullptr && head_valid) ? a.alibi_slopes[head] * kLog2e : 0.0f;
+
+    // ---- copy side: one code path for both roles (the V wavefronts' ninth load repeats their first) ----
+    const bool copies_v = wave < 4;
+    const int role_wave = wave & 3;
+    const char *copy_head = copies_v
+        ? reinterpret_cast<const char *>(static_cast<const S *>(a.v_cache) + kv_head * a.v_head_stride)
+        : reinterpret_cast<const char *>(static_cast<const S *>(a.k_cache) + kv_head * a.k_head_stride);
+    const int64_t copy_batch_stride = copies_v ? a.v_batch_stride : a.k_batch_stride;
+    const int64_t copy_row_stride = copies_v ? a.v_row_stride : a.k_row_stride;
+    const int block_mask = a.block_size - 1;
+    // Load j of a wavefront: which half of the tile (wave-uniform), this lane's byte offset inside the
+    // half, and for K where the chunk goes in LDS.
+    //   V: j = 4 h + i: token row 4g + i of half h, columns 128 role_wave + 8 c .. + 7
+    //   K: wave-instruction 4 j + role_wave of 36; 18 per half, 64 consecutive chunks each
+    uint32_t src_off[kLoads];
+    int k_dst[kLoads];
+#pragma unroll
+    for (int j = 0; j < kLoads; ++j) {
+        if (copies_v) {
+            const int i = j & 3;
+            src_off[j] = (4 * g + i) * static_cast<uint32_t>(a.v_row_stride) * sizeof(S) + 256 * role_wave + 16 * c;
+            k_dst[j] = 0;
+        } else {
+            const int inst = 4 * j + role_wave;
+            const int ch = 64 * (inst % 18) + lane; // chunk within the half
+            const int row = ch / kChunksPerRow, col = ch - row * kChunksPerRow;
+            src_off[j] = row * static_cast<uint32_t>(a.k_row_stride) * sizeof(S) + 16 * col;
+            k_dst[j] = (16 * (inst / 18) + row) * kPitch + col;
+        }
+    }
+    auto halfOfLoad = [&](int j) { return copies_v ? ((j >> 2) & 1) : ((4 * j + role_wave) / 18); };
+
+    uint4 stage[kLoads];
+#pragma unroll
+    for (int j = 0; j < kLoads; ++j) {
+        stage[j] = make_uint4(0, 0, 0, 0);
+    }
+    // Loads for a half past the end of the partition are issued all the same but read the partition's
+    // first rows (the loop body has no branch around a load).
+    auto loadStage = [&](int t) {
+        const char *half_base[2];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            int tok0 = start + t * kMlaWideTileTokens + 16 * h;
+            tok0 = tok0 < end ? tok0 : start;
+            const int page = __builtin_amdgcn_readlane(page_ids, (tok0 >> a.block_shift) - first_entry);
+            const int row0 = tok0 & block_mask;
+            half_base[h] = copy_head + (page * copy_batch_stride + row0 * copy_row_stride) * static_cast<int64_t>(sizeof(S));
+        }
+#pragma unroll
+        for (int j = 0; j < kLoads; ++j) {
+            stage[j] = loadLane16(halfOfLoad(j) ? half_base[1] : half_base[0], src_off[j]);
+        }
+    };
+    auto storeStage = [&](int t) {
+        const int buf = t & 1;
+        if (copies_v) {
+            // V rows beyond the sequence may hold anything (NaN included) and 0 * NaN is NaN: zeroed here
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const int valid = end - (start + t * kMlaWideTileTokens + 16 * h);
+                uint32_t r[4][4]; // [token row i][dword]
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const bool keep = 4 * g + i < valid;
+                    r[i][0] = keep ? stage[4 * h + i].x : 0u;
+                    r[i][1] = keep ? stage[4 * h + i].y : 0u;
+                    r[i][2] = keep ? stage[4 * h + i].z : 0u;
+                    r[i][3] = keep ? stage[4 * h + i].w : 0u;
+                }
+#pragma unroll
+                for (int wd = 0; wd < 4; ++wd) {
+                    uint2 even, odd;
+                    even.x = __builtin_amdgcn_perm(r[1][wd], r[0][wd], 0x05040100u);
+                    even.y = __builtin_amdgcn_perm(r[3][wd], r[2][wd], 0x05040100u);
+                    odd.x = __builtin_amdgcn_perm(r[1][wd], r[0][wd], 0x07060302u);
+                    odd.y = __builtin_amdgcn_perm(r[3][wd], r[2][wd], 0x07060302u);
+                    // column 128 role_wave + 8 c + 2 wd (+1) -> block 8 role_wave + 2 wd (+1), lane c
+                    uint2 *dst_even = reinterpret_cast<uint2 *>(&v_lds[buf][((8 * role_wave + 2 * wd) * 4 + g) * 16 + c]) + h;
+                    uint2 *dst_odd = reinterpret_cast<uint2 *>(&v_lds[buf][((8 * role_wave + 2 * wd + 1) * 4 + g) * 16 + c]) + h;
+                    *dst_even = even;
+                    *dst_odd = odd;
+                }
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < kLoads; ++j) {
+                k_lds[buf][k_dst[j]] = stage[j];
+            }
+        }
+    };
+
+    // o[e][r] = O[head 4g + r of the chunk][column 256 kh + 128 (e / 8) + 8 c + e % 8]
+    f32x4 o[16];
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+        o[e] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    float m = -INFINITY; // reference point of head c's exponentials (same value in the four lanes g = 0..3)
+    float l = 0.0f;      // sum of rounded probabilities of head c over this lane's tokens only
+
+    loadStage(0);
+    storeStage(0);
+    loadStage(1);
+    for (int t = 0; t < n_tiles; ++t) {
+        const int buf = t & 1;
+        __syncthreads(); // tile t is complete in LDS, and everybody has finished with tile t - 1
+        if (t + 1 < n_tiles) {
+            storeStage(t + 1);
+        }
+        loadStage(t + 2);
+        // partial scores of both halves over this wavefront's K-steps: four independent chains (a matrix
+        // instruction that accumulates into the result of the previous one waits ~44 cycles for it, an
+        // independent one issues after 16)
+        f32x4 sp[2][2] = {{{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}}, {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}}};
+#pragma unroll
+        for (int i = 0; i < kHalfSteps; ++i) {
+            const int kk = kh * kHalfSteps + i;
+            sp[0][i & 1] = T::mfmaK32(k_lds[buf][c * kPitch + 4 * kk + g], q_reg[i], sp[0][i & 1]);
+            sp[1][i & 1] = T::mfmaK32(k_lds[buf][(16 + c) * kPitch + 4 * kk + g], q_reg[i], sp[1][i & 1]);
+        }
+        f32x4 s0 = sp[0][0] + sp[0][1], s1 = sp[1][0] + sp[1][1];
+        s_lds[wave][0][lane] = s0;
+        s_lds[wave][1][lane] = s1;
+        __syncthreads(); // partial scores of both K halves are there
+        s0 += s_lds[wave ^ 4][0][lane];
+        s1 += s_lds[wave ^ 4][1][lane];
+
+        const int tok0 = start + t * kMlaWideTileTokens;
+        const int valid = min(kMlaWideTileTokens, end - tok0);
+        uint4 p_op, p_lo;
+        softmaxStepPair<T, 16>(o, m, l, s0, s1, g, a.scale_log2, slope, tok0 - (len - 1), valid, p_op, p_lo);
+        // all sixteen column blocks with the high parts first, then with the low parts (independent chains)
+        uint4 vf[16];
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            vf[e] = v_lds[buf][((16 * kh + e) * 4 + g) * 16 + c];
+        }
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            o[e] = T::mfmaK32(p_op, vf[e], o[e]);
+        }
+        if constexpr (T::kSplitProbabilities) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                o[e] = T::mfmaK32(p_lo, vf[e], o[e]);
+            }
+        }
+    }
+
+    // Epilogue, as in decodeMlaKernel
+    const float l_tot = sumAcrossTokenGroups(l);
+    const bool single = len <= a.partition_tokens;
+#pragma unroll
+    for (int rr = 0; rr < 4; ++rr) {
+        const int hl = 4 * g + rr; // head (within the chunk) of accumulator row rr
+        const float l_h = __shfl(l_tot, hl, 64);
+        const float m_h = __shfl(m, hl, 64);
+        const int hg = chunk * kHeadsPerWave + hl;
+        if (hg >= a.group) {
+            continue;
+        }
+        const int out_head = kv_head * a.group + hg;
+        const int col0 = 256 * kh + 8 * c;
+        if (single) {
+            const float inv_l = 1.0f / (l_h + 1e-6f);
+            S *o_ptr = static_cast<S *>(a.out) + seq * a.o_stride + out_head * a.o_head_stride + col0;
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                uint4 w;
+                w.x = T::pack2(o[8 * i + 0][rr] * inv_l, o[8 * i + 1][rr] * inv_l);
+                w.y = T::pack2(o[8 * i + 2][rr] * inv_l, o[8 * i + 3][rr] * inv_l);
+                w.z = T::pack2(o[8 * i + 4][rr] * inv_l, o[8 * i + 5][rr] * inv_l);
+                w.w = T::pack2(o[8 * i + 6][rr] * inv_l, o[8 * i + 7][rr] * inv_l);
+                *reinterpret_cast<uint4 *>(o_ptr + 128 * i) = w;
+            }
+        } else {
+            const int64_t slot = (static_cast<int64_t>(seq) * a.num_heads + out_head) * a.max_partitions + part;
+            float *dst = a.part_acc + slot * kMlaValueSize + col0;
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                reinterpret_cast<float4 *>(dst + 128 * i)[0] = make_float4(o[8 * i + 0][rr], o[8 * i + 1][rr], o[8 * i + 2][rr], o[8 * i + 3][rr]);
+                reinterpret_cast<float4 *>(dst + 128 * i)[1] = make_float4(o[8 * i + 4][rr], o[8 * i + 5][rr], o[8 * i + 6][rr], o[8 * i + 7][rr]);
+            }
+            if (c == 0 && kh == 0) {
+                a.part_m[slot] = m_h;
+                a.part_l[slot] = l_h;
+            }
+        }
+    }
+}
+
 } // namespace op::paged_attention::amd
 
 #endif

@@ -24,6 +24,7 @@ namespace {
 struct Plan {
     bool tiled;            // tiled matrix-core kernel (head 64 / 128 / 192 / 256 or 576 with values of 512, power-of-two pages >= 16, 16-byte aligned strides)
     bool balanced;         // tiled kernel under the work-equalising schedule (decode_balanced.h)
+    bool latent_wide;      // latent attention with more than 32 query heads per KV head: 64 heads per workgroup
     int partition_tokens;  // grid schedule: tokens per unit of work
     int max_partitions;    // grid schedule: partitions the longest representable sequence needs
     int dims_per_lane;     // element-wise kernel: ceil(max(head_size, value_size) / 64)
@@ -85,11 +86,27 @@ Plan makePlan(const PagedAttentionInfo &in, const device::amd::DeviceInfo &dev) 
     // A unit of the latent-attention kernel leaves 32 KiB of partial results and advances one tile per
     // ~2 us however many units there are: fewer, longer units measured best there (more units end the
     // decode kernel sooner, but writing and merging their partial results costs more than that gains).
-    long long want = latent_head ? units * max_tokens * 3 / (16LL * dev.compute_units)
-                   : small_job   ? units * max_tokens / (8LL * dev.compute_units)
-                                 : units * max_tokens / (16LL * dev.compute_units);
+    // Latent attention with more than two 16-head chunks per KV head runs 64 heads per workgroup
+    // (measured against the 16-head units: 32 heads 61.5 vs 62.0 us, 48 heads 65.7 vs 82.3, 64 heads
+    // 67.5 vs 104.2, 128 heads 122 vs 165; 128 sequences of 128 heads 368 vs 708). One workgroup per
+    // compute unit there, 128 KiB of partial results each: about one round of workgroups measured best.
+    const long long head_chunks = (group + kHeadsPerWave - 1) / kHeadsPerWave;
+    plan.latent_wide = plan.tiled && latent_head && head_chunks > 2;
+    if (const char *env = std::getenv("INFINIOP_AMD_PA_LATENT_KERNEL")) {
+        if (std::strcmp(env, "wide") == 0) {
+            plan.latent_wide = plan.tiled && latent_head;
+        } else if (std::strcmp(env, "narrow") == 0) {
+            plan.latent_wide = false;
+        }
+    }
+    const long long wide_units = static_cast<long long>(in.num_seqs) * in.num_kv_heads
+                               * ((head_chunks + kMlaWideChunks - 1) / kMlaWideChunks);
+    long long want = plan.latent_wide ? wide_units * max_tokens / dev.compute_units
+                   : latent_head      ? units * max_tokens * 3 / (16LL * dev.compute_units)
+                   : small_job        ? units * max_tokens / (8LL * dev.compute_units)
+                                      : units * max_tokens / (16LL * dev.compute_units);
     int p = floorPow2(want < 1 ? 1 : want);
-    const int p_min = latent_head ? 256 : 64;
+    const int p_min = plan.latent_wide ? 128 : (latent_head ? 256 : 64);
     p = p < p_min ? p_min : (p > 512 ? 512 : p);
     if (const char *env = std::getenv("INFINIOP_AMD_PA_PARTITION")) {
         const int forced = std::atoi(env);
@@ -196,6 +213,12 @@ void launchAll(const DecodeArgs &a, const Plan &plan, bool tiled, hipStream_t st
         default: {
             const int head_chunks = (a.group + kHeadsPerWave - 1) / kHeadsPerWave;
             const dim3 grid(plan.max_partitions, a.num_kv_heads * head_chunks, a.num_seqs);
+            if (plan.latent_wide) {
+                const int groups_of_chunks = (head_chunks + kMlaWideChunks - 1) / kMlaWideChunks;
+                const dim3 wide(plan.max_partitions, a.num_kv_heads * groups_of_chunks, a.num_seqs);
+                decodeMlaWideKernel<T, Tindex><<<wide, kMlaWideThreads, 0, stream>>>(a);
+                break;
+            }
             decodeMlaKernel<T, Tindex><<<grid, kMlaThreads, 0, stream>>>(a);
             break;
         }

@@ -216,12 +216,21 @@ def mla(name, dtype, B, H, bs, lo, hi, seed, **kw):
     return workloads.DecodeConfig(name, dtype, B, H, 1, 576, bs, lo, hi, seed=seed, value_size=512, **kw)
 
 
+@pytest.fixture(params=[None, "narrow", "wide"], ids=["auto", "narrow", "wide"])
+def latent_kernel(request, monkeypatch):
+    """The two latent-attention kernels: 16 query heads per workgroup of two wavefronts ("narrow"), 64 per
+    workgroup of eight ("wide"); left alone, more than 32 heads per KV head take the wide one."""
+    if request.param:
+        monkeypatch.setenv("INFINIOP_AMD_PA_LATENT_KERNEL", request.param)
+    return request.param
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("H", [16, 128, 20, 48, 80])
-def test_mla_ragged_batches(gpu_handle, oracle, dtype, H):
+def test_mla_ragged_batches(gpu_handle, oracle, dtype, H, latent_kernel):
     """Ragged lengths incl. 1 token and exactly one page, long enough that sequences are split into
-    partitions and merged; 16 heads (one chunk of 16 per workgroup), 20 (two chunks, one partly filled), 48
-    (three chunks in workgroups of two: one workgroup slot without heads), 80 (five in workgroups of four) and
+    partitions and merged; 16 heads (one chunk of 16), 20 (two chunks, one partly filled), 48 (three: a wide
+    workgroup with one slot without heads), 80 (five: two wide workgroups, the second with one chunk) and
     128 (eight)."""
     inp = workloads.make_decode_inputs(mla(f"mla_h{H}", dtype, 5, H, 16, 1, 2500, seed=400 + H))
     inp.seq_lens[0], inp.seq_lens[1] = 1, 16
@@ -230,12 +239,15 @@ def test_mla_ragged_batches(gpu_handle, oracle, dtype, H):
 
 
 @pytest.mark.parametrize("partition", [16, 48, 1024])
-def test_mla_partition_sizes(gpu_handle, oracle, monkeypatch, partition):
+def test_mla_partition_sizes(gpu_handle, oracle, monkeypatch, partition, latent_kernel):
+    """Partitions of one 16-token half tile, of one and a half 32-token tiles, and of the most one page-id
+    load covers."""
     monkeypatch.setenv("INFINIOP_AMD_PA_PARTITION", str(partition))
-    run_case(gpu_handle, oracle, workloads.make_decode_inputs(mla(f"mla_p{partition}", torch.bfloat16, 3, 16, 16, 1, 1200, seed=410)))
+    H = 48 if latent_kernel == "wide" else 16
+    run_case(gpu_handle, oracle, workloads.make_decode_inputs(mla(f"mla_p{partition}", torch.bfloat16, 3, H, 16, 1, 1200, seed=410)))
 
 
-def test_mla_matches_the_elementwise_kernel_in_layout(gpu_handle):
+def test_mla_matches_the_elementwise_kernel_in_layout(gpu_handle, latent_kernel):
     """Every output column lands where the element-wise kernel puts it: V with a distinct constant per
     column makes the expected output that constant, whatever the softmax does. Short sequences (written by the
     decode kernel) and long ones (merged from partitions)."""
@@ -248,7 +260,7 @@ def test_mla_matches_the_elementwise_kernel_in_layout(gpu_handle):
     assert torch.allclose(got, want, atol=2e-3 * float(ramp.abs().max()), rtol=0), (got - want).abs().max()
 
 
-def test_mla_alibi_pages_of_64_and_int32_indices(gpu_handle, oracle):
+def test_mla_alibi_pages_of_64_and_int32_indices(gpu_handle, oracle, latent_kernel):
     inp = workloads.make_decode_inputs(mla("mla_mix", torch.bfloat16, 4, 32, 64, 1, 1500, seed=430))
     slopes = torch.tensor([2.0 ** (-(i % 8 + 1)) for i in range(32)], dtype=torch.float32)
     q, k, v, bt, sl = to_device(inp)
@@ -257,7 +269,7 @@ def test_mla_alibi_pages_of_64_and_int32_indices(gpu_handle, oracle):
     assert_close(got, want, "mla_mix", want_f32)
 
 
-def test_mla_ignores_garbage_beyond_the_sequences(gpu_handle, oracle):
+def test_mla_ignores_garbage_beyond_the_sequences(gpu_handle, oracle, latent_kernel):
     inp = workloads.make_decode_inputs(mla("mla_poison", torch.float16, 4, 16, 16, 1, 600, seed=440))
     want = oracle_of(oracle, inp)
     k, v = inp.k_cache.clone(), inp.v_cache.clone()
@@ -272,7 +284,7 @@ def test_mla_ignores_garbage_beyond_the_sequences(gpu_handle, oracle):
     assert_close(got, want, "mla_poison")
 
 
-def test_mla_padded_cache_rows(gpu_handle, oracle):
+def test_mla_padded_cache_rows(gpu_handle, oracle, latent_kernel):
     """K and V rows that are not packed (views into wider pools): row strides of 640 and 576 elements."""
     inp = workloads.make_decode_inputs(mla("mla_strided", torch.bfloat16, 3, 16, 16, 1, 900, seed=450))
     nb = inp.k_cache.shape[0]
@@ -286,8 +298,9 @@ def test_mla_padded_cache_rows(gpu_handle, oracle):
     assert_close(got, want, "mla_strided", want_f32)
 
 
-def test_mla_full_size_against_oracle(gpu_handle, oracle):
-    run_case(gpu_handle, oracle, workloads.make_decode_inputs(workloads.DECODE_CONFIGS["m1_mla_16_heads_b32"]))
+@pytest.mark.parametrize("workload", ["m1_mla_16_heads_b32", "m2_mla_128_heads_b32"])
+def test_mla_full_size_against_oracle(gpu_handle, oracle, workload):
+    run_case(gpu_handle, oracle, workloads.make_decode_inputs(workloads.DECODE_CONFIGS[workload]))
 
 
 @pytest.mark.parametrize("B,lo,hi", [(1, 2100, 2100), (4, 512, 4096), (16, 512, 4096)])
@@ -310,6 +323,47 @@ def test_kernels_and_schedules_agree_with_oracle(gpu_handle, oracle, monkeypatch
     cfg = custom(f"ragged_{kernel}_{schedule}", dtype, 6, 32, 8, 128, 16, 1, 3000, seed=5)
     inp = workloads.make_decode_inputs(cfg)
     inp.seq_lens[0], inp.seq_lens[1] = 1, 16  # shortest possible and exactly one page
+    run_case(gpu_handle, oracle, inp)
+
+
+def climbing_keys(inp, step_log2=0.25, jump_every=200, jump_log2=12.0):
+    """Overwrites K so that the scores of every query head climb along the sequence: by step_log2 (in
+    powers of two of the softmax weight) per token, plus jump_log2 at every jump_every-th token. The
+    running maximum then moves in every tile, by less than a tile's rescaling threshold most of the time
+    and by much more at the jumps."""
+    cfg = inp.config
+    rng = np.random.default_rng(cfg.seed + 1)
+    direction = torch.from_numpy(rng.standard_normal((cfg.num_kv_heads, cfg.head_size)).astype(np.float32))
+    direction /= direction.norm(dim=1, keepdim=True)
+    group = cfg.num_heads // cfg.num_kv_heads
+    # every query head points along its KV head's direction: score = |q| * a(t) * scale
+    q_norm = 4.0
+    inp.q[:] = (direction.repeat_interleave(group, dim=0)[None] * q_norm).to(cfg.dtype).expand_as(inp.q)
+    per_unit = q_norm * inp.scale * 1.4426950408889634  # log2 of the weight per unit of a(t)
+    for s in range(cfg.num_seqs):
+        n = int(inp.seq_lens[s])
+        t = torch.arange(n, dtype=torch.float32)
+        a = (step_log2 * t + jump_log2 * torch.floor(t / jump_every)) / per_unit
+        a -= a.mean()
+        rows = a[:, None, None] * direction[None] + 0.05 * torch.from_numpy(
+            rng.standard_normal((n, cfg.num_kv_heads, cfg.head_size)).astype(np.float32))
+        pages = inp.block_tables[s, torch.arange(n) // cfg.block_size]
+        inp.k_cache[pages, :, torch.arange(n) % cfg.block_size] = rows.to(cfg.dtype)
+    return inp
+
+
+@pytest.mark.parametrize("schedule", [None, "grid"])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_scores_that_climb_along_the_sequence(gpu_handle, oracle, monkeypatch, dtype, schedule):
+    if schedule:
+        monkeypatch.setenv("INFINIOP_AMD_PA_SCHEDULE", schedule)
+    inp = climbing_keys(workloads.make_decode_inputs(custom(f"climb_{schedule}", dtype, 4, 32, 8, 128, 16, 300, 1500, seed=71)))
+    run_case(gpu_handle, oracle, inp)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_mla_scores_that_climb_along_the_sequence(gpu_handle, oracle, dtype, latent_kernel):
+    inp = climbing_keys(workloads.make_decode_inputs(mla("mla_climb", dtype, 3, 16, 16, 300, 1200, seed=72)))
     run_case(gpu_handle, oracle, inp)
 
 

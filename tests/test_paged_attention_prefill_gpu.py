@@ -13,7 +13,7 @@ import torch
 from infinicore_amd import workloads
 
 from capi import run_paged_attention_prefill
-from test_paged_attention_gpu import DEV, ORACLE_THREADS, assert_close
+from test_paged_attention_gpu import DEV, ORACLE_THREADS, assert_close, climbing_keys
 
 pytestmark = pytest.mark.gpu
 
@@ -122,6 +122,22 @@ def test_every_row_block_size_of_the_tiled_kernel(gpu_handle, oracle, monkeypatc
     monkeypatch.setenv("INFINIOP_AMD_PREFILL_GROUPS", groups)
     cfg = prefill_config(f"groups{groups}", dtype, 5, 16, 4, 128, 16, (1, 300), (0, 500), seed=31)
     run_case(gpu_handle, oracle, workloads.make_prefill_inputs(cfg))
+
+
+@pytest.mark.parametrize("groups", ["1", "2"])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_scores_that_climb_along_the_sequence(gpu_handle, oracle, monkeypatch, groups, dtype):
+    """Every row's running maximum moves in every step, mostly by less than the rescaling threshold and
+    at the jumps by much more (the keys are laid out by test_paged_attention_gpu.climbing_keys)."""
+    monkeypatch.setenv("INFINIOP_AMD_PREFILL_GROUPS", groups)
+    cfg = prefill_config(f"climb{groups}", dtype, 3, 16, 4, 128, 16, (100, 400), (0, 700), seed=73)
+    inp = workloads.make_prefill_inputs(cfg)
+    q = inp.q.clone()
+    climbing_keys(inp, step_log2=0.05, jump_every=150, jump_log2=12.0)
+    # keep distinct queries per token (same direction, different lengths), so rows differ
+    scale_rows = torch.linspace(0.5, 1.5, q.shape[0])[:, None, None]
+    inp.q[:] = (inp.q.float() * scale_rows).to(cfg.dtype)
+    run_case(gpu_handle, oracle, inp)
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
