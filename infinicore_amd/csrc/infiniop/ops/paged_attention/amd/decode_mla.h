@@ -1,6 +1,9 @@
-// Tiled decode kernel for latent-attention caches: head_size 576 (512 latent + 64 rotary columns),
+// Tiled decode kernels for latent-attention caches: head_size 576 (512 latent + 64 rotary columns),
 // value_size 512, the shape of the reference's dedicated kernel
 // (src/infiniop/ops/paged_attention/nvidia/paged_attention_mla_hd576_v512.cu). gfx950, 64-lane wavefronts.
+// Two kernels: decodeMlaKernel (16 query heads per workgroup of two wavefronts, described first) and
+// decodeMlaWideKernel (64 query heads per workgroup of eight, for more than 32 heads per KV head; further
+// down).
 //
 // Unit of work and arithmetic are those of the head-128 tiled kernel (decode_tiled.h): one unit = one
 // (partition, KV head x 16 query heads, sequence), tiles of 16 tokens, K . Q^T and P . V on the matrix
