@@ -303,14 +303,23 @@ template <typename T, int COLS>
 __device__ __forceinline__ void softmaxStepPair(f32x4 (&o)[COLS], float &m, float &l, const f32x4 s0, const f32x4 s1, int g,
                                                 float scale_log2, float slope, int rel_pos0, int valid, uint4 &p_op,
                                                 uint4 &p_lo) {
-    const bool tail = valid < kMlaWideTileTokens;
     float sc[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-        const int idx = 16 * (i >> 2) + 4 * g + (i & 3);
-        const float raw = i < 4 ? s0[i & 3] : s1[i & 3];
-        sc[i] = raw * scale_log2 + slope * static_cast<float>(rel_pos0 + idx);
-        sc[i] = (tail && idx >= valid) ? -INFINITY : sc[i];
+        sc[i] = (i < 4 ? s0[i & 3] : s1[i & 3]) * scale_log2;
+    }
+    // wave-uniform branches: ALiBi is rare, and only the last tile of a partition can be short
+    if (__builtin_amdgcn_ballot_w64(slope != 0.0f) != 0) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            sc[i] += slope * static_cast<float>(rel_pos0 + 16 * (i >> 2) + 4 * g + (i & 3));
+        }
+    }
+    if (valid < kMlaWideTileTokens) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            sc[i] = (16 * (i >> 2) + 4 * g + (i & 3) >= valid) ? -INFINITY : sc[i];
+        }
     }
     const float mx = maxAcrossTokenGroups(fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])),
                                                 fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7]))));
@@ -471,17 +480,23 @@ __global__ void __launch_bounds__(kMlaWideThreads, 2) decodeMlaWideKernel(Decode
         const int buf = t & 1;
         if (copies_v) {
             // V rows beyond the sequence may hold anything (NaN included) and 0 * NaN is NaN: zeroed here
+            const bool full_tile = end - (start + t * kMlaWideTileTokens) >= kMlaWideTileTokens;
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
                 const int valid = end - (start + t * kMlaWideTileTokens + 16 * h);
                 uint32_t r[4][4]; // [token row i][dword]
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    const bool keep = 4 * g + i < valid;
-                    r[i][0] = keep ? stage[4 * h + i].x : 0u;
-                    r[i][1] = keep ? stage[4 * h + i].y : 0u;
-                    r[i][2] = keep ? stage[4 * h + i].z : 0u;
-                    r[i][3] = keep ? stage[4 * h + i].w : 0u;
+                    r[i][0] = stage[4 * h + i].x, r[i][1] = stage[4 * h + i].y;
+                    r[i][2] = stage[4 * h + i].z, r[i][3] = stage[4 * h + i].w;
+                }
+                if (!full_tile) { // only the last tile of a partition can be short
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        if (4 * g + i >= valid) {
+                            r[i][0] = r[i][1] = r[i][2] = r[i][3] = 0u;
+                        }
+                    }
                 }
 #pragma unroll
                 for (int wd = 0; wd < 4; ++wd) {
