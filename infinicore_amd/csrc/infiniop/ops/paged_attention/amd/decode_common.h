@@ -32,6 +32,9 @@ struct DecodeArgs {
     float *part_m;
     float *part_l;
     int2 *seq_pieces; // work-equalising schedule only: per sequence {first piece, number of pieces}
+    // 64-head latent-attention kernel only: the partition size the decode kernel settled on for this
+    // call (>= partition_tokens), written by its first workgroup for the merge kernel; else nullptr
+    int32_t *chosen_partition;
 
     float scale_log2; // scale * log2(e)
     int32_t num_seqs;
@@ -46,6 +49,7 @@ struct DecodeArgs {
     int32_t max_blocks_per_seq;
     int32_t partition_tokens;
     int32_t max_partitions;
+    int32_t compute_units; // of the device the call runs on
 
     // element strides
     int64_t q_stride, q_head_stride;

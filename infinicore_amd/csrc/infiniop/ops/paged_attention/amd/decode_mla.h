@@ -356,6 +356,84 @@ __device__ __forceinline__ void softmaxStepPair(f32x4 (&o)[COLS], float &m, floa
     l += p_used;
 }
 
+// One workgroup per compute unit, 32 compute units per accelerator die, workgroups dealt to the eight dies
+// round-robin by linear id: 280 workgroups take as long as 512, and so do 230 if one die gets 33 of them.
+// Batches of up to 256 sequences are therefore planned by every workgroup for itself from the actual
+// lengths (the host only knows the width of the block table); same inputs, same answer in every wavefront,
+// no LDS, no barrier:
+//   * partition size of the call: among the planned size and larger ones, in steps of 64 tokens up to what
+//     one page-id load covers (64 pages) or 1024 tokens, the one that needs the fewest tiles in a row,
+//     i.e. (rounds of workgroups) x (tiles per partition); ties go to the larger size (fewer partial
+//     results);
+//   * the (sequence, partition) units are numbered densely; linear workgroup id = 8 streams (u / 8) +
+//     8 stream + u % 8, so the units that exist come first, the dies get equal shares, and the workgroups
+//     of one unit (one per 64 heads) sit on the same die and meet in its L2.
+struct WidePlan {
+    int partition_tokens;
+    int seq, part, stream; // this workgroup's unit; seq < 0: none
+};
+
+template <typename Tindex>
+__device__ __forceinline__ WidePlan planWide(const DecodeArgs &a, int lane, int streams, int linear_id) {
+    WidePlan plan{a.partition_tokens, -1, 0, 0};
+    const int64_t max_len = static_cast<int64_t>(a.max_blocks_per_seq) << a.block_shift;
+    int lens[4]; // the lengths once, up to four per lane (one round of independent loads)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        int64_t len = 0;
+        if (64 * i + lane < a.num_seqs) {
+            len = loadIndex<Tindex>(a.seq_lens, 64 * i + lane);
+            len = len < 0 ? 0 : (len < max_len ? len : max_len);
+        }
+        lens[i] = static_cast<int>(len);
+    }
+    const int cap = min(64 << a.block_shift, 1024);
+    int best_cost = 0x7fffffff;
+    for (int p = a.partition_tokens; p <= cap || p == a.partition_tokens; p += 64) {
+        // partitions of this lane's sequences: ceil(len / p) through the reciprocal, corrected to be exact
+        // (lengths above 2^24 are rounded, which only blunts the estimate)
+        const float pf = static_cast<float>(p), inv = 1.0f / pf;
+        int x = 0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float lf = static_cast<float>(lens[i]);
+            float q = floorf(lf * inv);
+            q = q * pf > lf ? q - 1.0f : q;          // one too many
+            q = (q + 1.0f) * pf <= lf ? q + 1.0f : q; // one too few
+            x += static_cast<int>(q) + (q * pf < lf ? 1 : 0);
+        }
+        const int workgroups = __builtin_amdgcn_readlane(waveInclusiveSum(x), 63) * streams;
+        const int rounds = (workgroups + a.compute_units - 1) / a.compute_units;
+        const int cost = rounds * ((p + kMlaWideTileTokens - 1) / kMlaWideTileTokens);
+        if (cost <= best_cost) {
+            best_cost = cost;
+            plan.partition_tokens = p;
+        }
+        if (rounds <= 1 && p == a.partition_tokens) {
+            break; // everything runs at once at the planned size: larger partitions only take longer
+        }
+    }
+    // dense unit of this workgroup
+    const int p = plan.partition_tokens;
+    const int group_of_8 = linear_id / (8 * streams), rest = linear_id - group_of_8 * (8 * streams);
+    plan.stream = rest >> 3;
+    const int u = 8 * group_of_8 + (rest & 7);
+    int running = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int k = (lens[i] + p - 1) / p;
+        const int incl = waveInclusiveSum(k) + running;
+        const unsigned long long hit = __builtin_amdgcn_ballot_w64(incl > u);
+        if (hit != 0 && plan.seq < 0) {
+            const int first = __builtin_ctzll(hit);
+            plan.seq = 64 * i + first;
+            plan.part = u - (__builtin_amdgcn_readlane(incl, first) - __builtin_amdgcn_readlane(k, first));
+        }
+        running = __builtin_amdgcn_readlane(incl, 63);
+    }
+    return plan;
+}
+
 template <typename T, typename Tindex>
 __global__ void __launch_bounds__(kMlaWideThreads, 2) decodeMlaWideKernel(DecodeArgs a) {
     using S = typename T::storage;
@@ -372,29 +450,48 @@ __global__ void __launch_bounds__(kMlaWideThreads, 2) decodeMlaWideKernel(Decode
 
     const int head_chunks = (a.group + kHeadsPerWave - 1) / kHeadsPerWave;
     const int groups_of_chunks = (head_chunks + kMlaWideChunks - 1) / kMlaWideChunks;
-    const int kv_head = blockIdx.y / groups_of_chunks;
-    const int chunk_group = blockIdx.y - kv_head * groups_of_chunks;
-    const int seq = blockIdx.z;
-    const int part = static_cast<int>((blockIdx.x + blockIdx.z) % gridDim.x); // see decodeMlaKernel
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int lane = threadIdx.x & 63;
     const int c = lane & 15;
     const int g = lane >> 4;
+
+    // Which (sequence, partition, KV head x group of four head chunks) this workgroup works on. Everything
+    // up to the first barrier depends on the workgroup only, so all wavefronts leave together.
+    int seq, part, stream, partition_tokens;
+    if (a.chosen_partition != nullptr) {
+        // planned per call (see planWide): one-dimensional grid
+        const WidePlan plan = planWide<Tindex>(a, lane, a.num_kv_heads * groups_of_chunks, static_cast<int>(blockIdx.x));
+        if (blockIdx.x == 0 && threadIdx.x == 0) {
+            a.chosen_partition[0] = plan.partition_tokens; // for the merge kernel
+        }
+        if (plan.seq < 0) {
+            return;
+        }
+        // wave-uniform by construction; saying so keeps the address arithmetic in scalar registers
+        seq = __builtin_amdgcn_readfirstlane(plan.seq);
+        part = __builtin_amdgcn_readfirstlane(plan.part);
+        stream = __builtin_amdgcn_readfirstlane(plan.stream);
+        partition_tokens = __builtin_amdgcn_readfirstlane(plan.partition_tokens);
+    } else {
+        // fixed partitions on a three-dimensional grid, rotated as in decodeMlaKernel
+        seq = blockIdx.z;
+        part = static_cast<int>((blockIdx.x + blockIdx.z) % gridDim.x);
+        stream = blockIdx.y;
+        partition_tokens = a.partition_tokens;
+    }
+    const int kv_head = stream / groups_of_chunks;
+    const int chunk_group = stream - kv_head * groups_of_chunks;
     const int chunk = chunk_group * kMlaWideChunks + (wave & 3); // may lie beyond the last chunk: no heads
     const int kh = wave >> 2; // half of the K-steps and half of the value columns
 
-    // Everything up to the first barrier depends on the workgroup only, so all wavefronts leave together.
     const int64_t len64 = loadIndex<Tindex>(a.seq_lens, seq);
-    if (len64 <= 0) {
-        return;
-    }
     const int64_t max_len = static_cast<int64_t>(a.max_blocks_per_seq) << a.block_shift;
     const int len = static_cast<int>(len64 < max_len ? len64 : max_len);
-    const int start = part * a.partition_tokens;
-    if (start >= len) {
+    const int start = part * partition_tokens;
+    if (len <= 0 || start >= len) {
         return;
     }
-    const int end = min(len, start + a.partition_tokens);
+    const int end = min(len, start + partition_tokens);
     const int n_tiles = (end - start + kMlaWideTileTokens - 1) / kMlaWideTileTokens;
 
     const int first_entry = start >> a.block_shift;
@@ -580,7 +677,7 @@ __global__ void __launch_bounds__(kMlaWideThreads, 2) decodeMlaWideKernel(Decode
 
     // Epilogue, as in decodeMlaKernel
     const float l_tot = sumAcrossTokenGroups(l);
-    const bool single = len <= a.partition_tokens;
+    const bool single = len <= partition_tokens;
 #pragma unroll
     for (int rr = 0; rr < 4; ++rr) {
         const int hl = 4 * g + rr; // head (within the chunk) of accumulator row rr

@@ -61,10 +61,11 @@ __global__ void __launch_bounds__(kReduceThreads) decodeReduceKernel(DecodeArgs 
     const int64_t len64 = loadIndex<Tindex>(a.seq_lens, seq);
     const int64_t max_len = static_cast<int64_t>(a.max_blocks_per_seq) * a.block_size;
     const int len = static_cast<int>(len64 < max_len ? len64 : max_len);
-    if (len <= a.partition_tokens) {
+    const int partition_tokens = a.chosen_partition != nullptr ? a.chosen_partition[0] : a.partition_tokens;
+    if (len <= partition_tokens) {
         return; // empty sequence, or already finished by the decode kernel (uniform for the workgroup)
     }
-    const int parts = (len + a.partition_tokens - 1) / a.partition_tokens;
+    const int parts = (len + partition_tokens - 1) / partition_tokens;
     const int64_t slot0 = (static_cast<int64_t>(seq) * a.num_heads + head) * a.max_partitions;
 
     // this thread's partitions: running (m, l, acc) merge
@@ -138,6 +139,107 @@ __global__ void __launch_bounds__(kReduceThreads) decodeReduceKernel(DecodeArgs 
         o_ptr[1] = T::fromFloat(sum.y * inv_l);
         o_ptr[2] = T::fromFloat(sum.z * inv_l);
         o_ptr[3] = T::fromFloat(sum.w * inv_l);
+    }
+}
+
+// The same merge for calls with at most 64 partitions per sequence and few of them in use: one WAVEFRONT
+// per (query head, sequence), four per workgroup. Lane p fetches (m, l) of partition p; the partial rows
+// are then added one after the other with every lane on its own columns (column lane * kVec + 64 kVec j:
+// every load instruction of the wavefront reads one contiguous piece of a row), all loads independent of
+// each other. No LDS, no barrier, and a sequence with three partitions keeps all 64 lanes busy, where the
+// kernel above would leave thirteen of its sixteen row groups idle.
+template <typename T, typename Tindex, int VALUE>
+__global__ void __launch_bounds__(kReduceThreads) decodeReduceWaveKernel(DecodeArgs a) {
+    using S = typename T::storage;
+    constexpr int kVec = VALUE % 256 == 0 ? 4 : (VALUE % 128 == 0 ? 2 : 1); // floats per load
+    constexpr int kLoads = VALUE / (64 * kVec);
+    static_assert(kLoads * 64 * kVec == VALUE, "value sizes are multiples of 64");
+
+    const int lane = threadIdx.x & 63;
+    const int64_t pair = static_cast<int64_t>(blockIdx.x) * (kReduceThreads / 64) + (threadIdx.x >> 6); // seq * num_heads + head
+    if (pair >= static_cast<int64_t>(a.num_seqs) * a.num_heads) {
+        return;
+    }
+    const int seq = static_cast<int>(pair / a.num_heads);
+    const int head = static_cast<int>(pair - static_cast<int64_t>(seq) * a.num_heads);
+    const int64_t len64 = loadIndex<Tindex>(a.seq_lens, seq);
+    const int64_t max_len = static_cast<int64_t>(a.max_blocks_per_seq) * a.block_size;
+    const int len = static_cast<int>(len64 < max_len ? len64 : max_len);
+    const int partition_tokens = a.chosen_partition != nullptr ? a.chosen_partition[0] : a.partition_tokens;
+    if (len <= partition_tokens) {
+        return; // empty sequence, or already finished by the decode kernel (uniform for the wavefront)
+    }
+    const int parts = (len + partition_tokens - 1) / partition_tokens; // <= max_partitions <= 64
+    const int64_t slot0 = pair * a.max_partitions;
+
+    const float m_p = lane < parts ? a.part_m[slot0 + lane] : -INFINITY;
+    const float l_p = lane < parts ? a.part_l[slot0 + lane] : 0.0f;
+    float m = m_p;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        m = fmaxf(m, __shfl_xor(m, off, 64));
+    }
+    const float w_p = mergeWeight(m_p, m);
+    float l = l_p * w_p;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        l += __shfl_xor(l, off, 64);
+    }
+
+    float acc[kLoads][kVec];
+#pragma unroll
+    for (int j = 0; j < kLoads; ++j) {
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) {
+            acc[j][e] = 0.0f;
+        }
+    }
+    // four partial rows per trip, so that their loads are in flight together; a trip past the last
+    // partition reads the last row again with weight 0
+    for (int p0 = 0; p0 < parts; p0 += 4) {
+        float w[4];
+        const float *row[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int p = min(p0 + u, parts - 1);
+            w[u] = p0 + u < parts ? __shfl(w_p, p, 64) : 0.0f;
+            row[u] = a.part_acc + (slot0 + p) * VALUE + lane * kVec;
+        }
+        float v[4][kLoads][kVec];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+#pragma unroll
+            for (int j = 0; j < kLoads; ++j) {
+                if constexpr (kVec == 4) {
+                    const float4 x = *reinterpret_cast<const float4 *>(row[u] + 64 * kVec * j);
+                    v[u][j][0] = x.x, v[u][j][1] = x.y, v[u][j][2] = x.z, v[u][j][3] = x.w;
+                } else if constexpr (kVec == 2) {
+                    const float2 x = *reinterpret_cast<const float2 *>(row[u] + 64 * kVec * j);
+                    v[u][j][0] = x.x, v[u][j][1] = x.y;
+                } else {
+                    v[u][j][0] = row[u][64 * j];
+                }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+#pragma unroll
+            for (int j = 0; j < kLoads; ++j) {
+#pragma unroll
+                for (int e = 0; e < kVec; ++e) {
+                    acc[j][e] += v[u][j][e] * w[u];
+                }
+            }
+        }
+    }
+    const float inv_l = 1.0f / (l + 1e-6f);
+    S *o_ptr = static_cast<S *>(a.out) + seq * a.o_stride + head * a.o_head_stride + lane * kVec;
+#pragma unroll
+    for (int j = 0; j < kLoads; ++j) {
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) {
+            o_ptr[64 * kVec * j + e] = T::fromFloat(acc[j][e] * inv_l);
+        }
     }
 }
 

@@ -25,6 +25,7 @@ struct Plan {
     bool tiled;            // tiled matrix-core kernel (head 64 / 128 / 192 / 256 or 576 with values of 512, power-of-two pages >= 16, 16-byte aligned strides)
     bool balanced;         // tiled kernel under the work-equalising schedule (decode_balanced.h)
     bool latent_wide;      // latent attention with more than 32 query heads per KV head: 64 heads per workgroup
+    bool partition_forced; // INFINIOP_AMD_PA_PARTITION set: the 64-head kernel keeps exactly that size
     int partition_tokens;  // grid schedule: tokens per unit of work
     int max_partitions;    // grid schedule: partitions the longest representable sequence needs
     int dims_per_lane;     // element-wise kernel: ceil(max(head_size, value_size) / 64)
@@ -112,6 +113,7 @@ Plan makePlan(const PagedAttentionInfo &in, const device::amd::DeviceInfo &dev) 
         const int forced = std::atoi(env);
         if (forced >= 16) {
             p = (forced + 15) / 16 * 16;
+            plan.partition_forced = true;
         }
     }
     // Bound the workspace: at most 128 partitions, unless that would exceed what one wavefront of
@@ -156,6 +158,9 @@ Plan makePlan(const PagedAttentionInfo &in, const device::amd::DeviceInfo &dev) 
         rows = rows > balanced_rows ? rows : balanced_rows;
         plan.pieces_bytes = alignUp(in.num_seqs * 2 * sizeof(int), 256);
     }
+    if (plan.latent_wide) {
+        plan.pieces_bytes = 256; // the partition size the decode kernel chose, for the merge kernel
+    }
     if (rows > 0) {
         plan.acc_bytes = alignUp(rows * in.num_heads * in.value_size * sizeof(float), 256);
         plan.ml_bytes = alignUp(rows * in.num_heads * sizeof(float), 256);
@@ -177,6 +182,20 @@ void launchGeneric(const DecodeArgs &a, const Plan &plan, hipStream_t stream) {
 
 template <typename T, typename Tindex>
 void launchReduce(const DecodeArgs &a, hipStream_t stream) {
+    if (a.max_partitions <= 16) {
+        // few partitions per sequence: one wavefront per (head, sequence)
+        const long long pairs = static_cast<long long>(a.num_heads) * a.num_seqs;
+        const dim3 few(static_cast<unsigned>((pairs + 3) / 4));
+        switch (a.value_size / 64) {
+        case 1: decodeReduceWaveKernel<T, Tindex, 64><<<few, kReduceThreads, 0, stream>>>(a); break;
+        case 2: decodeReduceWaveKernel<T, Tindex, 128><<<few, kReduceThreads, 0, stream>>>(a); break;
+        case 3: decodeReduceWaveKernel<T, Tindex, 192><<<few, kReduceThreads, 0, stream>>>(a); break;
+        case 4: decodeReduceWaveKernel<T, Tindex, 256><<<few, kReduceThreads, 0, stream>>>(a); break;
+        case 8: decodeReduceWaveKernel<T, Tindex, 512><<<few, kReduceThreads, 0, stream>>>(a); break;
+        default: decodeReduceWaveKernel<T, Tindex, 576><<<few, kReduceThreads, 0, stream>>>(a); break;
+        }
+        return;
+    }
     const dim3 grid(a.num_heads, a.num_seqs);
     switch (a.value_size / 16) { // value sizes the validator lets through: 64, 128, 192, 256, 512, 576
     case 4: decodeReduceKernel<T, Tindex, 4><<<grid, kReduceThreads, 0, stream>>>(a); break;
@@ -215,8 +234,16 @@ void launchAll(const DecodeArgs &a, const Plan &plan, bool tiled, hipStream_t st
             const dim3 grid(plan.max_partitions, a.num_kv_heads * head_chunks, a.num_seqs);
             if (plan.latent_wide) {
                 const int groups_of_chunks = (head_chunks + kMlaWideChunks - 1) / kMlaWideChunks;
-                const dim3 wide(plan.max_partitions, a.num_kv_heads * groups_of_chunks, a.num_seqs);
-                decodeMlaWideKernel<T, Tindex><<<wide, kMlaWideThreads, 0, stream>>>(a);
+                const int streams = a.num_kv_heads * groups_of_chunks;
+                if (a.chosen_partition != nullptr) {
+                    // units planned by the kernel from the actual lengths: at most one per (sequence, planned partition)
+                    const long long units = static_cast<long long>(a.num_seqs) * plan.max_partitions;
+                    const dim3 dense(static_cast<unsigned>((units + 7) / 8 * 8 * streams));
+                    decodeMlaWideKernel<T, Tindex><<<dense, kMlaWideThreads, 0, stream>>>(a);
+                } else {
+                    const dim3 wide(plan.max_partitions, streams, a.num_seqs);
+                    decodeMlaWideKernel<T, Tindex><<<wide, kMlaWideThreads, 0, stream>>>(a);
+                }
                 break;
             }
             decodeMlaKernel<T, Tindex><<<grid, kMlaThreads, 0, stream>>>(a);
@@ -325,6 +352,9 @@ infiniStatus_t Descriptor::calculate(void *workspace, size_t workspace_size, voi
         a.part_m = reinterpret_cast<float *>(ws + plan.acc_bytes);
         a.part_l = reinterpret_cast<float *>(ws + plan.acc_bytes + plan.ml_bytes);
         a.seq_pieces = reinterpret_cast<int2 *>(ws + plan.acc_bytes + 2 * plan.ml_bytes);
+        if (plan.latent_wide && !plan.partition_forced && in.num_seqs <= 256 && plan.tiled && aligned16(out) && aligned16(q) && aligned16(k_cache) && aligned16(v_cache)) {
+            a.chosen_partition = reinterpret_cast<int32_t *>(ws + plan.acc_bytes + 2 * plan.ml_bytes);
+        }
     }
     a.scale_log2 = in.scale * kLog2e;
     a.num_seqs = static_cast<int32_t>(in.num_seqs);
@@ -342,6 +372,7 @@ infiniStatus_t Descriptor::calculate(void *workspace, size_t workspace_size, voi
     a.max_blocks_per_seq = static_cast<int32_t>(in.max_num_blocks_per_seq);
     a.partition_tokens = plan.partition_tokens;
     a.max_partitions = plan.max_partitions;
+    a.compute_units = device::amd::deviceInfo(device_id).compute_units;
     a.q_stride = in.q_stride;
     a.q_head_stride = in.q_head_stride;
     a.o_stride = in.o_stride;
