@@ -2,8 +2,8 @@
 // value_size 512, the shape of the reference's dedicated kernel
 // (src/infiniop/ops/paged_attention/nvidia/paged_attention_mla_hd576_v512.cu). gfx950, 64-lane wavefronts.
 // Two kernels: decodeMlaKernel (16 query heads per workgroup of two wavefronts, described first) and
-// decodeMlaWideKernel (64 query heads per workgroup of eight, for more than 32 heads per KV head; further
-// down).
+// decodeMlaWideKernel (up to 64 query heads per workgroup of eight, for more than 16 heads per KV head;
+// further down).
 //
 // Unit of work and arithmetic are those of the head-128 tiled kernel (decode_tiled.h): one unit = one
 // (partition, KV head x 16 query heads, sequence), tiles of 16 tokens, K . Q^T and P . V on the matrix
@@ -275,7 +275,7 @@ __global__ void __launch_bounds__(kMlaThreads, 2) decodeMlaKernel(DecodeArgs a) 
 }
 
 // ---- many query heads per KV head ---------------------------------------------------------------------
-// With more than 32 query heads per KV head the kernel above fetches every K / V tile once per 16 heads
+// With more than 16 query heads per KV head the kernel above fetches every K / V tile once per 16 heads
 // (from L2) and each pair of wavefronts moves a whole tile through its own registers. The kernel below
 // gives a workgroup of EIGHT wavefronts 64 query heads of one (partition, sequence): a K / V tile of 32
 // tokens (two halves of 16, each inside one page) is fetched once for all of them and shared through

@@ -87,12 +87,13 @@ Plan makePlan(const PagedAttentionInfo &in, const device::amd::DeviceInfo &dev) 
     // A unit of the latent-attention kernel leaves 32 KiB of partial results and advances one tile per
     // ~2 us however many units there are: fewer, longer units measured best there (more units end the
     // decode kernel sooner, but writing and merging their partial results costs more than that gains).
-    // Latent attention with more than two 16-head chunks per KV head runs 64 heads per workgroup
-    // (measured against the 16-head units: 32 heads 61.5 vs 62.0 us, 48 heads 65.7 vs 82.3, 64 heads
-    // 67.5 vs 104.2, 128 heads 122 vs 165; 128 sequences of 128 heads 368 vs 708). One workgroup per
-    // compute unit there, 128 KiB of partial results each: about one round of workgroups measured best.
+    // Latent attention with more than one 16-head chunk per KV head runs up to 64 heads per workgroup
+    // (measured against the 16-head units, 32 sequences: 16 heads 54.4 vs 40.7 us, 32 heads 58.1 vs 62.0,
+    // 48 heads 60 vs 82, 64 heads 64 vs 104, 128 heads 83 vs 165; 128 sequences of 32 heads 163 vs 245, of
+    // 128 heads 314 vs 708). One workgroup per compute unit there, up to 128 KiB of partial results each:
+    // about one round of workgroups measured best.
     const long long head_chunks = (group + kHeadsPerWave - 1) / kHeadsPerWave;
-    plan.latent_wide = plan.tiled && latent_head && head_chunks > 2;
+    plan.latent_wide = plan.tiled && latent_head && head_chunks > 1;
     if (const char *env = std::getenv("INFINIOP_AMD_PA_LATENT_KERNEL")) {
         if (std::strcmp(env, "wide") == 0) {
             plan.latent_wide = plan.tiled && latent_head;
