@@ -24,7 +24,7 @@ namespace {
 struct Plan {
     bool tiled;            // tiled matrix-core kernel (head 64 / 128 / 192 / 256 or 576 with values of 512, power-of-two pages >= 16, 16-byte aligned strides)
     bool balanced;         // tiled kernel under the work-equalising schedule (decode_balanced.h)
-    bool latent_wide;      // latent attention with more than 32 query heads per KV head: 64 heads per workgroup
+    bool latent_wide;      // latent attention with more than 16 query heads per KV head: up to 64 heads per workgroup
     bool partition_forced; // INFINIOP_AMD_PA_PARTITION set: the 64-head kernel keeps exactly that size
     int partition_tokens;  // grid schedule: tokens per unit of work
     int max_partitions;    // grid schedule: partitions the longest representable sequence needs
