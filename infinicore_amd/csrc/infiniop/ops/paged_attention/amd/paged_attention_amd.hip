@@ -93,7 +93,11 @@ Plan makePlan(const PagedAttentionInfo &in, const device::amd::DeviceInfo &dev) 
     // 128 heads 314 vs 708). One workgroup per compute unit there, up to 128 KiB of partial results each:
     // about one round of workgroups measured best.
     const long long head_chunks = (group + kHeadsPerWave - 1) / kHeadsPerWave;
-    plan.latent_wide = plan.tiled && latent_head && head_chunks > 1;
+    // A single chunk takes it too while the batch is small (its finer, per-call planned partitions then
+    // count for more than its idle wavefronts: 16 heads, 1 / 4 / 16 sequences 19.0 / 21.2 / 29.4 vs
+    // 29.0 / 29.8 / 31.6 us).
+    plan.latent_wide = plan.tiled && latent_head
+                    && (head_chunks > 1 || static_cast<long long>(in.num_seqs) * in.num_kv_heads <= 16);
     if (const char *env = std::getenv("INFINIOP_AMD_PA_LATENT_KERNEL")) {
         if (std::strcmp(env, "wide") == 0) {
             plan.latent_wide = plan.tiled && latent_head;

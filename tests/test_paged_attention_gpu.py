@@ -219,7 +219,7 @@ def mla(name, dtype, B, H, bs, lo, hi, seed, **kw):
 @pytest.fixture(params=[None, "narrow", "wide"], ids=["auto", "narrow", "wide"])
 def latent_kernel(request, monkeypatch):
     """The two latent-attention kernels: 16 query heads per workgroup of two wavefronts ("narrow"), 64 per
-    workgroup of eight ("wide"); left alone, more than 16 heads per KV head take the wide one."""
+    workgroup of eight ("wide"); left alone, more than 16 heads per KV head and small batches take the wide one."""
     if request.param:
         monkeypatch.setenv("INFINIOP_AMD_PA_LATENT_KERNEL", request.param)
     return request.param
