@@ -303,6 +303,36 @@ def test_mla_full_size_against_oracle(gpu_handle, oracle, workload):
     run_case(gpu_handle, oracle, workloads.make_decode_inputs(workloads.DECODE_CONFIGS[workload]))
 
 
+def test_mla_empty_and_negative_lengths_in_the_per_call_plan(gpu_handle, oracle):
+    """The 64-head kernel numbers its units from the lengths it reads itself: sequences without tokens get
+    none, and their output rows stay untouched."""
+    inp = workloads.make_decode_inputs(mla("mla_empty", torch.float16, 7, 48, 16, 1, 2000, seed=460))
+    inp.seq_lens[0], inp.seq_lens[3], inp.seq_lens[6] = 0, -7, 0
+    q, k, v, bt, sl = to_device(inp)
+    out = torch.full((7, 48, 512), 7.0, dtype=torch.float16, device=DEV)
+    run_paged_attention(gpu_handle, q, k, v, bt, sl, inp.scale, out=out)
+    want = torch.full((7, 48, 512), 7.0, dtype=torch.float16)
+    oracle_of(oracle, inp, out=want)
+    for s in (0, 3, 6):
+        assert torch.all(out[s] == 7)
+    assert_close(out, want, "mla_empty")
+
+
+def test_mla_more_sequences_than_the_per_call_plan_handles(gpu_handle, oracle):
+    """More than 256 sequences: fixed partitions on the three-dimensional grid."""
+    run_case(gpu_handle, oracle, workloads.make_decode_inputs(mla("mla_b300", torch.bfloat16, 300, 32, 16, 1, 400, seed=470)))
+
+
+def test_mla_sequences_that_fit_one_partition_need_no_workspace(gpu_handle, oracle):
+    inp = workloads.make_decode_inputs(mla("mla_short", torch.float16, 5, 64, 16, 1, 100, seed=480))
+    q, k, v, bt, sl = to_device(inp)
+    out = torch.zeros((5, 64, 512), dtype=torch.float16, device=DEV)
+    status, op = create_paged_attention(gpu_handle, out, q, k, v, bt, sl, None, inp.scale)
+    assert status == 0 and workspace_size_attention(op) == 0
+    L.check_error(L.LIBINFINIOP.infiniopDestroyPagedAttentionDescriptor(op))
+    run_case(gpu_handle, oracle, inp)
+
+
 @pytest.mark.parametrize("B,lo,hi", [(1, 2100, 2100), (4, 512, 4096), (16, 512, 4096)])
 def test_default_schedule_choice(gpu_handle, oracle, monkeypatch, B, lo, hi):
     """No knob set: one sequence and four ragged ones take the fixed partitions (small job), sixteen the
@@ -541,12 +571,17 @@ def test_one_descriptor_many_calls_with_changing_lengths(gpu_handle, oracle):
     L.check_error(L.LIBINFINIOP.infiniopDestroyPagedAttentionDescriptor(op))
 
 
-def test_capture_and_replay(gpu_handle, oracle):
+@pytest.mark.parametrize("shape", ["head128", "latent64heads"])
+def test_capture_and_replay(gpu_handle, oracle, shape):
     """The run call allocates nothing and never synchronises, so it can be recorded into a graph;
-    every replay (with eager work in between) must reproduce the eager result."""
-    inp = workloads.make_decode_inputs(custom("graph", torch.float16, 6, 32, 8, 128, 16, 50, 1500, seed=59))
+    every replay (with eager work in between) must reproduce the eager result. The latent-attention case
+    plans its units inside the kernel, from the lengths in device memory."""
+    if shape == "head128":
+        inp = workloads.make_decode_inputs(custom("graph", torch.float16, 6, 32, 8, 128, 16, 50, 1500, seed=59))
+    else:
+        inp = workloads.make_decode_inputs(mla("graph_latent", torch.bfloat16, 6, 64, 16, 50, 1500, seed=60))
     q, k, v, bt, sl = to_device(inp)
-    out = torch.zeros_like(q)
+    out = torch.zeros((*q.shape[:2], v.shape[-1]), dtype=q.dtype, device=DEV)
     status, op = create_paged_attention(gpu_handle, out, q, k, v, bt, sl, None, inp.scale)
     assert status == 0
     size = workspace_size_attention(op)
