@@ -434,8 +434,16 @@ __device__ __forceinline__ WidePlan planWide(const DecodeArgs &a, int lane, int 
     return plan;
 }
 
-template <typename T, typename Tindex>
+// CHUNKS = 4: as described above. CHUNKS = 1 (16 query heads per KV head): the workgroup has a single
+// chunk and all eight wavefronts work for it - wavefront w computes the partial scores of token half
+// w % 2 over a quarter of the K-steps (5, 5, 4, 4 of the 18), all eight exchange them through LDS, and
+// each owns 64 value columns (16 accumulator registers). The copy side is the same.
+template <typename T, typename Tindex, int CHUNKS>
 __global__ void __launch_bounds__(kMlaWideThreads, 2) decodeMlaWideKernel(DecodeArgs a) {
+    static_assert(CHUNKS == 1 || CHUNKS == kMlaWideChunks, "one chunk or four per workgroup");
+    constexpr bool kOne = CHUNKS == 1;
+    constexpr int kOwnSteps = kOne ? 5 : 9;   // K-steps of one wavefront (the last of the five may be empty)
+    constexpr int kOwnBlocks = kOne ? 4 : 16; // 16-column blocks of one wavefront
     using S = typename T::storage;
     constexpr int kSteps = kMlaKeySize / 32;        // 18
     constexpr int kHalfSteps = kSteps / 2;          // K-steps per wavefront
@@ -446,10 +454,10 @@ __global__ void __launch_bounds__(kMlaWideThreads, 2) decodeMlaWideKernel(Decode
     constexpr int kBlocks = kMlaValueSize / 16;              // 32 column blocks of 16
     __shared__ uint4 k_lds[2][kMlaWideTileTokens * kPitch];
     __shared__ uint4 v_lds[2][kBlocks * 64];  // [column block][token group g][lane c]: .xy first half, .zw second
-    __shared__ f32x4 s_lds[8][2][64];         // partial scores of every wavefront, both halves
+    __shared__ f32x4 s_lds[8][kOne ? 1 : 2][64]; // partial scores of every wavefront (CHUNKS = 4: both halves)
 
     const int head_chunks = (a.group + kHeadsPerWave - 1) / kHeadsPerWave;
-    const int groups_of_chunks = (head_chunks + kMlaWideChunks - 1) / kMlaWideChunks;
+    const int groups_of_chunks = (head_chunks + CHUNKS - 1) / CHUNKS;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int lane = threadIdx.x & 63;
     const int c = lane & 15;
@@ -481,8 +489,12 @@ __global__ void __launch_bounds__(kMlaWideThreads, 2) decodeMlaWideKernel(Decode
     }
     const int kv_head = stream / groups_of_chunks;
     const int chunk_group = stream - kv_head * groups_of_chunks;
-    const int chunk = chunk_group * kMlaWideChunks + (wave & 3); // may lie beyond the last chunk: no heads
-    const int kh = wave >> 2; // half of the K-steps and half of the value columns
+    const int chunk = kOne ? chunk_group : chunk_group * kMlaWideChunks + (wave & 3); // may lie beyond the last chunk: no heads
+    const int kh = wave >> 2; // CHUNKS = 4: half of the K-steps and half of the value columns
+    // this wavefront's K-steps: [first_step, first_step + own_steps)
+    const int first_step = kOne ? (wave >> 1) * 5 - ((wave >> 1) == 3 ? 1 : 0) : kh * kHalfSteps;
+    const int own_steps = kOne ? ((wave >> 1) < 2 ? 5 : 4) : kHalfSteps;
+    const int th = wave & 1; // CHUNKS = 1: the token half whose scores this wavefront computes
 
     const int64_t len64 = loadIndex<Tindex>(a.seq_lens, seq);
     const int64_t max_len = static_cast<int64_t>(a.max_blocks_per_seq) << a.block_shift;
@@ -506,14 +518,14 @@ __global__ void __launch_bounds__(kMlaWideThreads, 2) decodeMlaWideKernel(Decode
     const int head_in_group = chunk * kHeadsPerWave + c;
     const bool head_valid = head_in_group < a.group;
     const int head = kv_head * a.group + head_in_group;
-    uint4 q_reg[kHalfSteps];
+    uint4 q_reg[kOwnSteps];
     {
-        const S *q_ptr = static_cast<const S *>(a.q) + seq * a.q_stride + (head_valid ? head : 0) * a.q_head_stride
-                       + kh * (kMlaKeySize / 2);
-        const uint32_t keep = head_valid ? 0xffffffffu : 0u;
+        const S *q_ptr = static_cast<const S *>(a.q) + seq * a.q_stride + (head_valid ? head : 0) * a.q_head_stride;
 #pragma unroll
-        for (int i = 0; i < kHalfSteps; ++i) {
-            uint4 x = *reinterpret_cast<const uint4 *>(q_ptr + 32 * i + 8 * g);
+        for (int i = 0; i < kOwnSteps; ++i) {
+            const int kk = min(first_step + i, kSteps - 1);
+            const uint32_t keep = (head_valid && i < own_steps) ? 0xffffffffu : 0u; // an empty step multiplies by zero
+            uint4 x = *reinterpret_cast<const uint4 *>(q_ptr + 32 * kk + 8 * g);
             x.x &= keep, x.y &= keep, x.z &= keep, x.w &= keep;
             q_reg[i] = x;
         }
@@ -551,14 +563,21 @@ __global__ void __launch_bounds__(kMlaWideThreads, 2) decodeMlaWideKernel(Decode
     }
     auto halfOfLoad = [&](int j) { return copies_v ? ((j >> 2) & 1) : ((4 * j + role_wave) / 18); };
 
-    uint4 stage[kLoads];
+    // Register sets for tiles on their way: one (tile t + 1 while tile t is computed). A second set fits
+    // the single-chunk variant (185 registers, no spills) and was measured: 38.7 vs 37.6 us at 32 sequences,
+    // 139 vs 136 at 128 - one more tile in flight is not what holds that variant back.
+    constexpr int kSets = 1;
+    uint4 stage_sets[kSets][kLoads];
 #pragma unroll
     for (int j = 0; j < kLoads; ++j) {
-        stage[j] = make_uint4(0, 0, 0, 0);
+#pragma unroll
+        for (int i = 0; i < kSets; ++i) {
+            stage_sets[i][j] = make_uint4(0, 0, 0, 0);
+        }
     }
     // Loads for a half past the end of the partition are issued all the same but read the partition's
     // first rows (the loop body has no branch around a load).
-    auto loadStage = [&](int t) {
+    auto loadStage = [&](int t, uint4 (&stage)[kLoads]) {
         const char *half_base[2];
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
@@ -573,7 +592,7 @@ __global__ void __launch_bounds__(kMlaWideThreads, 2) decodeMlaWideKernel(Decode
             stage[j] = loadLane16(halfOfLoad(j) ? half_base[1] : half_base[0], src_off[j]);
         }
     };
-    auto storeStage = [&](int t) {
+    auto storeStage = [&](int t, const uint4 (&stage)[kLoads]) {
         const int buf = t & 1;
         if (copies_v) {
             // V rows beyond the sequence may hold anything (NaN included) and 0 * NaN is NaN: zeroed here
@@ -617,62 +636,93 @@ __global__ void __launch_bounds__(kMlaWideThreads, 2) decodeMlaWideKernel(Decode
         }
     };
 
-    // o[e][r] = O[head 4g + r of the chunk][column 256 kh + 128 (e / 8) + 8 c + e % 8]
-    f32x4 o[16];
+    // CHUNKS = 4: o[e][r] = O[head 4g + r of the chunk][column 256 kh + 128 (e / 8) + 8 c + e % 8]
+    // CHUNKS = 1: o[e][r] = O[head 4g + r][column 128 (wave / 2) + 8 c + 4 (wave % 2) + e]
+    f32x4 o[kOwnBlocks];
 #pragma unroll
-    for (int e = 0; e < 16; ++e) {
+    for (int e = 0; e < kOwnBlocks; ++e) {
         o[e] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
+    const int first_block = kOne ? 4 * wave : 16 * kh;
     float m = -INFINITY; // reference point of head c's exponentials (same value in the four lanes g = 0..3)
     float l = 0.0f;      // sum of rounded probabilities of head c over this lane's tokens only
 
-    loadStage(0);
-    storeStage(0);
-    loadStage(1);
-    for (int t = 0; t < n_tiles; ++t) {
-        const int buf = t & 1;
-        __syncthreads(); // tile t is complete in LDS, and everybody has finished with tile t - 1
-        if (t + 1 < n_tiles) {
-            storeStage(t + 1);
-        }
-        loadStage(t + 2);
-        // partial scores of both halves over this wavefront's K-steps: four independent chains (a matrix
-        // instruction that accumulates into the result of the previous one waits ~44 cycles for it, an
-        // independent one issues after 16)
-        f32x4 sp[2][2] = {{{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}}, {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}}};
+    // Tile t is computed from LDS buffer t & 1 while tile t + 1 (and, with two register sets, t + 2) is
+    // on its way: set (t + 1) % kSets is stored at the start of tile t and refilled right away. With two
+    // sets, two tiles per trip so that the sets are addressed statically.
+    loadStage(0, stage_sets[0]);
+    if constexpr (kSets == 2) {
+        loadStage(1, stage_sets[1]);
+    }
+    storeStage(0, stage_sets[0]);
+    loadStage(kSets, stage_sets[0]);
+    for (int t0 = 0; t0 < n_tiles; t0 += kSets) {
 #pragma unroll
-        for (int i = 0; i < kHalfSteps; ++i) {
-            const int kk = kh * kHalfSteps + i;
-            sp[0][i & 1] = T::mfmaK32(k_lds[buf][c * kPitch + 4 * kk + g], q_reg[i], sp[0][i & 1]);
-            sp[1][i & 1] = T::mfmaK32(k_lds[buf][(16 + c) * kPitch + 4 * kk + g], q_reg[i], sp[1][i & 1]);
+    for (int d = 0; d < kSets; ++d) {
+        const int t = t0 + d;
+        if (t >= n_tiles) {
+            break; // the same for all wavefronts: they pass the same barriers
         }
-        f32x4 s0 = sp[0][0] + sp[0][1], s1 = sp[1][0] + sp[1][1];
-        s_lds[wave][0][lane] = s0;
-        s_lds[wave][1][lane] = s1;
-        __syncthreads(); // partial scores of both K halves are there
-        s0 += s_lds[wave ^ 4][0][lane];
-        s1 += s_lds[wave ^ 4][1][lane];
+        const int buf = kSets == 2 ? d : (t & 1);
+        __syncthreads(); // tile t is complete in LDS, and everybody has finished with tile t - 1
+        uint4 (&next_set)[kLoads] = stage_sets[kSets == 2 ? (d ^ 1) : 0];
+        if (t + 1 < n_tiles) {
+            storeStage(t + 1, next_set);
+        }
+        loadStage(t + 1 + kSets, next_set);
+        f32x4 s0, s1;
+        if constexpr (!kOne) {
+            // partial scores of both halves over this wavefront's K-steps: four independent chains (a
+            // matrix instruction that accumulates into the result of the previous one waits ~44 cycles
+            // for it, an independent one issues after 16)
+            f32x4 sp[2][2] = {{{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}}, {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}}};
+#pragma unroll
+            for (int i = 0; i < kOwnSteps; ++i) {
+                const int kk = first_step + i;
+                sp[0][i & 1] = T::mfmaK32(k_lds[buf][c * kPitch + 4 * kk + g], q_reg[i], sp[0][i & 1]);
+                sp[1][i & 1] = T::mfmaK32(k_lds[buf][(16 + c) * kPitch + 4 * kk + g], q_reg[i], sp[1][i & 1]);
+            }
+            s0 = sp[0][0] + sp[0][1], s1 = sp[1][0] + sp[1][1];
+            s_lds[wave][0][lane] = s0;
+            s_lds[wave][1][lane] = s1;
+            __syncthreads(); // partial scores of both K halves are there
+            s0 += s_lds[wave ^ 4][0][lane];
+            s1 += s_lds[wave ^ 4][1][lane];
+        } else {
+            // partial scores of this wavefront's token half over its quarter of the K-steps
+            f32x4 sp[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+#pragma unroll
+            for (int i = 0; i < kOwnSteps; ++i) {
+                const int kk = min(first_step + i, kSteps - 1);
+                sp[i & 1] = T::mfmaK32(k_lds[buf][(16 * th + c) * kPitch + 4 * kk + g], q_reg[i], sp[i & 1]);
+            }
+            s_lds[wave][0][lane] = sp[0] + sp[1];
+            __syncthreads(); // all eight partial tiles are there: wavefront 2 q + h holds quarter q of half h
+            s0 = (s_lds[0][0][lane] + s_lds[2][0][lane]) + (s_lds[4][0][lane] + s_lds[6][0][lane]);
+            s1 = (s_lds[1][0][lane] + s_lds[3][0][lane]) + (s_lds[5][0][lane] + s_lds[7][0][lane]);
+        }
 
         const int tok0 = start + t * kMlaWideTileTokens;
         const int valid = min(kMlaWideTileTokens, end - tok0);
         uint4 p_op, p_lo;
-        softmaxStepPair<T, 16>(o, m, l, s0, s1, g, a.scale_log2, slope, tok0 - (len - 1), valid, p_op, p_lo);
-        // all sixteen column blocks with the high parts first, then with the low parts (independent chains)
-        uint4 vf[16];
+        softmaxStepPair<T, kOwnBlocks>(o, m, l, s0, s1, g, a.scale_log2, slope, tok0 - (len - 1), valid, p_op, p_lo);
+        // all column blocks with the high parts first, then with the low parts (independent chains)
+        uint4 vf[kOwnBlocks];
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-            vf[e] = v_lds[buf][((16 * kh + e) * 4 + g) * 16 + c];
+        for (int e = 0; e < kOwnBlocks; ++e) {
+            vf[e] = v_lds[buf][((first_block + e) * 4 + g) * 16 + c];
         }
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
+        for (int e = 0; e < kOwnBlocks; ++e) {
             o[e] = T::mfmaK32(p_op, vf[e], o[e]);
         }
         if constexpr (T::kSplitProbabilities) {
 #pragma unroll
-            for (int e = 0; e < 16; ++e) {
+            for (int e = 0; e < kOwnBlocks; ++e) {
                 o[e] = T::mfmaK32(p_lo, vf[e], o[e]);
             }
         }
+    }
     }
 
     // Epilogue, as in decodeMlaKernel
@@ -688,12 +738,32 @@ __global__ void __launch_bounds__(kMlaWideThreads, 2) decodeMlaWideKernel(Decode
             continue;
         }
         const int out_head = kv_head * a.group + hg;
+        if constexpr (kOne) {
+            const int col0 = 128 * (wave >> 1) + 8 * c + 4 * (wave & 1);
+            if (single) {
+                const float inv_l = 1.0f / (l_h + 1e-6f);
+                S *o_ptr = static_cast<S *>(a.out) + seq * a.o_stride + out_head * a.o_head_stride + col0;
+                uint2 w;
+                w.x = T::pack2(o[0][rr] * inv_l, o[1][rr] * inv_l);
+                w.y = T::pack2(o[2][rr] * inv_l, o[3][rr] * inv_l);
+                *reinterpret_cast<uint2 *>(o_ptr) = w;
+            } else {
+                const int64_t slot = (static_cast<int64_t>(seq) * a.num_heads + out_head) * a.max_partitions + part;
+                float *dst = a.part_acc + slot * kMlaValueSize + col0;
+                *reinterpret_cast<float4 *>(dst) = make_float4(o[0][rr], o[1][rr], o[2][rr], o[3][rr]);
+                if (c == 0 && wave == 0) {
+                    a.part_m[slot] = m_h;
+                    a.part_l[slot] = l_h;
+                }
+            }
+            continue;
+        }
         const int col0 = 256 * kh + 8 * c;
         if (single) {
             const float inv_l = 1.0f / (l_h + 1e-6f);
             S *o_ptr = static_cast<S *>(a.out) + seq * a.o_stride + out_head * a.o_head_stride + col0;
 #pragma unroll
-            for (int i = 0; i < 2; ++i) {
+            for (int i = 0; i < kOwnBlocks / 8; ++i) {
                 uint4 w;
                 w.x = T::pack2(o[8 * i + 0][rr] * inv_l, o[8 * i + 1][rr] * inv_l);
                 w.y = T::pack2(o[8 * i + 2][rr] * inv_l, o[8 * i + 3][rr] * inv_l);
@@ -705,7 +775,7 @@ __global__ void __launch_bounds__(kMlaWideThreads, 2) decodeMlaWideKernel(Decode
             const int64_t slot = (static_cast<int64_t>(seq) * a.num_heads + out_head) * a.max_partitions + part;
             float *dst = a.part_acc + slot * kMlaValueSize + col0;
 #pragma unroll
-            for (int i = 0; i < 2; ++i) {
+            for (int i = 0; i < kOwnBlocks / 8; ++i) {
                 reinterpret_cast<float4 *>(dst + 128 * i)[0] = make_float4(o[8 * i + 0][rr], o[8 * i + 1][rr], o[8 * i + 2][rr], o[8 * i + 3][rr]);
                 reinterpret_cast<float4 *>(dst + 128 * i)[1] = make_float4(o[8 * i + 4][rr], o[8 * i + 5][rr], o[8 * i + 6][rr], o[8 * i + 7][rr]);
             }

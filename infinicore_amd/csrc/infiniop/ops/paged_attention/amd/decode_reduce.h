@@ -142,7 +142,7 @@ __global__ void __launch_bounds__(kReduceThreads) decodeReduceKernel(DecodeArgs 
     }
 }
 
-// The same merge for calls with at most 64 partitions per sequence and few of them in use: one WAVEFRONT
+// The same merge for calls with few partitions per sequence (the host uses it up to 8): one WAVEFRONT
 // per (query head, sequence), four per workgroup. Lane p fetches (m, l) of partition p; the partial rows
 // are then added one after the other with every lane on its own columns (column lane * kVec + 64 kVec j:
 // every load instruction of the wavefront reads one contiguous piece of a row), all loads independent of

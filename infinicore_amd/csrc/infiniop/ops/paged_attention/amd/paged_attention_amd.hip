@@ -93,11 +93,11 @@ Plan makePlan(const PagedAttentionInfo &in, const device::amd::DeviceInfo &dev) 
     // 128 heads 314 vs 708). One workgroup per compute unit there, up to 128 KiB of partial results each:
     // about one round of workgroups measured best.
     const long long head_chunks = (group + kHeadsPerWave - 1) / kHeadsPerWave;
-    // A single chunk takes it too while the batch is small (its finer, per-call planned partitions then
-    // count for more than its idle wavefronts: 16 heads, 1 / 4 / 16 sequences 19.0 / 21.2 / 29.4 vs
-    // 29.0 / 29.8 / 31.6 us).
+    // A single chunk gets all eight wavefronts of such a workgroup (decodeMlaWideKernel<.., 1>) up to 64
+    // sequences x KV heads (16 heads, 1 / 4 / 16 / 32 sequences: 16.0 / 18.9 / 26.2 / 37.8 vs 28.8 / 29.8 /
+    // 31.5 / 39.1 us on the 16-head units; 128 sequences: 135.8 vs 134.1).
     plan.latent_wide = plan.tiled && latent_head
-                    && (head_chunks > 1 || static_cast<long long>(in.num_seqs) * in.num_kv_heads <= 16);
+                    && (head_chunks > 1 || static_cast<long long>(in.num_seqs) * in.num_kv_heads <= 64);
     if (const char *env = std::getenv("INFINIOP_AMD_PA_LATENT_KERNEL")) {
         if (std::strcmp(env, "wide") == 0) {
             plan.latent_wide = plan.tiled && latent_head;
@@ -187,8 +187,9 @@ void launchGeneric(const DecodeArgs &a, const Plan &plan, hipStream_t stream) {
 
 template <typename T, typename Tindex>
 void launchReduce(const DecodeArgs &a, hipStream_t stream) {
-    if (a.max_partitions <= 16) {
-        // few partitions per sequence: one wavefront per (head, sequence)
+    if (a.max_partitions <= 8) {
+        // few partitions per sequence: one wavefront per (head, sequence) (up to 8: m2 14.6 -> 8.2 us; with
+        // 16, of which m1 uses up to 16, the workgroup-per-row kernel is the faster one: 4.7 vs 5.4 us)
         const long long pairs = static_cast<long long>(a.num_heads) * a.num_seqs;
         const dim3 few(static_cast<unsigned>((pairs + 3) / 4));
         switch (a.value_size / 64) {
@@ -238,16 +239,20 @@ void launchAll(const DecodeArgs &a, const Plan &plan, bool tiled, hipStream_t st
             const int head_chunks = (a.group + kHeadsPerWave - 1) / kHeadsPerWave;
             const dim3 grid(plan.max_partitions, a.num_kv_heads * head_chunks, a.num_seqs);
             if (plan.latent_wide) {
-                const int groups_of_chunks = (head_chunks + kMlaWideChunks - 1) / kMlaWideChunks;
+                // a single chunk of 16 heads gets the whole workgroup; otherwise four chunks share one
+                const bool one_chunk = head_chunks == 1;
+                const int groups_of_chunks = one_chunk ? 1 : (head_chunks + kMlaWideChunks - 1) / kMlaWideChunks;
                 const int streams = a.num_kv_heads * groups_of_chunks;
+                dim3 wide(plan.max_partitions, streams, a.num_seqs);
                 if (a.chosen_partition != nullptr) {
                     // units planned by the kernel from the actual lengths: at most one per (sequence, planned partition)
                     const long long units = static_cast<long long>(a.num_seqs) * plan.max_partitions;
-                    const dim3 dense(static_cast<unsigned>((units + 7) / 8 * 8 * streams));
-                    decodeMlaWideKernel<T, Tindex><<<dense, kMlaWideThreads, 0, stream>>>(a);
+                    wide = dim3(static_cast<unsigned>((units + 7) / 8 * 8 * streams));
+                }
+                if (one_chunk) {
+                    decodeMlaWideKernel<T, Tindex, 1><<<wide, kMlaWideThreads, 0, stream>>>(a);
                 } else {
-                    const dim3 wide(plan.max_partitions, streams, a.num_seqs);
-                    decodeMlaWideKernel<T, Tindex><<<wide, kMlaWideThreads, 0, stream>>>(a);
+                    decodeMlaWideKernel<T, Tindex, kMlaWideChunks><<<wide, kMlaWideThreads, 0, stream>>>(a);
                 }
                 break;
             }
