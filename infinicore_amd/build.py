@@ -1,4 +1,4 @@
-"""Compile ``libinfinirt.so`` and ``libinfiniop.so`` for gfx950 with hipcc (no GPU needed)."""
+"""Compile ``libinfinirt.so``, ``libinfiniop.so`` and ``libinfinicore_ops.so`` for gfx950 with hipcc (no GPU needed)."""
 from __future__ import annotations
 
 import os
@@ -8,7 +8,7 @@ from pathlib import Path
 PACKAGE_DIR = Path(__file__).resolve().parent
 CSRC_DIR = PACKAGE_DIR / "csrc"
 LIB_DIR = PACKAGE_DIR / "lib"
-LIBRARIES = ("libinfinirt.so", "libinfiniop.so")
+LIBRARIES = ("libinfinirt.so", "libinfiniop.so", "libinfinicore_ops.so")
 
 
 def libraries_present() -> bool:

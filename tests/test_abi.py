@@ -35,14 +35,19 @@ def test_headers_declare_the_expected_entry_points():
 
 @pytest.mark.parametrize("header,symbol", declared_symbols())
 def test_symbol_is_exported(lib, header, symbol):
-    owner = lib.LIBINFINIRT if symbol.startswith("infinirt") else lib.LIBINFINIOP
+    if symbol.startswith("infinicoreOp"):
+        from infinicore_amd import libinfinicore_ops
+
+        owner = libinfinicore_ops.LIBINFINICORE_OPS
+    else:
+        owner = lib.LIBINFINIRT if symbol.startswith("infinirt") else lib.LIBINFINIOP
     assert hasattr(owner, symbol), f"{symbol} (declared in {header}) is not exported"
 
 
 def test_headers_compile_as_c():
     import subprocess
 
-    for header in ("infiniop.h", "infinirt.h"):
+    for header in ("infiniop.h", "infinirt.h", "infinicore_ops.h"):
         subprocess.run(["gcc", "-fsyntax-only", "-x", "c", "-I", str(ROOT / "include"), str(ROOT / "include" / header)],
                        check=True)
 
