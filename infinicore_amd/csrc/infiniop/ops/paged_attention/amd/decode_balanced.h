@@ -492,7 +492,7 @@ __global__ void __launch_bounds__(64) decodeBalancedKernel(DecodeArgs a, int wav
 // strip of HEAD/16 columns c = lane % 16): row group g merges rows g, g+4, ... of the sequence, the four
 // groups are then combined with lane swaps, and the lanes of group 0 store 16 bytes each. The piece
 // range of the sequence was left in seq_pieces by the decode kernel, so the only dependent memory
-// round trips are {length, piece range} -> rows.
+// round trips are {length, piece range} -> rows (one trip for up to eight segments).
 template <typename T, typename Tindex, int HEAD>
 __global__ void __launch_bounds__(256) decodeBalancedMergeKernel(DecodeArgs a) {
     using S = typename T::storage;
@@ -519,27 +519,41 @@ __global__ void __launch_bounds__(256) decodeBalancedMergeKernel(DecodeArgs a) {
     for (int i = 0; i < kCols; ++i) {
         acc[i] = 0.0f;
     }
-    for (int p = g; p < parts; p += 4) {
-        const int64_t slot = static_cast<int64_t>(piece_first + p + seq) * a.num_heads + head;
-        const float m_p = a.part_m[slot];
-        const float l_p = a.part_l[slot];
-        const float4 *row = reinterpret_cast<const float4 *>(a.part_acc + slot * HEAD + kCols * c);
-        float4 v[kCols / 4];
+    // Two rows per row group are requested before either is used, so that a sequence of up to eight
+    // segments costs one memory round trip, not two. A row past the sequence's last segment re-reads
+    // segment 0 (written, finite) and enters with weight 0.
+    for (int p0 = 0; p0 < parts; p0 += 8) {
+        float m_p[2], l_p[2];
+        float4 v[2][kCols / 4];
 #pragma unroll
-        for (int i = 0; i < kCols / 4; ++i) {
-            v[i] = row[i];
-        }
-        const float m_new = fmaxf(m_loc, m_p);
-        const float w_old = mergeWeight(m_loc, m_new), w_p = mergeWeight(m_p, m_new);
-        l_loc = l_loc * w_old + l_p * w_p;
+        for (int j = 0; j < 2; ++j) {
+            const int p = p0 + 4 * j + g;
+            const bool real = p < parts;
+            const int64_t slot = static_cast<int64_t>(piece_first + (real ? p : 0) + seq) * a.num_heads + head;
+            const float m_row = a.part_m[slot];
+            const float l_row = a.part_l[slot];
+            const float4 *row = reinterpret_cast<const float4 *>(a.part_acc + slot * HEAD + kCols * c);
 #pragma unroll
-        for (int i = 0; i < kCols / 4; ++i) {
-            acc[4 * i + 0] = acc[4 * i + 0] * w_old + v[i].x * w_p;
-            acc[4 * i + 1] = acc[4 * i + 1] * w_old + v[i].y * w_p;
-            acc[4 * i + 2] = acc[4 * i + 2] * w_old + v[i].z * w_p;
-            acc[4 * i + 3] = acc[4 * i + 3] * w_old + v[i].w * w_p;
+            for (int i = 0; i < kCols / 4; ++i) {
+                v[j][i] = row[i];
+            }
+            m_p[j] = real ? m_row : -INFINITY;
+            l_p[j] = real ? l_row : 0.0f;
         }
-        m_loc = m_new;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const float m_new = fmaxf(m_loc, m_p[j]);
+            const float w_old = mergeWeight(m_loc, m_new), w_p = mergeWeight(m_p[j], m_new);
+            l_loc = l_loc * w_old + l_p[j] * w_p;
+#pragma unroll
+            for (int i = 0; i < kCols / 4; ++i) {
+                acc[4 * i + 0] = acc[4 * i + 0] * w_old + v[j][i].x * w_p;
+                acc[4 * i + 1] = acc[4 * i + 1] * w_old + v[j][i].y * w_p;
+                acc[4 * i + 2] = acc[4 * i + 2] * w_old + v[j][i].z * w_p;
+                acc[4 * i + 3] = acc[4 * i + 3] * w_old + v[j][i].w * w_p;
+            }
+            m_loc = m_new;
+        }
     }
     const float m_all = swapMax(m_loc);
     const float f = mergeWeight(m_loc, m_all);
