@@ -115,8 +115,15 @@ struct TileRun {
     bool valid;      // false past the end of the wavefront's piece
 };
 
+// Register budget: at head 128 the kernel is compiled for two wavefronts per SIMD (256 vector registers,
+// no accumulation registers). It runs one per SIMD all the same (the grid has four wavefronts per compute
+// unit); the point is the allocation: left alone the compiler takes 234 vector + 36 accumulation registers
+// and moves values between the two files in the tile loop, with the budget it fits 230 vector registers
+// without spilling (c2 57.7 -> 56.6 us, three runs each on one box). Heads 192 and 256 spill under that
+// budget, head 64 fits it anyway: they are left to the compiler.
 template <typename T, typename Tindex, int HEAD>
-__global__ void __launch_bounds__(64) decodeBalancedKernel(DecodeArgs a, int waves_per_stream) {
+__global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(HEAD == 128 ? 2 : 1, HEAD == 128 ? 2 : 8)))
+decodeBalancedKernel(DecodeArgs a, int waves_per_stream) {
     using S = typename T::storage;
     using G = TileGeometry<HEAD>;
     constexpr int NBUF = G::kBuffers;

@@ -44,6 +44,13 @@ rule("amd.hip")
             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
             "-Iinclude", "-Isrc", "-c", sourcefile, "-o", objectfile,
         }
+        -- per-file flags given with add_files(..., {cxflags = ...})
+        local fileconfig = target:fileconfig(sourcefile)
+        if fileconfig and fileconfig.cxflags then
+            for _, flag in ipairs(fileconfig.cxflags) do
+                table.insert(args, #args - 3, flag)
+            end
+        end
         depend.on_changed(function ()
             os.vrunv(ROCM .. "/bin/hipcc", args)
         end, {files = sourcefile})
@@ -78,8 +85,8 @@ target("infiniop-amd")
     add_links("amdhip64")
     add_cxflags("-fPIC")
     add_files("../src/infiniop/devices/amd/*.cc")
-    add_files("../src/infiniop/ops/paged_attention/amd/*.hip", "../src/infiniop/ops/paged_caching/amd/*.hip",
-              "../src/infiniop/ops/kv_caching/amd/*.hip")
-    -- the prefill kernel keeps its matrix-instruction accumulators in ordinary vector registers
-    add_files("../src/infiniop/ops/paged_attention_prefill/amd/*.hip", {cxflags = {"-mllvm", "-amdgpu-mfma-vgpr-form=1"}})
+    add_files("../src/infiniop/ops/paged_caching/amd/*.hip", "../src/infiniop/ops/kv_caching/amd/*.hip")
+    -- the attention kernels keep their matrix-instruction accumulators in ordinary vector registers
+    add_files("../src/infiniop/ops/paged_attention/amd/*.hip", "../src/infiniop/ops/paged_attention_prefill/amd/*.hip",
+              {cxflags = {"-mllvm", "-amdgpu-mfma-vgpr-form=1"}})
 target_end()
