@@ -57,19 +57,20 @@ __device__ __forceinline__ int waveInclusiveSum(int x) {
 // Inclusive prefix sums of the per-sequence tile counts into LDS; returns the total. Executed by
 // one wavefront (lanes 0..63 of the caller).
 template <typename Tindex>
-__device__ __forceinline__ int tilePrefixSums(const DecodeArgs &a, int lane, int *pre_incl) {
-    const int64_t max_len = static_cast<int64_t>(a.max_blocks_per_seq) << a.block_shift;
+__device__ __forceinline__ int tilePrefixSums(const void *seq_lens, int num_seqs, int max_blocks_per_seq, int block_shift,
+                                              int lane, int *pre_incl) {
+    const int64_t max_len = static_cast<int64_t>(max_blocks_per_seq) << block_shift;
     int running = 0;
-    for (int base = 0; base < a.num_seqs; base += 64) {
+    for (int base = 0; base < num_seqs; base += 64) {
         const int b = base + lane;
         int x = 0;
-        if (b < a.num_seqs) {
-            int64_t len = loadIndex<Tindex>(a.seq_lens, b);
+        if (b < num_seqs) {
+            int64_t len = loadIndex<Tindex>(seq_lens, b);
             len = len < max_len ? len : max_len;
             x = len > 0 ? static_cast<int>((len + kTileTokens - 1) / kTileTokens) : 0;
         }
         x = waveInclusiveSum(x) + running;
-        if (b < a.num_seqs) {
+        if (b < num_seqs) {
             pre_incl[b] = x;
         }
         running = __builtin_amdgcn_readlane(x, 63);
@@ -115,6 +116,11 @@ struct TileRun {
     bool valid;      // false past the end of the wavefront's piece
 };
 
+// Early arguments: the four scalars in front of the argument block are what the first memory request (the
+// sequence lengths) needs. The file is compiled with -amdgpu-kernarg-preload-count=5, which has the
+// dispatcher put the first five argument words into scalar registers before the wavefront starts, so that
+// request goes out without waiting for the scalar load of the argument block (which proceeds beside it).
+// They repeat a.seq_lens, a.num_seqs, a.max_blocks_per_seq and a.block_shift.
 // Register budget: at head 128 the kernel is compiled for two wavefronts per SIMD (256 vector registers,
 // no accumulation registers). It runs one per SIMD all the same (the grid has four wavefronts per compute
 // unit); the point is the allocation: left alone the compiler takes 234 vector + 36 accumulation registers
@@ -123,7 +129,8 @@ struct TileRun {
 // budget, head 64 fits it anyway: they are left to the compiler.
 template <typename T, typename Tindex, int HEAD>
 __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(HEAD == 128 ? 2 : 1, HEAD == 128 ? 2 : 8)))
-decodeBalancedKernel(DecodeArgs a, int waves_per_stream) {
+decodeBalancedKernel(const void *early_seq_lens, int early_num_seqs, int early_max_blocks_per_seq, int early_block_shift,
+                     DecodeArgs a, int waves_per_stream) {
     using S = typename T::storage;
     using G = TileGeometry<HEAD>;
     constexpr int NBUF = G::kBuffers;
@@ -149,7 +156,8 @@ decodeBalancedKernel(DecodeArgs a, int waves_per_stream) {
         g_pa_trace[w * 8 + 7] = __builtin_amdgcn_s_getreg(63508); // XCC_ID
     }
 #endif
-    const int total_tiles = tilePrefixSums<Tindex>(a, lane, pre_incl);
+    const int total_tiles = tilePrefixSums<Tindex>(early_seq_lens, early_num_seqs, early_max_blocks_per_seq,
+                                                   early_block_shift, lane, pre_incl);
     PA_STAMP(1);
     // The flat range is not cut into equal tile counts but into equal COST: a sequence that begins inside
     // a piece costs its wavefront about as much time as kStartCost more tiles would (measured: pieces with
@@ -501,7 +509,8 @@ decodeBalancedKernel(DecodeArgs a, int waves_per_stream) {
 // range of the sequence was left in seq_pieces by the decode kernel, so the only dependent memory
 // round trips are {length, piece range} -> rows (one trip for up to eight segments).
 template <typename T, typename Tindex, int HEAD>
-__global__ void __launch_bounds__(256) decodeBalancedMergeKernel(DecodeArgs a) {
+__global__ void __launch_bounds__(256)
+decodeBalancedMergeKernel(const void *early_seq_lens, const int2 *early_seq_pieces, int early_num_heads, DecodeArgs a) {
     using S = typename T::storage;
     constexpr int kCols = TileGeometry<HEAD>::kCols;
     const int head = blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -509,11 +518,12 @@ __global__ void __launch_bounds__(256) decodeBalancedMergeKernel(DecodeArgs a) {
     const int lane = threadIdx.x & 63;
     const int c = lane & 15;
     const int g = lane >> 4;
-    if (head >= a.num_heads) {
+    // (the early arguments repeat a.seq_lens, a.seq_pieces and a.num_heads: see decodeBalancedKernel)
+    if (head >= early_num_heads) {
         return;
     }
-    const int64_t len64 = loadIndex<Tindex>(a.seq_lens, seq);
-    const int2 pieces = a.seq_pieces[seq]; // written by the decode kernel for every sequence with tokens
+    const int64_t len64 = loadIndex<Tindex>(early_seq_lens, seq);
+    const int2 pieces = early_seq_pieces[seq]; // written by the decode kernel for every sequence with tokens
     if (len64 <= 0 || pieces.y <= 1) {
         return; // no tokens, or one segment covered the whole sequence and wrote `out` itself
     }

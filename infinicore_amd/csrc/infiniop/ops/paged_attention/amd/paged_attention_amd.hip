@@ -219,8 +219,10 @@ void launchTiled(const DecodeArgs &a, const Plan &plan, hipStream_t stream) {
     const int head_chunks = (a.group + kHeadsPerWave - 1) / kHeadsPerWave;
     if (plan.balanced) {
         const dim3 grid(plan.waves_per_stream, a.num_kv_heads * head_chunks);
-        decodeBalancedKernel<T, Tindex, HEAD><<<grid, 64, 0, stream>>>(a, plan.waves_per_stream);
-        decodeBalancedMergeKernel<T, Tindex, HEAD><<<dim3((a.num_heads + 3) / 4, a.num_seqs), 256, 0, stream>>>(a);
+        decodeBalancedKernel<T, Tindex, HEAD><<<grid, 64, 0, stream>>>(a.seq_lens, a.num_seqs, a.max_blocks_per_seq,
+                                                                       a.block_shift, a, plan.waves_per_stream);
+        decodeBalancedMergeKernel<T, Tindex, HEAD><<<dim3((a.num_heads + 3) / 4, a.num_seqs), 256, 0, stream>>>(
+            a.seq_lens, a.seq_pieces, a.num_heads, a);
     } else {
         const dim3 grid(plan.max_partitions, a.num_kv_heads * head_chunks, a.num_seqs);
         decodeTiledKernel<T, Tindex, HEAD><<<grid, 64, 0, stream>>>(a);

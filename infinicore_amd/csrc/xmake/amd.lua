@@ -87,6 +87,8 @@ target("infiniop-amd")
     add_files("../src/infiniop/devices/amd/*.cc")
     add_files("../src/infiniop/ops/paged_caching/amd/*.hip", "../src/infiniop/ops/kv_caching/amd/*.hip")
     -- the attention kernels keep their matrix-instruction accumulators in ordinary vector registers
-    add_files("../src/infiniop/ops/paged_attention/amd/*.hip", "../src/infiniop/ops/paged_attention_prefill/amd/*.hip",
-              {cxflags = {"-mllvm", "-amdgpu-mfma-vgpr-form=1"}})
+    add_files("../src/infiniop/ops/paged_attention_prefill/amd/*.hip", {cxflags = {"-mllvm", "-amdgpu-mfma-vgpr-form=1"}})
+    -- decode also gets the first five argument words of its work-equalising kernels in scalar registers at wavefront start
+    add_files("../src/infiniop/ops/paged_attention/amd/*.hip",
+              {cxflags = {"-mllvm", "-amdgpu-mfma-vgpr-form=1", "-mllvm", "-amdgpu-kernarg-preload-count=5"}})
 target_end()
