@@ -85,7 +85,9 @@ target("infiniop-amd")
     add_links("amdhip64")
     add_cxflags("-fPIC")
     add_files("../src/infiniop/devices/amd/*.cc")
-    add_files("../src/infiniop/ops/paged_caching/amd/*.hip", "../src/infiniop/ops/kv_caching/amd/*.hip")
+    add_files("../src/infiniop/ops/kv_caching/amd/*.hip")
+    -- the scatter kernel gets its first 14 argument words in scalar registers at wavefront start
+    add_files("../src/infiniop/ops/paged_caching/amd/*.hip", {cxflags = {"-mllvm", "-amdgpu-kernarg-preload-count=14"}})
     -- the attention kernels keep their matrix-instruction accumulators in ordinary vector registers
     add_files("../src/infiniop/ops/paged_attention_prefill/amd/*.hip", {cxflags = {"-mllvm", "-amdgpu-mfma-vgpr-form=1"}})
     -- decode also gets the first five argument words of its work-equalising kernels in scalar registers at wavefront start
