@@ -39,7 +39,7 @@ MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 / fp16 matrix peak
 # file, each scaled by what the same counter reads for a 256 MiB copy (summaries and commands: profiles/).
 # Counters cannot be read from inside this process, so the figures are recorded here, per workload.
 MEASURED_TRAFFIC_BYTES = {
-    "c2_llama3_8b_b32": 322_400_000,       # decodeBalancedKernel: 319.8 MB fetched + 2.6 MB written
+    "c2_llama3_8b_b32": 322_300_000,       # decodeBalancedKernel: 319.7 MB fetched + 2.6 MB written
     "m1_mla_16_heads_b32": 155_000_000,    # decodeMlaWideKernel<.., 1>: 146.4 MB fetched + 8.6 MB written
     "m2_mla_128_heads_b32": 215_500_000,   # decodeMlaWideKernel: 184.1 MB fetched + 31.4 MB written
     "c5_prefill_scatter": 32_100_000,      # pagedCachingScatterKernel: 16.2 MB fetched + 15.9 MB written
