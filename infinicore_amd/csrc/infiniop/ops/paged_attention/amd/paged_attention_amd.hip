@@ -151,8 +151,9 @@ Plan makePlan(const PagedAttentionInfo &in, const device::amd::DeviceInfo &dev) 
         }
     }
     if (plan.balanced) {
-        // head 64 moves half the bytes per tile with half the registers: two wavefronts per SIMD measured best there
-        int waves_per_cu = in.head_size == 64 ? 8 : 4;
+        // one wavefront per SIMD at every head size (head 64, half the bytes per tile, ran two per SIMD until
+        // its matrix results stayed in vector registers: now 33.3 us with four per compute unit, 34.0 - 34.7 with eight)
+        int waves_per_cu = 4;
         if (const char *env = std::getenv("INFINIOP_AMD_PA_WAVES_PER_CU")) {
             const int forced = std::atoi(env);
             waves_per_cu = forced >= 1 && forced <= 64 ? forced : waves_per_cu;
