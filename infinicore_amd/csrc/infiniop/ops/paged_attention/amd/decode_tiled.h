@@ -100,8 +100,9 @@ struct TileGeometry {
     static constexpr int kSwizzle = (HEAD == 64 || HEAD == 192) ? 8 : 16;
     static constexpr int kCols = HEAD / 16;           // V / output columns per lane
     static constexpr int kWords = kCols / 2;          // dwords of one V row strip
-    // register sets in flight: about 16 KiB of requests per wavefront whatever the head size
-    static constexpr int kBuffers = HEAD == 64 ? 5 : (HEAD == 256 ? 2 : 3);
+    // register sets: about 16 KiB of requests in flight per wavefront (12 KiB at head 192, where a third set
+    // pushed the kernel out of the vector register file: 91.5 -> 90.9 us at the c2 shape with two)
+    static constexpr int kBuffers = HEAD == 64 ? 5 : (HEAD >= 192 ? 2 : 3);
     static __device__ __forceinline__ int kRow(int j, int lane) { return (64 * j + lane) / kChunksPerRow; }
     static __device__ __forceinline__ int kChunk(int j, int lane) { return (64 * j + lane) % kChunksPerRow; }
     // position (in 16-byte units) of chunk `chunk` of row `row` in the LDS tile
