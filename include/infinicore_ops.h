@@ -73,7 +73,8 @@ __INFINI_C __export infiniStatus_t infinicoreOpPlanKVCaching(
 
 /* ---- run (paged_attention_infiniop.cc:48-63): one InfiniOP call on `stream`; allocates nothing, so it
  *      may be recorded into a captured graph. Runs of one plan share its workspace: order them on one
- *      stream (or by events). ---- */
+ *      stream (or by events). The calling thread's current InfiniRT device must be the one the plan was
+ *      made on, else INFINI_STATUS_BAD_PARAM. ---- */
 __INFINI_C __export infiniStatus_t infinicoreOpRun(infinicorePlannedOp_t plan, infinirtStream_t stream);
 /* ---- cleanup (paged_attention_infiniop.cc:65-68): frees the plan's workspace (which waits for the
  *      device), drops its reference to the descriptor, sets *plan_ptr to NULL. ---- */

@@ -182,6 +182,7 @@ infiniStatus_t getOrCreate(infinicoreOpKind_t kind, const MetaKey &key, const Cr
 
 struct InfinicorePlannedOp {
     std::shared_ptr<Descriptor> descriptor;
+    infiniDevice_t device = INFINI_DEVICE_CPU;
     int device_id = 0;
     Workspace workspace;
     CallFn call; // holds the tensors' data pointers
@@ -190,14 +191,15 @@ struct InfinicorePlannedOp {
 namespace {
 
 // plan = descriptor + a workspace of the plan's own (INFINIOP_WORKSPACE_TENSOR, infiniop_impl.hpp:68-76)
-infiniStatus_t makePlan(infinicorePlannedOp_t *plan_ptr, std::shared_ptr<Descriptor> descriptor, int device_id,
-                        CallFn call) {
+infiniStatus_t makePlan(infinicorePlannedOp_t *plan_ptr, std::shared_ptr<Descriptor> descriptor, infiniDevice_t device,
+                        int device_id, CallFn call) {
     auto plan = std::make_unique<InfinicorePlannedOp>();
     if (descriptor->workspace_bytes != 0) {
         RETURN_IF_ERROR(infinirtMalloc(&plan->workspace.ptr, descriptor->workspace_bytes));
         plan->workspace.bytes = descriptor->workspace_bytes;
     }
     plan->descriptor = std::move(descriptor);
+    plan->device = device;
     plan->device_id = device_id;
     plan->call = std::move(call);
     *plan_ptr = plan.release();
@@ -347,7 +349,7 @@ infiniStatus_t prepareKVCaching(Prepared *p, const infinicoreTensorView_t *k_cac
 
 infiniStatus_t finishPlan(infinicorePlannedOp_t *plan_ptr, infiniStatus_t prepared, Prepared &p) {
     RETURN_IF_ERROR(prepared);
-    return makePlan(plan_ptr, std::move(p.descriptor), p.device_id, std::move(p.call));
+    return makePlan(plan_ptr, std::move(p.descriptor), p.device, p.device_id, std::move(p.call));
 }
 
 infiniStatus_t finishImmediate(infiniStatus_t prepared, const Prepared &p, infinirtStream_t stream) {
@@ -410,6 +412,14 @@ __INFINI_C infiniStatus_t infinicoreOpPlanKVCaching(
 __INFINI_C infiniStatus_t infinicoreOpRun(infinicorePlannedOp_t plan, infinirtStream_t stream) {
     if (plan == nullptr) {
         return INFINI_STATUS_NULL_POINTER;
+    }
+    // the plan's workspace, tensors and stream belong to the device it was planned on: that device must be
+    // the calling thread's current one (the reference's graph runs on the context's current device too)
+    infiniDevice_t device = INFINI_DEVICE_CPU;
+    int device_id = 0;
+    RETURN_IF_ERROR(infinirtGetDevice(&device, &device_id));
+    if (device != plan->device || device_id != plan->device_id) {
+        return INFINI_STATUS_BAD_PARAM;
     }
     return plan->call(plan->descriptor->desc, plan->workspace.ptr, plan->workspace.bytes, stream);
 }

@@ -165,6 +165,7 @@ class PlannedOp:
 
     def run(self, stream: torch.cuda.Stream | None = None) -> None:
         s = stream if stream is not None else torch.cuda.current_stream(self._device_index)
+        lib.set_device(InfiniDevice.AMD, self._device_index)  # a plan runs on the device it was made on only
         check_error(LIBINFINICORE_OPS.infinicoreOpRun(self._handle, c_void_p(s.cuda_stream)), "infinicoreOpRun")
 
     def cleanup(self) -> None:

@@ -78,7 +78,7 @@ def test_immediate_workspace_grows_with_the_larger_call(core, oracle):
         assert close(out, want), inp.config.name
 
 
-def test_plan_run_cleanup_and_graph_replay(core, oracle):
+def test_plan_run_cleanup_and_graph_replay(core, oracle, lib):
     print("case plan / run / cleanup", flush=True)
     inp, (q, k, v, bt, sl), want = decode_case(oracle, "plan", torch.bfloat16, 8, 32, 8, 128, 100, 2500, 74)
     out = torch.zeros_like(q)
@@ -110,6 +110,12 @@ def test_plan_run_cleanup_and_graph_replay(core, oracle):
         plan_b.run()
         torch.cuda.synchronize()
         assert torch.equal(bits(out_b), bits(eager)), f"second plan after replay {replay}"
+    # a plan runs on the device it was made on only
+    import ctypes
+    lib.set_device(lib.InfiniDevice.CPU, 0)
+    status = core.LIBINFINICORE_OPS.infinicoreOpRun(plan._handle, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    lib.set_device(lib.InfiniDevice.AMD, 0)
+    assert status == lib.InfiniStatus.BAD_PARAM
     # the cache forgets the descriptor; the plans keep it alive
     core.cache_clear()
     assert core.cache_stats(core.OpKind.PAGED_ATTENTION)[0] == 0
