@@ -25,20 +25,6 @@
 
 namespace op::paged_attention::amd {
 
-#ifdef INFINIOP_AMD_PA_TRACE
-// Diagnostic build only: per-wavefront timestamps (100 MHz constant clock) of the decode phases.
-__device__ unsigned long long *g_pa_trace = nullptr;
-#define PA_STAMP(slot)                                                                                   \
-    do {                                                                                                 \
-        if (g_pa_trace != nullptr && threadIdx.x == 0) {                                                 \
-            g_pa_trace[(static_cast<size_t>(blockIdx.y) * gridDim.x + blockIdx.x) * 8 + (slot)] = __builtin_amdgcn_s_memrealtime(); \
-        }                                                                                                \
-    } while (0)
-#else
-#define PA_STAMP(slot) do {} while (0)
-#endif
-
-constexpr int kBalancedMaxSeqs = 1024; // prefix sums of the batch live in LDS
 constexpr int kBalancedMinTiles = 4;   // never cut pieces finer than 64 tokens
 
 // Inclusive prefix sum over the 64 lanes with data-parallel-primitive moves (no LDS-unit permutes: this
@@ -148,17 +134,8 @@ decodeBalancedKernel(const void *early_seq_lens, int early_num_seqs, int early_m
     const int c = lane & 15;
     const int g = lane >> 4;
 
-    PA_STAMP(0);
-#ifdef INFINIOP_AMD_PA_TRACE
-    if (g_pa_trace != nullptr && threadIdx.x == 0) {
-        const size_t w = static_cast<size_t>(blockIdx.y) * gridDim.x + blockIdx.x;
-        g_pa_trace[w * 8 + 6] = __builtin_amdgcn_s_getreg(63492); // HW_ID
-        g_pa_trace[w * 8 + 7] = __builtin_amdgcn_s_getreg(63508); // XCC_ID
-    }
-#endif
     const int total_tiles = tilePrefixSums<Tindex>(early_seq_lens, early_num_seqs, early_max_blocks_per_seq,
                                                    early_block_shift, lane, pre_incl);
-    PA_STAMP(1);
     // The flat range is not cut into equal tile counts but into equal COST: a sequence that begins inside
     // a piece costs its wavefront about as much time as kStartCost more tiles would (measured: pieces with
     // such a start finish level with the others when they hold three to four tiles fewer at head 128), and they were
@@ -166,6 +143,7 @@ decodeBalancedKernel(const void *early_seq_lens, int early_num_seqs, int early_m
     // equal ranges of that axis, and a piece's tiles are the real tiles its range covers: tile i of
     // sequence s sits at virtual position (tiles before s) + i + kStartCost * (s + 1).
     constexpr int kStartCost = HEAD <= 128 ? 384 / HEAD : 2;
+    static_assert(kStartCost <= kBalancedMaxStartCost, "the launch plan bounds the flat axis with this");
     const int q = tilesPerPiece(total_tiles + kStartCost * a.num_seqs, waves_per_stream);
     // Real tiles below virtual positions x0 = piece * q and x1 = x0 + q: count the sequences that lie
     // entirely below each (one pass over the prefix sums for both), then add the part of the next one.
@@ -431,7 +409,6 @@ decodeBalancedKernel(const void *early_seq_lens, int early_num_seqs, int early_m
                              min(kTileTokens, c_len - tok0));
         if (++c_t == c_seg_end) {
             if (next_seq >= 0) {
-                PA_STAMP(3);
                 // The next sequence's query and length were asked for when this segment began.
                 const int next_len = clampLength(len_next);
 #pragma unroll
@@ -445,7 +422,6 @@ decodeBalancedKernel(const void *early_seq_lens, int early_num_seqs, int early_m
                 const int flat = seqFirstTile(c_seq) + c_seg_end;
                 parkSegment();
                 beginSegment(next_seq, flat, next_len);
-                PA_STAMP(5);
             }
         }
     };
@@ -472,7 +448,6 @@ decodeBalancedKernel(const void *early_seq_lens, int early_num_seqs, int early_m
     }
     // The first tiles are requested before the first query: the query's round trip then overlaps
     // with theirs.
-    PA_STAMP(2);
     const int n_flat = f1 - f0;
     TileRegs<HEAD> buf[NBUF];
 #pragma unroll
@@ -499,7 +474,6 @@ decodeBalancedKernel(const void *early_seq_lens, int early_num_seqs, int early_m
     if (stash_seq >= 0) {
         flushStash();
     }
-    PA_STAMP(4);
 }
 
 // Merge of the segment rows of one (query head, sequence); see decode_reduce.h for the arithmetic.

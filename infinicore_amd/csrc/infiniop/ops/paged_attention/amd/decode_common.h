@@ -3,6 +3,7 @@
 #ifndef INFINICORE_AMD_PA_DECODE_COMMON_H
 #define INFINICORE_AMD_PA_DECODE_COMMON_H
 
+#include "decode_plan.h"
 #include <cstdint>
 #include <hip/hip_runtime.h>
 

@@ -40,8 +40,6 @@
 
 namespace op::paged_attention::amd {
 
-constexpr int kMlaKeySize = 576;
-constexpr int kMlaValueSize = 512;
 constexpr int kMlaThreads = 128; // two wavefronts per unit of work
 
 struct MlaGeometry {
@@ -57,17 +55,6 @@ struct MlaGeometry {
     static __device__ __forceinline__ int kChunk(int j, int lane) { return (64 * j + lane) % kChunksPerRow; }
     static __device__ __forceinline__ int ldsIndex(int row, int chunk) { return row * kLdsPitch + chunk; }
 };
-
-#ifdef INFINIOP_AMD_PA_TRACE
-#define MLA_STAMP(slot)                                                                                   \
-    do {                                                                                                 \
-        if (g_pa_trace != nullptr && threadIdx.x == 0) {                                                 \
-            g_pa_trace[((static_cast<size_t>(blockIdx.z) * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * 8 + (slot)] = __builtin_amdgcn_s_memrealtime(); \
-        }                                                                                                \
-    } while (0)
-#else
-#define MLA_STAMP(slot) do {} while (0)
-#endif
 
 template <typename T, typename Tindex>
 __global__ void __launch_bounds__(kMlaThreads, 2) decodeMlaKernel(DecodeArgs a) {
@@ -89,7 +76,6 @@ __global__ void __launch_bounds__(kMlaThreads, 2) decodeMlaKernel(DecodeArgs a) 
     const int c = lane & 15; // column strip / head within the chunk / token for the K operand
     const int g = lane >> 4; // group of four tokens
 
-    MLA_STAMP(0);
     // Everything up to the first barrier depends on the unit only, so both wavefronts leave together.
     const int64_t len64 = loadIndex<Tindex>(a.seq_lens, seq);
     if (len64 <= 0) {
@@ -189,7 +175,6 @@ __global__ void __launch_bounds__(kMlaThreads, 2) decodeMlaKernel(DecodeArgs a) 
 
     uint4 k[G::kLoads];
     uint32_t v[4][4 * G::kStrips];
-    MLA_STAMP(1);
     loadK(0, k);
 #pragma unroll
     for (int i = 0; i < G::kStrips; ++i) {
@@ -224,12 +209,6 @@ __global__ void __launch_bounds__(kMlaThreads, 2) decodeMlaKernel(DecodeArgs a) 
         }
     }
 
-    MLA_STAMP(2);
-#ifdef INFINIOP_AMD_PA_TRACE
-    if (g_pa_trace != nullptr && threadIdx.x == 0) {
-        g_pa_trace[((static_cast<size_t>(blockIdx.z) * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * 8 + 5] = n_tiles;
-    }
-#endif
     // Epilogue. Denominator of head c over all 16 token slots, then move per-head scalars to the
     // lanes that hold that head's accumulators.
     const float l_tot = sumAcrossTokenGroups(l);
@@ -271,7 +250,6 @@ __global__ void __launch_bounds__(kMlaThreads, 2) decodeMlaKernel(DecodeArgs a) 
             }
         }
     }
-    MLA_STAMP(3);
 }
 
 // ---- many query heads per KV head ---------------------------------------------------------------------
@@ -292,7 +270,6 @@ __global__ void __launch_bounds__(kMlaThreads, 2) decodeMlaKernel(DecodeArgs a) 
 //     registers; P . V as 32-deep matrix instructions). Two workgroup barriers per tile.
 // Partial results and their merge are those of the kernel above.
 constexpr int kMlaWideThreads = 512;
-constexpr int kMlaWideChunks = 4;      // head chunks of 16 per workgroup
 constexpr int kMlaWideTileTokens = 32; // two halves of 16
 
 // Online-softmax step of one 32-token tile. s0 / s1 = raw scores of head c for tokens 4g..4g+3 of the

@@ -80,9 +80,8 @@ struct TileF16 : Half {
     }
 };
 
-constexpr int kTileTokens = 16;     // tokens per tile = rows of one matrix instruction
+// (kTileTokens = 16 tokens per tile and kHeadsPerWave = 16 query heads per wavefront: decode_plan.h)
 constexpr int kTiledHead = 128;     // the head size the kernels were tuned on (others: 64, 192, 256)
-constexpr int kHeadsPerWave = 16;   // query heads of one KV head packed into one wavefront
 constexpr float kLazyRescaleLog2 = 8.0f; // how far (in powers of two) a maximum may outgrow its reference point
 
 // Geometry of a 16-token tile for head_size = value_size = HEAD (64, 128, 192 or 256).

@@ -1,0 +1,102 @@
+"""The decode launch plan (decode_plan.h) on the host: partitions never span more block-table entries than a
+wavefront holds, the work-equalising schedule is only chosen where its 32-bit tile axis fits, and the workspace
+is sized for that schedule alone (the element-wise fallback is cut to fit it)."""
+import ctypes
+import subprocess
+from pathlib import Path
+
+import pytest
+
+ROOT = Path(__file__).resolve().parents[1]
+KNOBS = ("INFINIOP_AMD_PA_KERNEL", "INFINIOP_AMD_PA_SCHEDULE", "INFINIOP_AMD_PA_LATENT_KERNEL",
+         "INFINIOP_AMD_PA_PARTITION", "INFINIOP_AMD_PA_WAVES_PER_CU")
+FIELDS = ("tiled", "balanced", "latent_wide", "partition_tokens", "max_partitions", "fallback_partition_tokens",
+          "fallback_max_partitions", "waves_per_stream", "workspace_bytes", "launchable")
+
+
+@pytest.fixture(scope="module")
+def probe(tmp_path_factory):
+    out = tmp_path_factory.mktemp("plan") / "libplanprobe.so"
+    subprocess.run(["g++", "-std=c++17", "-O1", "-shared", "-fPIC", f"-I{ROOT / 'include'}",
+                    f"-I{ROOT / 'infinicore_amd' / 'csrc'}", str(ROOT / "tests" / "plan_probe.cc"), "-o", str(out)],
+                   check=True, capture_output=True, text=True)
+    lib = ctypes.CDLL(str(out))
+    lib.planProbe.argtypes = [ctypes.POINTER(ctypes.c_longlong), ctypes.POINTER(ctypes.c_longlong)]
+    lib.planProbe.restype = None
+
+    def plan(num_seqs, num_heads, num_kv_heads, head_size, block_size, max_blocks, value_size=0, num_blocks=1 << 20,
+             compute_units=256):
+        args = (ctypes.c_longlong * 9)(num_seqs, num_heads, num_kv_heads, head_size, value_size or head_size, block_size,
+                                      max_blocks, num_blocks, compute_units)
+        res = (ctypes.c_longlong * len(FIELDS))()
+        lib.planProbe(args, res)
+        return dict(zip(FIELDS, res))
+
+    return plan
+
+
+@pytest.fixture(autouse=True)
+def no_knobs(monkeypatch):
+    for k in KNOBS:
+        monkeypatch.delenv(k, raising=False)
+
+
+def entries_spanned(p, bs, k):
+    """Block-table entries partition k (tokens [k p, (k + 1) p)) touches."""
+    return ((k + 1) * p - 1) // bs - (k * p) // bs + 1
+
+
+@pytest.mark.parametrize("bs", [16, 32, 64, 128, 256])
+def test_partitions_fit_one_page_id_load(probe, monkeypatch, bs):
+    """Every partition of the tiled kernels must lie inside 64 consecutive block-table entries, for the planned
+    size, for the size grown to bound the workspace (very wide tables) and for any forced size."""
+    monkeypatch.setenv("INFINIOP_AMD_PA_SCHEDULE", "grid")
+    widths = [1, 7, 64, 513, 8129, 8130, 8160, 8161, 8192, 8097, 8184, 70000]
+    for forced in (None, 16, 48, 1000, 4080, 4081, 5000, 100000):
+        if forced is None:
+            monkeypatch.delenv("INFINIOP_AMD_PA_PARTITION", raising=False)
+        else:
+            monkeypatch.setenv("INFINIOP_AMD_PA_PARTITION", str(forced))
+        for width in widths:
+            for heads, kv, head_size, value in ((32, 8, 128, 0), (128, 1, 576, 512), (16, 1, 576, 512)):
+                pl = probe(4, heads, kv, head_size, bs, width, value_size=value)
+                assert pl["tiled"]
+                p = pl["partition_tokens"]
+                assert pl["max_partitions"] == -(-width * bs // p)
+                worst = max(entries_spanned(p, bs, k) for k in range(min(pl["max_partitions"], 4096)))
+                assert worst <= 64, (bs, width, forced, p, worst)
+
+
+def test_advisor_case_pages_of_64_table_of_8160(probe, monkeypatch):
+    """Pages of 64 tokens, a table 8160 wide: the grown size used to be 4080 tokens (not a multiple of the
+    page), whose second partition spans 65 entries."""
+    monkeypatch.setenv("INFINIOP_AMD_PA_SCHEDULE", "grid")
+    pl = probe(2, 32, 8, 128, 64, 8160)
+    assert pl["partition_tokens"] % 64 == 0 and pl["partition_tokens"] <= 64 * 64
+
+
+def test_work_equalising_schedule_needs_its_flat_axis_in_32_bits(probe):
+    wide = probe(1024, 32, 8, 128, 16, 1 << 20)  # 1024 sequences x 2^20 tiles
+    assert wide["tiled"] and not wide["balanced"]
+    usual = probe(32, 32, 8, 128, 16, 256)
+    assert usual["balanced"] and usual["waves_per_stream"] == 128
+
+
+def test_workspace_is_that_of_the_chosen_schedule(probe):
+    """c2: (128 pieces + 32 sequences) rows x 32 heads x (128 + 2) floats, plus the piece table and alignment
+    slack - below the reference's 8 * B * H * (D + 2) * 4 = 4.26 MB."""
+    c2 = probe(32, 32, 8, 128, 16, 256)
+    rows = 128 + 32
+    assert c2["workspace_bytes"] == rows * 32 * 128 * 4 + 2 * rows * 32 * 4 + 256 + 256
+    assert c2["workspace_bytes"] < 8 * 32 * 32 * 130 * 4
+    # the element-wise fallback (operands that are not 16-byte aligned at run time) fits the same rows
+    assert c2["fallback_max_partitions"] * 32 <= rows
+    assert c2["fallback_partition_tokens"] * c2["fallback_max_partitions"] >= 256 * 16
+    c4 = probe(128, 64, 8, 128, 16, 512)
+    assert c4["balanced"] and c4["fallback_max_partitions"] * 128 <= 128 + 128
+
+
+def test_shapes_beyond_the_launch_limits_are_not_launchable(probe):
+    assert probe(65535, 8, 8, 128, 16, 4)["launchable"]
+    assert not probe(65536, 8, 8, 128, 16, 4)["launchable"]
+    assert not probe(4, 65536, 65536, 128, 16, 4)["launchable"]

@@ -95,7 +95,12 @@ def custom(name, dtype, B, H, Hkv, D, bs, lo, hi, seed, **kw):
 
 # ---- the benchmark configurations -------------------------------------------------------------------
 
-def test_c1_plumbing_mha_against_oracle_and_committed_fixture(gpu_handle, oracle):
+@pytest.mark.parametrize("schedule", [None, "balanced"], ids=["default_schedule", "balanced"])
+def test_c1_plumbing_mha_against_oracle_and_committed_fixture(gpu_handle, oracle, monkeypatch, schedule):
+    """c1 under the schedule the library picks for it by itself (a small job: fixed partitions) and under the
+    work-equalising one."""
+    if schedule is None:
+        monkeypatch.delenv("INFINIOP_AMD_PA_SCHEDULE", raising=False)
     inp = workloads.make_decode_inputs(workloads.DECODE_CONFIGS["c1_plumbing_mha"])
     got, _ = run_case(gpu_handle, oracle, inp)
     from pathlib import Path
@@ -134,6 +139,36 @@ def test_c4_70b_share_full_size(gpu_handle, oracle):
 )
 def test_reference_test_shapes(gpu_handle, oracle, dtype, B, H, Hkv, D, bs, max_len):
     cfg = custom(f"ref_{B}_{H}_{Hkv}_{D}", dtype, B, H, Hkv, D, bs, 1, max_len - 1, seed=7 * B + H + D)
+    run_case(gpu_handle, oracle, workloads.make_decode_inputs(cfg))
+
+
+@pytest.mark.parametrize("schedule", [None, "balanced"], ids=["default_schedule", "balanced"])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize(
+    "B,H,Hkv,D,bs,max_len,Dv",
+    [
+        # test/infinicore/ops/paged_attention.py:22-38, literally: (num_seqs, num_heads, num_kv_heads, head_size,
+        # block_size, max_seq_len[, value_size]); lengths are drawn from [1, max_seq_len) as that test does (:71)
+        (1, 1, 1, 128, 16, 15, 0),
+        (4, 40, 40, 128, 16, 1024, 0),
+        (6, 40, 40, 128, 16, 1024, 0),
+        (3, 8, 8, 128, 16, 1024, 0),
+        (3, 8, 8, 64, 16, 1024, 0),
+        (8, 64, 8, 128, 16, 2048, 0),
+        (1, 24, 4, 256, 16, 32, 0),
+        (1, 12, 2, 256, 16, 32, 0),
+        (1, 6, 1, 256, 16, 32, 0),
+        (1, 16, 1, 576, 16, 32, 512),
+    ],
+)
+def test_reference_framework_test_shapes(gpu_handle, oracle, monkeypatch, dtype, B, H, Hkv, D, bs, max_len, Dv, schedule):
+    """The shape list of the reference's framework-level test (groups of 6 query heads at head 256, a sequence
+    shorter than one page, the latent-attention wrapper case), under the schedule the library picks by itself
+    and under the work-equalising one (which the latent shape does not have: it runs its own kernels twice)."""
+    if schedule is None:
+        monkeypatch.delenv("INFINIOP_AMD_PA_SCHEDULE", raising=False)
+    cfg = custom(f"fw_{B}_{H}_{Hkv}_{D}_{max_len}", dtype, B, H, Hkv, D, bs, 1, max_len - 1, seed=11 * B + H + D + max_len,
+                 value_size=Dv)
     run_case(gpu_handle, oracle, workloads.make_decode_inputs(cfg))
 
 
@@ -404,6 +439,18 @@ def test_grid_schedule_partition_sizes(gpu_handle, oracle, monkeypatch, partitio
     run_case(gpu_handle, oracle, workloads.make_decode_inputs(custom("part", torch.bfloat16, 4, 16, 4, 128, 16, 1, 2500, seed=3)))
 
 
+@pytest.mark.parametrize("heads,D,Dv", [(16, 128, 0), (16, 576, 512), (48, 576, 512)])
+def test_partitions_of_large_pages_stay_inside_one_page_id_load(gpu_handle, oracle, monkeypatch, heads, D, Dv):
+    """Pages of 64 tokens and a requested partition of 4080 tokens (not a multiple of the page): the plan rounds
+    it to whole pages, so that partition 1 of a sequence of more than 8200 tokens does not start inside a page
+    and need a 65th block-table entry. Fixed partitions, all three tiled kernel families."""
+    monkeypatch.setenv("INFINIOP_AMD_PA_SCHEDULE", "grid")
+    monkeypatch.setenv("INFINIOP_AMD_PA_PARTITION", "4080")
+    cfg = custom(f"bigpages_{heads}_{D}", torch.bfloat16, 2, heads, 1 if D == 576 else 4, D, 64, 8300, 8900, seed=83,
+                 value_size=Dv)
+    run_case(gpu_handle, oracle, workloads.make_decode_inputs(cfg))
+
+
 @pytest.mark.parametrize("waves_per_cu", [1, 2, 8, 16])
 def test_balanced_schedule_any_piece_count(gpu_handle, oracle, monkeypatch, waves_per_cu):
     monkeypatch.setenv("INFINIOP_AMD_PA_WAVES_PER_CU", str(waves_per_cu))
@@ -484,6 +531,25 @@ def test_unaligned_base_addresses_take_the_elementwise_kernel(gpu_handle, oracle
 
     got = run_paged_attention(gpu_handle, shifted(q), shifted(k), shifted(v), bt, sl, inp.scale)
     assert_close(got, oracle_of(oracle, inp), "unaligned")
+
+
+def test_unaligned_operands_of_a_large_job_fit_the_planned_workspace(gpu_handle, oracle):
+    """A descriptor planned for the work-equalising schedule sizes the workspace for that schedule; when the
+    operands of a call are not 16-byte aligned the element-wise kernel runs on partitions cut to fit it."""
+    inp = workloads.make_decode_inputs(custom("unaligned_big", torch.bfloat16, 12, 8, 2, 128, 16, 100, 3000, seed=38))
+    q, k, v, bt, sl = to_device(inp)
+
+    def shifted(t):
+        flat = torch.zeros(t.numel() + 1, dtype=t.dtype, device=DEV)
+        view = flat[1:].view(t.shape)
+        view.copy_(t)
+        return view
+
+    aligned = run_paged_attention(gpu_handle, q, k, v, bt, sl, inp.scale)
+    got = run_paged_attention(gpu_handle, shifted(q), k, v, bt, sl, inp.scale)
+    want, want_f32 = oracle_of(oracle, inp, return_fp32=True)
+    assert_close(aligned, want, "aligned", want_f32)
+    assert_close(got, want, "unaligned_big", want_f32)
 
 
 # ---- what must not be read, what must not be written -------------------------------------------------

@@ -133,6 +133,28 @@ def test_paged_attention_descriptor_owns_its_metadata_and_reports_device(lib, ho
     assert lib.LIBINFINIOP.infiniopDestroyPagedAttentionDescriptor(None) == NULLP
 
 
+def test_paged_attention_shapes_beyond_one_launch_are_refused_at_creation(lib, host_amd_handle):
+    """Sequences and heads sit on the y / z axes of some launches (limit 65535 each): larger batches are
+    answered with BAD_TENSOR_SHAPE when the descriptor is made, not with a failed launch later."""
+    status, op = create_attention(lib, host_amd_handle, attention_specs(B=65535, NB=4, maxb=2))
+    assert status == OK
+    lib.check_error(lib.LIBINFINIOP.infiniopDestroyPagedAttentionDescriptor(op))
+    status, _ = create_attention(lib, host_amd_handle, attention_specs(B=65536, NB=4, maxb=2))
+    assert status == BAD_SHAPE
+
+
+def test_paged_attention_workspace_is_sized_for_the_planned_schedule(lib, host_amd_handle):
+    """The Llama-3-8B batch-32 decode shape: (128 pieces + 32 sequences) rows of partial results, 2.7 MB - less
+    than the 8 * B * H * (D + 2) * 4 = 4.26 MB of the reference's nvidia backend."""
+    specs = attention_specs(B=32, H=32, Hkv=8, NB=5400, maxb=256, dtype=BF16)
+    status, op = create_attention(lib, host_amd_handle, specs)
+    assert status == OK
+    size = ctypes.c_size_t(0)
+    lib.check_error(lib.LIBINFINIOP.infiniopGetPagedAttentionWorkspaceSize(op, ctypes.byref(size)))
+    assert 2_600_000 < size.value < 2_700_000
+    lib.check_error(lib.LIBINFINIOP.infiniopDestroyPagedAttentionDescriptor(op))
+
+
 def test_paged_attention_null_arguments(lib, host_amd_handle):
     t = lib.create_tensor_descriptor((4, 8, 128), None, F16)
     op = lib.infiniopOperatorDescriptor_t()
