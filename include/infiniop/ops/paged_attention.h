@@ -69,6 +69,25 @@ __INFINI_C __export infiniStatus_t infiniopPagedAttention(
     const void *alibi_slopes,
     void *stream);
 
+/* infiniopPagedAttention without the workspace argument, for callers that cannot allocate device memory
+ * (code under stream capture that owns no buffer, serving loops and harnesses that forbid allocation).
+ * It has no counterpart in the reference. The partial results go to an array of 32 MiB that the library
+ * itself holds on every GPU it runs on; a descriptor whose workspace size (see above) exceeds that is
+ * answered with INSUFFICIENT_WORKSPACE and a message on stderr. It calls no allocator. All calls on one GPU
+ * share the array: calls that overlap there (two streams, two threads) race; calls on one stream are
+ * ordered and safe. The calling thread's current device must be the descriptor's. Results are those of
+ * infiniopPagedAttention, bit for bit. */
+__INFINI_C __export infiniStatus_t infiniopPagedAttentionNoAlloc(
+    infiniopPagedAttentionDescriptor_t desc,
+    void *out,
+    const void *q,
+    const void *k_cache,
+    const void *v_cache,
+    const void *block_tables,
+    const void *seq_lens,
+    const void *alibi_slopes,
+    void *stream);
+
 /* Replaces src/infiniop/ops/paged_attention/operator.cc:154-190. */
 __INFINI_C __export infiniStatus_t infiniopDestroyPagedAttentionDescriptor(
     infiniopPagedAttentionDescriptor_t desc);

@@ -13,8 +13,10 @@
 #include "decode_tiled.h"
 #include "decode_mla.h"
 #include "decode_plan.h"
+#include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 
 namespace op::paged_attention::amd {
 
@@ -136,6 +138,45 @@ bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
 
 } // namespace
 
+// ---- scratch of the entry point that takes no workspace (infiniopPagedAttentionNoAlloc) ----
+// One array per GPU, held from the moment the library's code is loaded on that GPU until the process
+// ends. In host code the array's name is only a handle for the runtime: the address a kernel can use is
+// looked up once per device (with that device current) and kept; every use below goes through that address.
+constexpr size_t kScratchBytes = size_t{32} << 20;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
+namespace {
+
+constexpr int kMaxScratchDevices = 64;
+std::mutex g_scratch_mutex;
+void *g_scratch_ptr[kMaxScratchDevices] = {};
+
+// Device address of this GPU's scratch array; nullptr (and a status) when it cannot be had. The caller's
+// current device must be `device_id`: the lookup answers for the current device.
+infiniStatus_t scratchAddress(int device_id, void **ptr) {
+    *ptr = nullptr;
+    if (device_id < 0 || device_id >= kMaxScratchDevices) {
+        return INFINI_STATUS_DEVICE_NOT_FOUND;
+    }
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[device_id] == nullptr) {
+        int current = -1;
+        if (hipGetDevice(&current) != hipSuccess || current != device_id) {
+            return INFINI_STATUS_BAD_PARAM;
+        }
+        void *address = nullptr;
+        if (hipGetSymbolAddress(&address, HIP_SYMBOL(scratch)) != hipSuccess || address == nullptr) {
+            (void)hipGetLastError();
+            return INFINI_STATUS_INTERNAL_ERROR;
+        }
+        g_scratch_ptr[device_id] = address;
+    }
+    *ptr = g_scratch_ptr[device_id];
+    return INFINI_STATUS_SUCCESS;
+}
+
+} // namespace
+
 struct Descriptor::Opaque {
     Plan plan;
 };
@@ -158,6 +199,13 @@ infiniStatus_t Descriptor::create(infiniopHandle_t handle, Descriptor **desc_ptr
     // includes 256 spare bytes that let calculate() align the carve-up itself, whatever pointer the caller passes
     const size_t workspace_bytes = plan.workspaceBytes();
     *desc_ptr = new Descriptor(new Opaque{plan}, in, workspace_bytes, handle->device, handle->device_id);
+    // Set-up for calculateNoAlloc(): look the scratch array up now if this thread is on the descriptor's
+    // GPU, so that the first call (which may sit inside a stream capture) finds the address ready. Not an
+    // error when it cannot be done here (no GPU visible, another device current): the call does it then.
+    if (device::amd::deviceInfo(handle->device_id).queried && workspace_bytes > 0 && workspace_bytes <= kScratchBytes) {
+        void *unused = nullptr;
+        (void)scratchAddress(handle->device_id, &unused);
+    }
     return INFINI_STATUS_SUCCESS;
 }
 
@@ -168,6 +216,30 @@ infiniStatus_t Descriptor::calculate(void *workspace, size_t workspace_size, voi
         return INFINI_STATUS_INSUFFICIENT_WORKSPACE;
     }
     return launch(workspace, out, q, k_cache, v_cache, block_tables, seq_lens, alibi_slopes, stream_);
+}
+
+// The call without a workspace argument: partial results go to this GPU's scratch array (32 MiB). Calls
+// whose descriptor needs more are refused. Nothing in the array has to start at zero (every row that is
+// read was written by the same call), so nothing is cleared; two calls that overlap on one GPU (different
+// streams, or threads) share the array and race.
+infiniStatus_t Descriptor::calculateNoAlloc(void *out, const void *q, const void *k_cache, const void *v_cache,
+                                            const void *block_tables, const void *seq_lens, const void *alibi_slopes,
+                                            void *stream_) const {
+    if (_workspace_size > kScratchBytes) {
+        std::fprintf(stderr,
+                     "infiniopPagedAttentionNoAlloc: this descriptor needs %zu bytes of scratch, the built-in array holds "
+                     "%zu; use infiniopPagedAttention with a caller-provided workspace\n",
+                     _workspace_size, kScratchBytes);
+        return INFINI_STATUS_INSUFFICIENT_WORKSPACE;
+    }
+    void *ptr = nullptr;
+    if (_workspace_size > 0) {
+        const infiniStatus_t status = scratchAddress(device_id, &ptr);
+        if (status != INFINI_STATUS_SUCCESS) {
+            return status;
+        }
+    }
+    return launch(ptr, out, q, k_cache, v_cache, block_tables, seq_lens, alibi_slopes, stream_);
 }
 
 infiniStatus_t Descriptor::launch(void *workspace, void *out, const void *q, const void *k_cache, const void *v_cache,

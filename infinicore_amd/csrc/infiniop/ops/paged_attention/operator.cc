@@ -60,6 +60,22 @@ __INFINI_C infiniStatus_t infiniopPagedAttention(infiniopPagedAttentionDescripto
     }
 }
 
+__INFINI_C infiniStatus_t infiniopPagedAttentionNoAlloc(infiniopPagedAttentionDescriptor_t desc, void *out, const void *q,
+                                                        const void *k_cache, const void *v_cache,
+                                                        const void *block_tables, const void *seq_lens,
+                                                        const void *alibi_slopes, void *stream) {
+    if (desc == nullptr) {
+        return INFINI_STATUS_NULL_POINTER;
+    }
+    switch (desc->device_type) {
+    case INFINI_DEVICE_AMD:
+        return reinterpret_cast<AmdDescriptor *>(desc)->calculateNoAlloc(out, q, k_cache, v_cache, block_tables,
+                                                                         seq_lens, alibi_slopes, stream);
+    default:
+        return INFINI_STATUS_DEVICE_TYPE_NOT_SUPPORTED;
+    }
+}
+
 __INFINI_C infiniStatus_t infiniopDestroyPagedAttentionDescriptor(infiniopPagedAttentionDescriptor_t desc) {
     if (desc == nullptr) {
         return INFINI_STATUS_NULL_POINTER;

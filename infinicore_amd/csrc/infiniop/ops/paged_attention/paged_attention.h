@@ -33,6 +33,10 @@
         infiniStatus_t calculate(void *workspace, size_t workspace_size, void *out, const void *q,           \
                                  const void *k_cache, const void *v_cache, const void *block_tables,         \
                                  const void *seq_lens, const void *alibi_slopes, void *stream) const;        \
+        /* same call with the partial results in the library's own per-device scratch array */               \
+        infiniStatus_t calculateNoAlloc(void *out, const void *q, const void *k_cache, const void *v_cache,  \
+                                        const void *block_tables, const void *seq_lens,                      \
+                                        const void *alibi_slopes, void *stream) const;                       \
                                                                                                              \
     private:                                                                                                 \
         infiniStatus_t launch(void *workspace, void *out, const void *q, const void *k_cache,                \

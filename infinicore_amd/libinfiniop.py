@@ -150,6 +150,7 @@ def _open():
     _declare(op, "infiniopCreatePagedAttentionDescriptor", [infiniopHandle_t, POINTER(D), T, T, T, T, T, T, T, c_float])
     _declare(op, "infiniopGetPagedAttentionWorkspaceSize", [D, POINTER(c_size_t)])
     _declare(op, "infiniopPagedAttention", [D, vp, c_size_t, vp, vp, vp, vp, vp, vp, vp, vp])
+    _declare(op, "infiniopPagedAttentionNoAlloc", [D, vp, vp, vp, vp, vp, vp, vp, vp])
     _declare(op, "infiniopDestroyPagedAttentionDescriptor", [D])
 
     # ---- paged_attention_prefill ----
