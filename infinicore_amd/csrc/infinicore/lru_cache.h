@@ -25,10 +25,12 @@ struct MetaKey {
     std::vector<int64_t> words;
 
     void add(int64_t w) { words.push_back(w); }
-    // dtype, then every extent, then every stride (hash.hpp:24-30); an absent optional tensor is a single 0
-    // after its presence flag (hash.hpp:35-40).
+    // dtype, rank, then every extent, then every stride (hash.hpp:24-30, with the rank added: the word runs
+    // of the tensors are concatenated, and without it two argument lists whose ranks differ could spell the
+    // same words); an absent optional tensor is a single 0 after its presence flag (hash.hpp:35-40).
     void addTensor(int dtype, size_t ndim, const size_t *shape, const ptrdiff_t *strides) {
         add(dtype);
+        add(static_cast<int64_t>(ndim));
         for (size_t i = 0; i < ndim; ++i) {
             add(static_cast<int64_t>(shape[i]));
         }

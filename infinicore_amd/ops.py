@@ -61,15 +61,23 @@ def _ptr(t: torch.Tensor | None):
 
 
 class _Plan:
-    """An operator descriptor plus its workspace; owns both until evicted from the cache."""
+    """An operator descriptor plus its workspace; owns both until evicted from the cache. A plan belongs to one
+    stream (the stream is part of the cache key): two calls with the same shapes on different streams would
+    otherwise write their partial results into the same workspace at the same time."""
 
     def __init__(self, descriptor, destroy, workspace_bytes: int, device: torch.device):
         self.descriptor = descriptor
         self._destroy = destroy
         self.workspace_bytes = workspace_bytes
         self.workspace = torch.empty(workspace_bytes, dtype=torch.uint8, device=device) if workspace_bytes else None
+        self.stream = torch.cuda.current_stream(device)  # the stream of the cache key this plan is stored under
 
     def close(self):
+        if self.workspace is not None:
+            # evicted while a kernel on the plan's stream may still be using the workspace: the caching
+            # allocator may hand the memory out again only after that stream has passed this point
+            self.workspace.record_stream(self.stream)
+            self.workspace = None
         if self.descriptor is not None:
             check_error(self._destroy(self.descriptor))
             self.descriptor = None
@@ -94,6 +102,10 @@ def clear_plan_cache() -> None:
         plan.close()
 
 
+def _stream_key(device_index: int) -> int:
+    return int(torch.cuda.current_stream(device_index).cuda_stream)
+
+
 def _stream_ptr(device_index: int):
     return c_void_p(torch.cuda.current_stream(device_index).cuda_stream)
 
@@ -108,7 +120,7 @@ def paged_attention(q, k_cache, v_cache, block_tables, cache_lens, alibi_slopes=
     if out is None:
         out = torch.empty((*q.shape[:-1], v_cache.shape[-1]), dtype=q.dtype, device=q.device)
     tensors = (out, q, k_cache, v_cache, block_tables, cache_lens)
-    key = ("paged_attention", index, float(scale), *(_meta(t) for t in tensors), _meta(alibi_slopes))
+    key = ("paged_attention", index, _stream_key(index), float(scale), *(_meta(t) for t in tensors), _meta(alibi_slopes))
 
     def make():
         handle = _handle_for(index)
@@ -153,7 +165,7 @@ def paged_attention_prefill(q, k_cache, v_cache, block_tables, seq_lens, cum_seq
     if out is None:
         out = torch.empty((*q.shape[:-1], v_cache.shape[-1]), dtype=q.dtype, device=q.device)
     tensors = (out, q, k_cache, v_cache, block_tables, seq_lens, cum_seq_lens_q)
-    key = ("paged_attention_prefill", index, float(scale), *(_meta(t) for t in tensors), _meta(alibi_slopes))
+    key = ("paged_attention_prefill", index, _stream_key(index), float(scale), *(_meta(t) for t in tensors), _meta(alibi_slopes))
 
     def make():
         handle = _handle_for(index)
@@ -192,7 +204,7 @@ def paged_caching(k_cache, v_cache, k, v, slot_mapping):
     """Scatter ``k`` / ``v`` [num_tokens, num_kv_heads, d] into the pools in place; returns the pools."""
     index = _device_index(k)
     tensors = (k_cache, v_cache, k, v, slot_mapping)
-    key = ("paged_caching", index, *(_meta(t) for t in tensors))
+    key = ("paged_caching", index, _stream_key(index), *(_meta(t) for t in tensors))
 
     def make():
         handle = _handle_for(index)
@@ -228,7 +240,7 @@ def kv_caching(k_cache, v_cache, k, v, past_kv_lengths):
     the caches (argument order of the reference's infiniopKVCaching, include/infiniop/ops/kv_caching.h:8-29)."""
     index = _device_index(k)
     tensors = (k_cache, v_cache, k, v, past_kv_lengths)
-    key = ("kv_caching", index, *(_meta(t) for t in tensors))
+    key = ("kv_caching", index, _stream_key(index), *(_meta(t) for t in tensors))
 
     def make():
         handle = _handle_for(index)

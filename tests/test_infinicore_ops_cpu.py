@@ -55,6 +55,18 @@ int main() {
     a.addTensor(19, 3, shape, nullptr); b.addTensor(19, 3, shape, contiguous); d.addTensor(19, 3, shape, padded);
     e.addTensor(12, 3, shape, nullptr);
     std::printf("same=%d padded_differs=%d dtype_differs=%d hash_same=%d\n", a == b, !(a == d), !(a == e), a.hash() == b.hash());
+    // two argument lists whose ranks differ must not spell the same words: (rank 3 [4, 32, 128]) + (rank 1 [7])
+    // against (rank 2 [4, 32]) + (rank 2 ...) built so that the concatenated extents and strides coincide
+    {
+        size_t s3[3] = {2, 3, 1}, s1[1] = {1};
+        size_t s2a[2] = {2, 3}, s2b[2] = {1, 1};
+        ptrdiff_t t3[3] = {3, 1, 1}, t1[1] = {1};
+        ptrdiff_t t2a[2] = {3, 1}, t2b[2] = {1, 1};
+        MetaKey x, y;
+        x.addTensor(19, 3, s3, t3); x.addTensor(19, 1, s1, t1);
+        y.addTensor(19, 2, s2a, t2a); y.addTensor(19, 2, s2b, t2b);
+        std::printf("ranks_differ=%d\n", !(x == y));
+    }
     // the reference's fold: seed ^= hash(v) + 0x9e3779b9 + (seed << 6) + (seed >> 2), starting from 0
     MetaKey k; k.add(7); k.add(9);
     size_t seed = 0;
@@ -83,6 +95,7 @@ def test_lru_cache_and_metadata_key(tmp_path):
         "alive_after_overwrite=2",
         "alive_after_clear=0",
         "same=1 padded_differs=1 dtype_differs=1 hash_same=1",
+        "ranks_differ=1",
         "fold=1",
     ]
 
