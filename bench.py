@@ -1,12 +1,13 @@
 #!/usr/bin/env python3
 """Paged-attention benchmark on one MI355X: decode (default, the headline) or prefill.
 
-A step is one ``infiniopPagedAttention`` call (decode kernel + partition merge) through the C ABI on
-the Llama-3-8B GQA batch-32 decode shape (bf16, 32 query / 8 KV heads, head 128, pages of 16
-tokens, ragged lengths 512..4096 through a shuffled block table). Inputs are resident in HBM before
-the timed region. Consecutive steps read different KV pools (same content, different addresses,
-together far larger than the 256 MiB last-level cache), so every step streams its K/V from HBM as a
-real model does when it moves from layer to layer.
+A step is one decode step's worth of attention for a 32-layer model: 32 ``infiniopPagedAttention`` calls
+(decode kernel + segment merge each) through the C ABI, one per layer, on the Llama-3-8B GQA batch-32
+decode shape (bf16, 32 query / 8 KV heads, head 128, pages of 16 tokens, ragged lengths 512..4096 through a
+shuffled block table). Every layer has a KV pool of its own (same content, different addresses, 11 GB
+together), so every call streams its K/V from HBM as a real model does when it moves from layer to layer.
+Inputs are resident in HBM before the timed region. ``us_per_call`` = step time / 32; ``value`` is the
+algorithmic bytes of the step over its time.
 
 With ``--workload p2_llama3_8b_prompt`` or ``p3_llama3_8b_chunked`` a step is one
 ``infiniopPagedAttentionPrefill`` call instead, bounded by the bf16 matrix-core peak; the line then
@@ -51,13 +52,14 @@ MEASURED_TRAFFIC_BYTES = {
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=None, help="default 400 (decode) / 50 (prefill)")
-    ap.add_argument("--warmup", type=int, default=None, help="default 40 (decode) / 5 (prefill)")
+    ap.add_argument("--steps", type=int, default=None, help="default 20 (decode: 32 calls each) / 50 (prefill) / 400 (scatter)")
+    ap.add_argument("--warmup", type=int, default=None, help="default 3 (decode) / 5 (prefill) / 40 (scatter)")
+    ap.add_argument("--layers", type=int, default=32, help="decode: calls per step, each on a KV pool of its own")
     ap.add_argument("--workload", default="c2_llama3_8b_b32")
     ap.add_argument("--head-size", type=int, default=0,
                     help="run the workload's shape with this head size (64 / 192 / 256) instead of its own; the "
                          "workload name in the output gets a _d<head> suffix")
-    ap.add_argument("--pools", type=int, default=4, help="distinct KV pools the steps rotate over")
+    ap.add_argument("--pools", type=int, default=4, help="scatter workloads: distinct cache sets the steps rotate over")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-check", action="store_true", help="skip the oracle check of the output")
     ap.add_argument("--pmc-calibration", action="store_true",
@@ -217,6 +219,7 @@ def run_prefill(args, torch, L, workloads, dev):
             "value": round(sample_flops / cpu_s / 1e12, 5),
             "unit": "TFLOP/s",
             "cores": threads,
+            "host_cores": os.cpu_count(),
             "kind": "port",
             "sample": f"{reps} passes of the C oracle over {len(rows)} of the {cum[-1]} query rows "
                       f"({sample_flops / flops * 100:.2f} % of the call's flops), {cpu_s * 1e3:.1f} ms per pass",
@@ -355,7 +358,7 @@ def run_caching(args, torch, L, workloads, dev):
             reps += 1
         cpu_s = (time.perf_counter() - t0) / reps
         result["cpu_baseline"] = {
-            "value": round(algo_bytes / cpu_s / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+            "value": round(algo_bytes / cpu_s / 1e9, 3), "unit": "GB/s", "cores": 1, "host_cores": os.cpu_count(), "kind": "port",
             "sample": f"{reps} full calls of the same workload through the C oracle (one thread), {cpu_s * 1e6:.0f} us per call",
         }
     print(json.dumps(result))
@@ -389,8 +392,9 @@ def main():
         args.steps = 50 if args.steps is None else args.steps
         args.warmup = 5 if args.warmup is None else args.warmup
         return run_prefill(args, torch, L, workloads, dev)
-    args.steps = 400 if args.steps is None else args.steps
-    args.warmup = 40 if args.warmup is None else args.warmup
+    args.steps = 20 if args.steps is None else args.steps
+    args.warmup = 3 if args.warmup is None else args.warmup
+    layers = max(1, args.layers)
     cfg = workloads.DECODE_CONFIGS[args.workload]
     if args.head_size:
         cfg = dataclasses.replace(cfg, head_size=args.head_size, name=f"{cfg.name}_d{args.head_size}")
@@ -405,7 +409,7 @@ def main():
     sl = inp.seq_lens.to(dev)
     k_pools = [inp.k_cache.to(dev)]
     v_pools = [inp.v_cache.to(dev)]
-    for _ in range(1, max(1, args.pools)):
+    for _ in range(1, layers):
         k_pools.append(k_pools[0].clone())
         v_pools.append(v_pools[0].clone())
     out = torch.zeros((*q.shape[:-1], v_pools[0].shape[-1]), dtype=q.dtype, device=dev)
@@ -431,12 +435,15 @@ def main():
     L.check_error(L.LIBINFINIRT.infinirtEventCreate(ctypes.byref(ev0)))
     L.check_error(L.LIBINFINIRT.infinirtEventCreate(ctypes.byref(ev1)))
 
-    def step(i):
-        p = i % len(k_pools)
+    def call(p):
         L.check_error(L.LIBINFINIOP.infiniopPagedAttention(
             op, c_void_p(workspace.data_ptr()), ws_size.value, c_void_p(out.data_ptr()), c_void_p(q.data_ptr()),
             c_void_p(k_pools[p].data_ptr()), c_void_p(v_pools[p].data_ptr()), c_void_p(bt.data_ptr()),
             c_void_p(sl.data_ptr()), c_void_p(0), stream))
+
+    def step(i):
+        for p in range(layers):
+            call(p)
 
     if args.pmc_calibration:
         pmc_calibration_copies(torch, dev)
@@ -458,8 +465,9 @@ def main():
     ms = c_float(0)
     L.check_error(L.LIBINFINIRT.infinirtEventElapsedTime(ctypes.byref(ms), ev0, ev1))
 
-    us_wall = wall_s / args.steps * 1e6
-    us_dev = ms.value / args.steps * 1e3           # device time per call on the kernels' stream
+    calls = args.steps * layers
+    us_wall = wall_s / calls * 1e6
+    us_dev = ms.value / calls * 1e3                # device time per call on the kernels' stream
     gbps_wall = algo_bytes / (us_wall * 1e-6) / 1e9
     gbps_dev = algo_bytes / (us_dev * 1e-6) / 1e9
 
@@ -471,7 +479,7 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": round(us_wall / 1e3, 6),
+        "ms_per_step": round(us_wall * layers / 1e3, 6),
         "us_per_call": round(us_wall, 2),
         "higher_is_better": True,
         "scaling": "weak",
@@ -483,7 +491,8 @@ def main():
             "num_seqs": cfg.num_seqs, "num_heads": cfg.num_heads, "num_kv_heads": cfg.num_kv_heads,
             "head_size": cfg.head_size, "value_size": cfg.v_size, "block_size": cfg.block_size,
             "seq_lens": f"uniform[{cfg.min_len},{cfg.max_len}] sum={int(inp.seq_lens.sum())}",
-            "kv_pools_rotated": len(k_pools),
+            "calls_per_step": layers,
+            "kv_pools": len(k_pools),
             "algorithmic_bytes_per_call": algo_bytes,
         },
         "roofline": {
@@ -504,7 +513,7 @@ def main():
         # not timed: one more call on pool 0, compared with the CPU oracle
         from oracle import paged_oracle
 
-        step(0)
+        call(0)
         L.check_error(L.LIBINFINIRT.infinirtStreamSynchronize(stream))
         # against the oracle's value before its final rounding to the storage dtype: two correctly rounded
         # results can sit one bf16 step apart, which above |x| = 2.44 is already more than the tolerance
@@ -534,9 +543,10 @@ def main():
             "value": round(algo_bytes / cpu_s / 1e9, 3),
             "unit": "GB/s",
             "cores": threads,
+            "host_cores": os.cpu_count(),
             "kind": "port",
-            "sample": f"{reps} full calls of the same workload through the C oracle (OpenMP over sequence x head), "
-                      f"{cpu_s * 1e3:.1f} ms per call",
+            "sample": f"{reps} full calls of the same workload through the C oracle (OpenMP over sequence x head, "
+                      f"{threads} threads of the host's {os.cpu_count()} cores), {cpu_s * 1e3:.1f} ms per call",
             "us_per_call": round(cpu_s * 1e6, 1),
         }
         # the torch statement the reference's own test uses as expected value (vectorised gather), one call
@@ -545,10 +555,25 @@ def main():
         paged_oracle.torch_reference_attention(inp.q, inp.k_cache, inp.v_cache, inp.block_tables, inp.seq_lens, inp.scale)
         torch_s = time.perf_counter() - t0
         result["cpu_baseline_torch"] = {
-            "value": round(algo_bytes / torch_s / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
-            "sample": "1 full call of the reference test's torch formulation (vectorised gather) on CPU",
+            "value": round(algo_bytes / torch_s / 1e9, 3), "unit": "GB/s", "cores": threads, "host_cores": os.cpu_count(),
+            "kind": "port",
+            "sample": f"1 full call of the reference test's torch formulation (vectorised gather) on CPU, "
+                      f"torch.get_num_threads() = {torch.get_num_threads()}",
             "us_per_call": round(torch_s * 1e6, 1),
         }
+        if cfg.name == "c1_plumbing_mha":
+            # the literal form of the reference's test: a Python loop over every token of every sequence
+            # (test/infiniop/paged_attention.py:60-73); only on the smallest workload, where it ends in seconds
+            t0 = time.perf_counter()
+            paged_oracle.torch_reference_attention(inp.q, inp.k_cache, inp.v_cache, inp.block_tables, inp.seq_lens,
+                                                   inp.scale, vectorised=False)
+            loop_s = time.perf_counter() - t0
+            result["cpu_baseline_torch_token_loop"] = {
+                "value": round(algo_bytes / loop_s / 1e9, 4), "unit": "GB/s", "cores": threads,
+                "host_cores": os.cpu_count(), "kind": "port",
+                "sample": "1 full call of the reference test's torch formulation with its per-token Python loop",
+                "us_per_call": round(loop_s * 1e6, 1),
+            }
 
     print(json.dumps(result))
     L.check_error(L.LIBINFINIOP.infiniopDestroyPagedAttentionDescriptor(op))

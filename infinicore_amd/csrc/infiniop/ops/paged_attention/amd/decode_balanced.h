@@ -26,6 +26,7 @@
 namespace op::paged_attention::amd {
 
 constexpr int kBalancedMinTiles = 4;   // never cut pieces finer than 64 tokens
+constexpr int kReaderSpinLimit = 1 << 22; // polls (~0.5 us each) before a reader gives up on a flag
 
 // Inclusive prefix sum over the 64 lanes with data-parallel-primitive moves (no LDS-unit permutes: this
 // runs at the head of every wavefront, before its first memory request can go out). Rows of 16 lanes are
@@ -113,7 +114,16 @@ struct TileRun {
 // and moves values between the two files in the tile loop, with the budget it fits 230 vector registers
 // without spilling (c2 57.7 -> 56.6 us, three runs each on one box). Heads 192 and 256 spill under that
 // budget, head 64 fits it anyway: they are left to the compiler.
-template <typename T, typename Tindex, int HEAD>
+//
+// FUSED: the segments of a sequence are merged by the decode kernel itself instead of by a second kernel. The
+// wavefront whose piece holds a sequence's LAST segment is that sequence's reader: it keeps its own segment's
+// state, and when its piece is done it waits for the rows of the sequence's earlier segments, merges them and
+// writes the output. The earlier segments belong to earlier pieces of the same stream, i.e. to workgroups with
+// lower linear ids, and a wavefront publishes its rows before it starts to wait for anybody else's: a reader
+// only ever waits for wavefronts that were dispatched before it and that never wait before they publish, so
+// the scheme cannot deadlock however few of the workgroups are resident at a time (the wait is bounded all
+// the same). Rows and flags cross between accelerator dies with agent-scope accesses (decode_common.h).
+template <typename T, typename Tindex, int HEAD, bool FUSED>
 __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(HEAD == 128 ? 2 : 1, HEAD == 128 ? 2 : 8)))
 decodeBalancedKernel(const void *early_seq_lens, int early_num_seqs, int early_max_blocks_per_seq, int early_block_shift,
                      DecodeArgs a, int waves_per_stream) {
@@ -125,6 +135,8 @@ decodeBalancedKernel(const void *early_seq_lens, int early_num_seqs, int early_m
     // one finished segment's state (accumulators, denominator, maximum), word-major so that lane i
     // always touches bank i: written and read back by the same lane
     __shared__ float stash[(4 * G::kCols + 2) * 64];
+    // FUSED: the state of the segment this wavefront is the reader of, until the end of the piece
+    __shared__ float reader_stash[FUSED ? (4 * G::kCols + 2) * 64 : 1];
 
     const int piece = blockIdx.x;
     const int head_chunks = (a.group + kHeadsPerWave - 1) / kHeadsPerWave;
@@ -145,6 +157,7 @@ decodeBalancedKernel(const void *early_seq_lens, int early_num_seqs, int early_m
     constexpr int kStartCost = HEAD <= 128 ? 384 / HEAD : 2;
     static_assert(kStartCost <= kBalancedMaxStartCost, "the launch plan bounds the flat axis with this");
     const int q = tilesPerPiece(total_tiles + kStartCost * a.num_seqs, waves_per_stream);
+    auto pieceOf = [&](int x) { return x / q; }; // the piece that holds virtual slot x
     // Real tiles below virtual positions x0 = piece * q and x1 = x0 + q: count the sequences that lie
     // entirely below each (one pass over the prefix sums for both), then add the part of the next one.
     const int x0 = piece * q, x1 = x0 + q;
@@ -362,6 +375,38 @@ decodeBalancedKernel(const void *early_seq_lens, int early_num_seqs, int early_m
             }
         }
     };
+    // FUSED: partial rows of a segment for the reader of its sequence, and the flag that says they are there.
+    // A row of head h is HEAD floats, stored as 16-byte chunks in the order (chunk of the lane, strip c): each
+    // store instruction then writes 256 contiguous bytes per head. (m, l) of the 16 heads follow as pairs in the
+    // place of the m and l arrays. Heads beyond the group lie beyond the buffers' sizes: nothing is stored.
+    const int heads_here = min(kHeadsPerWave, a.group - chunk * kHeadsPerWave);
+    const int first_head = kv_head * a.group + chunk * kHeadsPerWave;
+    auto rowsOf = [&](int row_group) { // row_group = piece + sequence
+        return agentBuffer(a.part_acc + (static_cast<int64_t>(row_group) * a.num_heads + first_head) * HEAD,
+                           heads_here * HEAD * static_cast<int>(sizeof(float)));
+    };
+    auto pairsOf = [&](int row_group) {
+        return agentBuffer(reinterpret_cast<float2 *>(a.part_m) + static_cast<int64_t>(row_group) * a.num_heads + first_head,
+                           heads_here * static_cast<int>(sizeof(float2)));
+    };
+    auto publishSegment = [&](const TileState<HEAD> &state, float l_tot, int seq) {
+        const auto rows = rowsOf(piece + seq);
+#pragma unroll
+        for (int rr = 0; rr < 4; ++rr) {
+#pragma unroll
+            for (int h = 0; h < G::kCols / 4; ++h) {
+                storeAgent16(rows, (4 * g + rr) * HEAD * 4 + 256 * h + 16 * c, state.o[4 * h][rr], state.o[4 * h + 1][rr],
+                             state.o[4 * h + 2][rr], state.o[4 * h + 3][rr]);
+            }
+        }
+        if (g == 0) {
+            storeAgent8(pairsOf(piece + seq), 8 * c, state.m, l_tot); // lane c holds head c's maximum and sum
+        }
+        waitVectorMemory(); // the rows are in memory before the flag says so
+        if (lane == 0) {
+            storeAgent(a.seg_flags + static_cast<int64_t>(piece + seq) * gridDim.y + blockIdx.y, a.token);
+        }
+    };
 
     // A segment that ends in the middle of the piece is not stored at once: stores count as outstanding
     // memory operations like the tile loads, the waits of the tile loop are fixed counts, and with a
@@ -385,7 +430,27 @@ decodeBalancedKernel(const void *early_seq_lens, int early_num_seqs, int early_m
         writeResult(parked, l_tot, stash_seq, stash_whole);
         stash_seq = -1;
     };
+    int reader_seq = -1; // FUSED: the sequence whose last segment this piece holds next to earlier ones elsewhere
+    auto parkReaderSegment = [&]() {
+        const float l_tot = sumAcrossTokenGroups(st.l);
+#pragma unroll
+        for (int e = 0; e < G::kCols; ++e) {
+#pragma unroll
+            for (int rr = 0; rr < 4; ++rr) {
+                reader_stash[(4 * e + rr) * 64 + lane] = st.o[e][rr];
+            }
+        }
+        reader_stash[(4 * G::kCols) * 64 + lane] = l_tot;
+        reader_stash[(4 * G::kCols + 1) * 64 + lane] = st.m;
+        reader_seq = c_seq;
+    };
     auto parkSegment = [&]() {
+        if constexpr (FUSED) {
+            if (c_t_begin > 0 && c_seg_end == c_seq_tiles) {
+                parkReaderSegment(); // ends a sequence that began in an earlier piece
+                return;
+            }
+        }
         if (stash_seq >= 0) {
             flushStash();
         }
@@ -429,7 +494,7 @@ decodeBalancedKernel(const void *early_seq_lens, int early_num_seqs, int early_m
     // Tell the merge kernel which pieces hold each sequence that starts in this piece (one writer per
     // sequence: the wavefront of the first stream whose piece contains the sequence's first tile).
     // Done before the first tile is requested, for the reason given at parkSegment.
-    if (blockIdx.y == 0) {
+    if (!FUSED && blockIdx.y == 0) {
         for (int base = seq0; base < a.num_seqs; base += 64) {
             const int s = base + lane;
             bool more = false;
@@ -438,7 +503,7 @@ decodeBalancedKernel(const void *early_seq_lens, int early_num_seqs, int early_m
                 const int last = pre_incl[s];
                 more = first < f1;
                 if (last > first && first >= f0 && first < f1) {
-                    a.seq_pieces[s] = make_int2(piece, (last - 1 + kStartCost * (s + 1)) / q - piece + 1);
+                    a.seq_pieces[s] = make_int2(piece, pieceOf(last - 1 + kStartCost * (s + 1)) - piece + 1);
                 }
             }
             if (__builtin_amdgcn_ballot_w64(more) == 0) {
@@ -470,9 +535,119 @@ decodeBalancedKernel(const void *early_seq_lens, int early_num_seqs, int early_m
         }
     }
     // the piece's last segment, then the parked one
-    writeResult(st, sumAcrossTokenGroups(st.l), c_seq, c_t_begin == 0 && c_seg_end == c_seq_tiles);
+    {
+        const bool begins = c_t_begin == 0, ends = c_seg_end == c_seq_tiles;
+        if (FUSED && !begins && ends) {
+            parkReaderSegment();
+        } else if (FUSED && !ends) {
+            publishSegment(st, sumAcrossTokenGroups(st.l), c_seq);
+        } else {
+            writeResult(st, sumAcrossTokenGroups(st.l), c_seq, begins && ends);
+        }
+    }
     if (stash_seq >= 0) {
         flushStash();
+    }
+    if constexpr (FUSED) {
+        if (reader_seq < 0) {
+            return;
+        }
+        // ---- reader: merge the earlier segments of sequence reader_seq into the parked state ----
+        const int s = reader_seq;
+        const int first_piece = pieceOf(seqFirstTile(s) + kStartCost * (s + 1)); // piece of the sequence's first tile
+        const int count = piece - first_piece;                                // earlier segments, >= 1
+        const int64_t flag_stride = gridDim.y;
+        unsigned long long *flags = a.seg_flags + static_cast<int64_t>(first_piece + s) * flag_stride + blockIdx.y;
+        bool arrived = true;
+        for (int base = 0; base < count && arrived; base += 64) {
+            const int idx = base + lane;
+            int spins = 0;
+            while (true) {
+                const unsigned long long v = idx < count ? loadAgent(flags + idx * flag_stride) : a.token;
+                if (__builtin_amdgcn_ballot_w64(v != a.token) == 0) {
+                    break;
+                }
+                __builtin_amdgcn_s_sleep(1);
+                if (++spins > kReaderSpinLimit) {
+                    arrived = false; // cannot happen with in-order dispatch; never spin for ever
+                    break;
+                }
+            }
+        }
+        compilerMemoryBarrier(); // the row loads below stay below the flag loads above
+        if (!arrived) {
+            return;
+        }
+        TileState<HEAD> own;
+#pragma unroll
+        for (int e = 0; e < G::kCols; ++e) {
+#pragma unroll
+            for (int rr = 0; rr < 4; ++rr) {
+                own.o[e][rr] = reader_stash[(4 * e + rr) * 64 + lane];
+            }
+        }
+        const float own_l = reader_stash[(4 * G::kCols) * 64 + lane];
+        const float own_m = reader_stash[(4 * G::kCols + 1) * 64 + lane];
+        float m_run[4], l_run[4];
+#pragma unroll
+        for (int rr = 0; rr < 4; ++rr) {
+            l_run[rr] = __shfl(own_l, 4 * g + rr, 64);
+            m_run[rr] = __shfl(own_m, 4 * g + rr, 64);
+        }
+        if (4 * g < heads_here) { // lanes that hold at least one real head
+            constexpr int kBatch = 4; // segments per round trip
+            for (int i0 = 0; i0 < count; i0 += kBatch) {
+                float2 ml[kBatch][4];
+                float4 v[kBatch][4][G::kCols / 4];
+#pragma unroll
+                for (int j = 0; j < kBatch; ++j) {
+                    const int i = min(i0 + j, count - 1); // past the end: the last one again, merged with weight 0
+                    const auto rows = rowsOf(first_piece + i + s);
+                    const auto pairs = pairsOf(first_piece + i + s);
+#pragma unroll
+                    for (int rr = 0; rr < 4; ++rr) {
+                        ml[j][rr] = loadAgent8(pairs, 8 * (4 * g + rr));
+#pragma unroll
+                        for (int h = 0; h < G::kCols / 4; ++h) {
+                            v[j][rr][h] = loadAgent16(rows, (4 * g + rr) * HEAD * 4 + 256 * h + 16 * c);
+                        }
+                    }
+                }
+#pragma unroll
+                for (int j = 0; j < kBatch; ++j) {
+                    const bool real = i0 + j < count;
+#pragma unroll
+                    for (int rr = 0; rr < 4; ++rr) {
+                        const float m_i = real ? ml[j][rr].x : -INFINITY;
+                        const float m_new = fmaxf(m_run[rr], m_i);
+                        const float w_old = mergeWeight(m_run[rr], m_new), w_i = mergeWeight(m_i, m_new);
+                        l_run[rr] = l_run[rr] * w_old + (real ? ml[j][rr].y : 0.0f) * w_i;
+#pragma unroll
+                        for (int h = 0; h < G::kCols / 4; ++h) {
+                            own.o[4 * h][rr] = own.o[4 * h][rr] * w_old + v[j][rr][h].x * w_i;
+                            own.o[4 * h + 1][rr] = own.o[4 * h + 1][rr] * w_old + v[j][rr][h].y * w_i;
+                            own.o[4 * h + 2][rr] = own.o[4 * h + 2][rr] * w_old + v[j][rr][h].z * w_i;
+                            own.o[4 * h + 3][rr] = own.o[4 * h + 3][rr] * w_old + v[j][rr][h].w * w_i;
+                        }
+                        m_run[rr] = m_new;
+                    }
+                }
+            }
+#pragma unroll
+            for (int rr = 0; rr < 4; ++rr) {
+                if (4 * g + rr < heads_here) {
+                    S *o_ptr = static_cast<S *>(a.out) + s * a.o_stride + (first_head + 4 * g + rr) * a.o_head_stride;
+                    storeOutputRow<T, HEAD>(o_ptr + G::kCols * c, own, rr, 1.0f / (l_run[rr] + 1e-6f));
+                }
+            }
+        }
+        // the flags are consumed: clear them, so that a replay of this call (same token) starts clean
+        for (int base = 0; base < count; base += 64) {
+            const int idx = base + lane;
+            if (idx < count) {
+                flags[idx * flag_stride] = 0;
+            }
+        }
     }
 }
 

@@ -32,7 +32,11 @@ struct DecodeArgs {
     float *part_acc; // [.., value_size]
     float *part_m;
     float *part_l;
-    int2 *seq_pieces; // work-equalising schedule only: per sequence {first piece, number of pieces}
+    int2 *seq_pieces; // work-equalising schedule, merge by a second kernel: per sequence {first piece, number of pieces}
+    // work-equalising schedule, merge inside the decode kernel: one word per partial row group
+    // [(piece + sequence) x streams]; it holds `token` once the rows of that segment are complete in memory
+    unsigned long long *seg_flags;
+    unsigned long long token; // differs from call to call (a replayed graph repeats it: flags are cleared by their reader)
     // 64-head latent-attention kernel only: the partition size the decode kernel settled on for this
     // call (>= partition_tokens), written by its first workgroup for the merge kernel; else nullptr
     int32_t *chosen_partition;
@@ -90,6 +94,59 @@ struct BFloat16 {
 };
 
 __device__ __forceinline__ float fastExp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// ---- hand-over of data between wavefronts of one kernel ----
+// Each of the eight accelerator dies (XCDs) has its own L2, and the L2s are not kept coherent with one another
+// for ordinary accesses inside a kernel: an ordinary store stays in the writer's L2 until the kernel ends, and an
+// ordinary load may be served from the reader's own L1 / L2 copy of the line. Accesses with the sc1 bit
+// ("agent scope") are the ones that work across dies: such a store is written through to memory and such a
+// load is served from memory, past both caches. Measured with a ping-pong of 1 KiB rows between wavefronts
+// on different dies (and on the same die), the reader's caches holding the previous round's lines: sc1 stores +
+// `s_waitcnt vmcnt(0)` + an sc1 flag store, against an sc1 poll of the flag followed by sc1 loads of the rows:
+// 0 wrong words in 3.4e7 hand-overs, ~1 us per hand-over on an idle device; with ordinary stores or ordinary
+// loads on either side every hand-over between dies reads stale data.
+// Rows travel 16 bytes per lane through raw buffer accesses that carry the sc1 bit (the compiler knows these
+// instructions, so its wait-count bookkeeping covers them); the buffer descriptor holds a wave-uniform base
+// and a size, lanes whose offset lies beyond the size store nothing and load zeros. Flags are relaxed atomics
+// of agent scope, which compile to global_load / global_store ... sc1.
+constexpr int kAgentScope = 16; // cache-policy operand of the raw buffer builtins: sc1
+typedef unsigned agent_u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned agent_u32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t agentBuffer(const void *uniform_base, int bytes) {
+    const uint64_t b = reinterpret_cast<uint64_t>(uniform_base);
+    // (the lane read returns a signed int: widen both halves as unsigned, or a low half with its top bit set
+    // would smear ones over the high half)
+    const uint32_t hi = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<uint32_t>(b >> 32)));
+    const uint32_t lo = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<uint32_t>(b)));
+    const uint64_t u = (static_cast<uint64_t>(hi) << 32) | lo;
+    return __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void *>(u), 0, bytes, 0x00020000);
+}
+__device__ __forceinline__ void storeAgent16(__amdgpu_buffer_rsrc_t buffer, int byte_offset, float a, float b, float c, float d) {
+    const agent_u32x4 w = {__float_as_uint(a), __float_as_uint(b), __float_as_uint(c), __float_as_uint(d)};
+    __builtin_amdgcn_raw_buffer_store_b128(w, buffer, byte_offset, 0, kAgentScope);
+}
+__device__ __forceinline__ void storeAgent8(__amdgpu_buffer_rsrc_t buffer, int byte_offset, float a, float b) {
+    const agent_u32x2 w = {__float_as_uint(a), __float_as_uint(b)};
+    __builtin_amdgcn_raw_buffer_store_b64(w, buffer, byte_offset, 0, kAgentScope);
+}
+__device__ __forceinline__ float4 loadAgent16(__amdgpu_buffer_rsrc_t buffer, int byte_offset) {
+    const agent_u32x4 w = __builtin_amdgcn_raw_buffer_load_b128(buffer, byte_offset, 0, kAgentScope);
+    return make_float4(__uint_as_float(w[0]), __uint_as_float(w[1]), __uint_as_float(w[2]), __uint_as_float(w[3]));
+}
+__device__ __forceinline__ float2 loadAgent8(__amdgpu_buffer_rsrc_t buffer, int byte_offset) {
+    const agent_u32x2 w = __builtin_amdgcn_raw_buffer_load_b64(buffer, byte_offset, 0, kAgentScope);
+    return make_float2(__uint_as_float(w[0]), __uint_as_float(w[1]));
+}
+__device__ __forceinline__ void storeAgent(unsigned long long *p, unsigned long long v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ unsigned long long loadAgent(const unsigned long long *p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// Every vector memory operation this wavefront has issued is complete: loads have delivered, stores have been
+// written (agent-scope stores: to memory). Also a barrier for the compiler's own reordering of memory accesses.
+__device__ __forceinline__ void waitVectorMemory() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+__device__ __forceinline__ void compilerMemoryBarrier() { asm volatile("" ::: "memory"); }
 
 // Sum / max over the 64 lanes of a wavefront; every lane receives the result.
 __device__ __forceinline__ float waveSum(float x) {

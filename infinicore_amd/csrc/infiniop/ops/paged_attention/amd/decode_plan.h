@@ -10,6 +10,7 @@
 #include "../../../devices/amd/amd_device.h"
 #include "../info.h"
 #include <cstddef>
+#include <cstdio>
 #include <cstdlib>
 #include <cstring>
 
@@ -28,6 +29,7 @@ constexpr size_t kGridLimitYZ = 65535; // largest y / z extent of a launch
 struct Plan {
     bool tiled;            // tiled matrix-core kernel (head 64 / 128 / 192 / 256 or 576 with values of 512, power-of-two pages >= 16, 16-byte aligned strides)
     bool balanced;         // tiled kernel under the work-equalising schedule (decode_balanced.h)
+    bool fused_merge;      // balanced: segments merged inside the decode kernel (no second launch)
     bool latent_wide;      // latent attention with more than 16 query heads per KV head: up to 64 heads per workgroup
     bool partition_forced; // INFINIOP_AMD_PA_PARTITION set: the 64-head kernel keeps exactly that size
     int partition_tokens;  // grid schedule: tokens per unit of work
@@ -39,9 +41,11 @@ struct Plan {
     int fallback_max_partitions;
     int dims_per_lane;     // element-wise kernel: ceil(max(head_size, value_size) / 64)
     int waves_per_stream;  // balanced: wavefronts that share the tiles of one (KV head, 16-head chunk)
-    // Workspace regions, each 256-byte aligned: [acc][m][l][pieces].
-    size_t acc_bytes, ml_bytes, pieces_bytes;
-    size_t workspaceBytes() const { return acc_bytes > 0 ? acc_bytes + 2 * ml_bytes + pieces_bytes + 256 : 0; }
+    // Workspace regions, each 256-byte aligned: [acc][m][l][pieces][flags].
+    size_t acc_bytes, ml_bytes, pieces_bytes, flags_bytes;
+    size_t workspaceBytes() const {
+        return acc_bytes > 0 ? acc_bytes + 2 * ml_bytes + pieces_bytes + flags_bytes + 256 : 0;
+    }
 };
 
 inline size_t alignUp(size_t x, size_t a) { return (x + a - 1) / a * a; }
@@ -64,7 +68,7 @@ inline bool launchable(const PagedAttentionInfo &in) {
 
 // Environment knobs (all optional, read at descriptor creation only): INFINIOP_AMD_PA_KERNEL=generic,
 // INFINIOP_AMD_PA_SCHEDULE=grid|balanced, INFINIOP_AMD_PA_LATENT_KERNEL=wide|narrow,
-// INFINIOP_AMD_PA_PARTITION=<tokens>, INFINIOP_AMD_PA_WAVES_PER_CU=<n>.
+// INFINIOP_AMD_PA_PARTITION=<tokens>, INFINIOP_AMD_PA_WAVES_PER_CU=<n>, INFINIOP_AMD_PA_MERGE=kernel|fused.
 inline Plan makePlan(const PagedAttentionInfo &in, const device::amd::DeviceInfo &dev) {
     Plan plan{};
     const long long bs = static_cast<long long>(in.page_block_size);
@@ -189,6 +193,12 @@ inline Plan makePlan(const PagedAttentionInfo &in, const device::amd::DeviceInfo
         plan.waves_per_stream = static_cast<int>(wps < 1 ? 1 : wps);
         rows = static_cast<size_t>(plan.waves_per_stream) + in.num_seqs;
         plan.pieces_bytes = alignUp(in.num_seqs * 2 * sizeof(int), 256);
+        plan.fused_merge = false;
+        if (const char *env = std::getenv("INFINIOP_AMD_PA_MERGE")) {
+            plan.fused_merge = std::strcmp(env, "fused") == 0;
+        }
+        // one flag per (row, stream), whichever way the merge runs (the knob must not change the size)
+        plan.flags_bytes = alignUp(rows * static_cast<size_t>(stream_count) * sizeof(unsigned long long), 256);
         // the element-wise kernel's rows are (sequence, partition): as many partitions as those rows hold
         long long fallback = static_cast<long long>(rows / in.num_seqs);
         fallback = fallback > plan.max_partitions ? plan.max_partitions : fallback;

@@ -13,6 +13,8 @@
 #include "decode_tiled.h"
 #include "decode_mla.h"
 #include "decode_plan.h"
+#include <atomic>
+#include <chrono>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -68,8 +70,13 @@ void launchTiled(const DecodeArgs &a, const Plan &plan, hipStream_t stream) {
     const int head_chunks = (a.group + kHeadsPerWave - 1) / kHeadsPerWave;
     if (plan.balanced) {
         const dim3 grid(plan.waves_per_stream, a.num_kv_heads * head_chunks);
-        decodeBalancedKernel<T, Tindex, HEAD><<<grid, 64, 0, stream>>>(a.seq_lens, a.num_seqs, a.max_blocks_per_seq,
-                                                                       a.block_shift, a, plan.waves_per_stream);
+        if (plan.fused_merge) {
+            decodeBalancedKernel<T, Tindex, HEAD, true><<<grid, 64, 0, stream>>>(
+                a.seq_lens, a.num_seqs, a.max_blocks_per_seq, a.block_shift, a, plan.waves_per_stream);
+            return;
+        }
+        decodeBalancedKernel<T, Tindex, HEAD, false><<<grid, 64, 0, stream>>>(
+            a.seq_lens, a.num_seqs, a.max_blocks_per_seq, a.block_shift, a, plan.waves_per_stream);
         decodeBalancedMergeKernel<T, Tindex, HEAD><<<dim3((a.num_heads + 3) / 4, a.num_seqs), 256, 0, stream>>>(
             a.seq_lens, a.seq_pieces, a.num_heads, a);
     } else {
@@ -135,6 +142,16 @@ infiniStatus_t launchByIndex(infiniDtype_t index_dtype, const DecodeArgs &a, con
 }
 
 bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// A 64-bit value no earlier call of this process has used and that is never 0 (the value of a cleared flag):
+// a counter that starts at a point of the clock, spread over the word by an odd multiplier. What a workspace
+// holds before its first use can only be mistaken for it by a 2^-64 accident.
+unsigned long long nextToken() {
+    static std::atomic<unsigned long long> counter{
+        static_cast<unsigned long long>(std::chrono::steady_clock::now().time_since_epoch().count()) | 1ull};
+    unsigned long long t = counter.fetch_add(1, std::memory_order_relaxed) * 0x9e3779b97f4a7c15ull;
+    return t != 0 ? t : 0x9e3779b97f4a7c15ull;
+}
 
 } // namespace
 
@@ -281,9 +298,8 @@ infiniStatus_t Descriptor::launch(void *workspace, void *out, const void *q, con
         a.part_m = reinterpret_cast<float *>(ws + plan.acc_bytes);
         a.part_l = reinterpret_cast<float *>(ws + plan.acc_bytes + plan.ml_bytes);
         a.seq_pieces = reinterpret_cast<int2 *>(ws + plan.acc_bytes + 2 * plan.ml_bytes);
-        if (plan.latent_wide && !plan.partition_forced && in.num_seqs <= 256 && plan.tiled && aligned16(out) && aligned16(q) && aligned16(k_cache) && aligned16(v_cache)) {
-            a.chosen_partition = reinterpret_cast<int32_t *>(ws + plan.acc_bytes + 2 * plan.ml_bytes);
-        }
+        a.seg_flags = reinterpret_cast<unsigned long long *>(ws + plan.acc_bytes + 2 * plan.ml_bytes + plan.pieces_bytes);
+        a.token = nextToken();
     }
     a.scale_log2 = in.scale * kLog2e;
     a.num_seqs = static_cast<int32_t>(in.num_seqs);

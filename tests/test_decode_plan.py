@@ -87,7 +87,8 @@ def test_workspace_is_that_of_the_chosen_schedule(probe):
     slack - below the reference's 8 * B * H * (D + 2) * 4 = 4.26 MB."""
     c2 = probe(32, 32, 8, 128, 16, 256)
     rows = 128 + 32
-    assert c2["workspace_bytes"] == rows * 32 * 128 * 4 + 2 * rows * 32 * 4 + 256 + 256
+    flags = rows * 8 * 8  # one 8-byte flag per (row, KV-head stream)
+    assert c2["workspace_bytes"] == rows * 32 * 128 * 4 + 2 * rows * 32 * 4 + 256 + flags + 256
     assert c2["workspace_bytes"] < 8 * 32 * 32 * 130 * 4
     # the element-wise fallback (operands that are not 16-byte aligned at run time) fits the same rows
     assert c2["fallback_max_partitions"] * 32 <= rows

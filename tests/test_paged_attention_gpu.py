@@ -191,13 +191,16 @@ def test_mla_key_576_value_512(gpu_handle, oracle, dtype):
 
 # ---- head sizes of the tiled kernels -------------------------------------------------------------------
 
-@pytest.mark.parametrize("schedule", [None, "grid"])
+@pytest.mark.parametrize("schedule", [None, "grid", "fused"])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("D", [64, 192, 256])
 def test_tiled_kernels_other_head_sizes(gpu_handle, oracle, monkeypatch, D, dtype, schedule):
-    """Head sizes 64 / 192 / 256 on the matrix-core kernels, both schedules: ragged lengths incl. 1 token and
-    exactly one page, GQA 4, long enough that sequences are split and merged."""
-    if schedule:
+    """Head sizes 64 / 192 / 256 on the matrix-core kernels, both schedules (the work-equalising one also with
+    the segments merged inside the decode kernel): ragged lengths incl. 1 token and exactly one page, GQA 4,
+    long enough that sequences are split and merged."""
+    if schedule == "fused":
+        monkeypatch.setenv("INFINIOP_AMD_PA_MERGE", "fused")
+    elif schedule:
         monkeypatch.setenv("INFINIOP_AMD_PA_SCHEDULE", schedule)
     cfg = custom(f"head{D}_{schedule}", dtype, 6, 16, 4, D, 16, 1, 2500, seed=300 + D)
     inp = workloads.make_decode_inputs(cfg)
@@ -378,12 +381,14 @@ def test_default_schedule_choice(gpu_handle, oracle, monkeypatch, B, lo, hi):
 
 # ---- every kernel and schedule against the same oracle ---------------------------------------------
 
-@pytest.mark.parametrize("kernel,schedule", [("generic", None), (None, "grid"), (None, None)])
+@pytest.mark.parametrize("kernel,schedule", [("generic", None), (None, "grid"), (None, None), (None, "fused")])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_kernels_and_schedules_agree_with_oracle(gpu_handle, oracle, monkeypatch, kernel, schedule, dtype):
     if kernel:
         monkeypatch.setenv("INFINIOP_AMD_PA_KERNEL", kernel)
-    if schedule:
+    if schedule == "fused":  # the work-equalising schedule with the segments merged inside the decode kernel
+        monkeypatch.setenv("INFINIOP_AMD_PA_MERGE", "fused")
+    elif schedule:
         monkeypatch.setenv("INFINIOP_AMD_PA_SCHEDULE", schedule)
     cfg = custom(f"ragged_{kernel}_{schedule}", dtype, 6, 32, 8, 128, 16, 1, 3000, seed=5)
     inp = workloads.make_decode_inputs(cfg)
@@ -634,6 +639,31 @@ def test_one_descriptor_many_calls_with_changing_lengths(gpu_handle, oracle):
                                       num_threads=ORACLE_THREADS)
         assert_close(out, want, f"step {step}")
     L.check_error(L.LIBINFINIRT.infinirtStreamDestroy(stream))
+    L.check_error(L.LIBINFINIOP.infiniopDestroyPagedAttentionDescriptor(op))
+
+
+@pytest.mark.parametrize("merge", ["kernel", "fused"])
+@pytest.mark.parametrize("pools", [1, 3])
+def test_many_calls_on_one_workspace(gpu_handle, oracle, monkeypatch, pools, merge):
+    """One descriptor and workspace, many calls back to back on one or three KV pools, the workspace full of
+    random bytes before the first: every call must stay within the tolerance of the oracle. With the segments
+    merged by the second kernel and inside the decode kernel (whose flags each call must leave cleared)."""
+    monkeypatch.setenv("INFINIOP_AMD_PA_MERGE", merge)
+    inp = workloads.make_decode_inputs(custom("adaptive", torch.bfloat16, 16, 32, 8, 128, 16, 200, 2500, seed=91))
+    q, k, v, bt, sl = to_device(inp)
+    ks, vs = [k] + [k.clone() for _ in range(pools - 1)], [v] + [v.clone() for _ in range(pools - 1)]
+    out = torch.zeros_like(q)
+    status, op = create_paged_attention(gpu_handle, out, q, k, v, bt, sl, None, inp.scale)
+    assert status == 0
+    size = workspace_size_attention(op)
+    ws = torch.empty(size, dtype=torch.uint8, device=DEV).random_(0, 255)
+    want, want_f32 = oracle_of(oracle, inp, return_fp32=True)
+    for call in range(12):
+        out.zero_()
+        L.check_error(L.LIBINFINIOP.infiniopPagedAttention(op, ptr(ws), size, ptr(out), ptr(q), ptr(ks[call % pools]),
+                                                           ptr(vs[call % pools]), ptr(bt), ptr(sl), None, None))
+        torch.cuda.synchronize()
+        assert_close(out, want, f"call {call}", want_f32)
     L.check_error(L.LIBINFINIOP.infiniopDestroyPagedAttentionDescriptor(op))
 
 
