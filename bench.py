@@ -239,10 +239,26 @@ def run_caching(args, torch, L, workloads, dev):
     def oracle_fn(*operands):  # the checker and the CPU baseline; never on the timed path
         from oracle import paged_oracle
 
+        if rope:
+            return paged_oracle.rope_paged_caching(*operands, pos, sin, cos, True)
         return (paged_oracle.paged_caching if paged else paged_oracle.kv_caching)(*operands)
 
     paged = args.workload in workloads.CACHING_CONFIGS
-    if paged:
+    rope = args.workload in workloads.ROPE_CACHING_CONFIGS
+    if rope:
+        cfg = workloads.ROPE_CACHING_CONFIGS[args.workload]
+        inp, pos, sin, cos = workloads.make_rope_caching_inputs(cfg)
+        index = inp.slot_mapping
+        algo_bytes = workloads.rope_caching_algorithmic_bytes(cfg, index.numpy())
+        create = lambda handle, op, *descs: L.LIBINFINIOP.infiniopCreateRoPEPagedCachingDescriptor(handle, op, *descs, L.RoPEAlgo.GPT_NEOX)
+        size_of = L.LIBINFINIOP.infiniopGetRoPEPagedCachingWorkspaceSize
+        call, destroy = L.LIBINFINIOP.infiniopRoPEPagedCaching, L.LIBINFINIOP.infiniopDestroyRoPEPagedCachingDescriptor
+        metric = ("rotary embedding + paged_caching scatter achieved HBM GB/s (rows read + rows written + slot ids + "
+                  "positions + table rows / time per call), 1 GPU")
+        config = {"workload": cfg.name, "num_tokens": cfg.num_tokens, "valid_tokens": int((index >= 0).sum()),
+                  "num_kv_heads": cfg.num_kv_heads, "head_size": cfg.head_size, "block_size": cfg.block_size,
+                  "num_slots": cfg.num_slots, "table_len": workloads.ROPE_CACHING_TABLE_LEN, "algo": "gpt_neox"}
+    elif paged:
         cfg = workloads.CACHING_CONFIGS[args.workload]
         inp = workloads.make_caching_inputs(cfg)
         index = inp.slot_mapping
@@ -272,7 +288,8 @@ def run_caching(args, torch, L, workloads, dev):
     n_sets = max(1, min(args.pools, (8 << 30) // max(set_bytes, 1)))
     sets = [(inp.k_cache.to(dev), inp.v_cache.to(dev), inp.k.to(dev), inp.v.to(dev)) for _ in range(n_sets)]
     DTYPES = {torch.float16: L.InfiniDtype.F16, torch.bfloat16: L.InfiniDtype.BF16, torch.int64: L.InfiniDtype.I64}
-    descs = [L.create_tensor_descriptor(tuple(t.shape), tuple(t.stride()), DTYPES[t.dtype]) for t in (*sets[0], index_dev)]
+    extra = [t.to(dev) for t in (pos, sin, cos)] if rope else []
+    descs = [L.create_tensor_descriptor(tuple(t.shape), tuple(t.stride()), DTYPES[t.dtype]) for t in (*sets[0], index_dev, *extra)]
     op = L.infiniopOperatorDescriptor_t()
     L.check_error(create(handle, ctypes.byref(op), *descs))
     for d in descs:
@@ -289,7 +306,8 @@ def run_caching(args, torch, L, workloads, dev):
     def step(i):
         kc, vc, k, v = sets[i % len(sets)]
         L.check_error(call(op, c_void_p(0), 0, c_void_p(kc.data_ptr()), c_void_p(vc.data_ptr()), c_void_p(k.data_ptr()),
-                           c_void_p(v.data_ptr()), c_void_p(index_dev.data_ptr()), stream))
+                           c_void_p(v.data_ptr()), c_void_p(index_dev.data_ptr()), *[c_void_p(t.data_ptr()) for t in extra],
+                           stream))
 
     if args.pmc_calibration:
         pmc_calibration_copies(torch, dev)
@@ -384,7 +402,8 @@ def main():
         print("bench.py: no GPU visible; the HIP path has no CPU fallback", file=sys.stderr)
         sys.exit(3)
     dev = torch.device("cuda:0")
-    if args.workload in workloads.CACHING_CONFIGS or args.workload in workloads.KV_CACHING_CONFIGS:
+    if (args.workload in workloads.CACHING_CONFIGS or args.workload in workloads.KV_CACHING_CONFIGS
+            or args.workload in workloads.ROPE_CACHING_CONFIGS):
         args.steps = 400 if args.steps is None else args.steps
         args.warmup = 40 if args.warmup is None else args.warmup
         return run_caching(args, torch, L, workloads, dev)

@@ -8,6 +8,7 @@
 #include "infiniop/ops/paged_attention.h"
 #include "infiniop/ops/paged_attention_prefill.h"
 #include "infiniop/ops/paged_caching.h"
+#include "infiniop/ops/rope_paged_caching.h"
 #include "infiniop/tensor_descriptor.h"
 
 #endif

@@ -1,0 +1,300 @@
+// Rotary position embedding of the new K vectors fused with the scatter of K and V into the paged pool, on
+// AMD Instinct (gfx950): one launch for what the reference runs as two operators with a tensor in between
+// (rotation: src/infiniop/ops/rope/cuda/kernel.cuh:4-118, arithmetic as in src/infiniop/ops/rope/cpu/
+// rope_cpu.cc:56-98; scatter: src/infiniop/ops/paged_caching/cuda/kernel.cuh:22-89).
+//
+// Like the plain scatter the kernel is written for memory transactions: a workgroup is a (units of a row) x
+// (heads) x (tokens) box of 256 threads, a unit being 16 bytes. A thread that rotates takes the 16 bytes
+// that hold the first elements of 16 / sizeof(element) pairs and the 16 bytes that hold their partners
+// (neighbouring for GPT_J, half a vector away for GPT_NEOX), plus 16 bytes of each table, and writes two
+// 16-byte units of the K page row; V units are copied. Operands whose sizes, strides or addresses are not
+// multiples of 16 bytes take the same kernel with one pair / one element per step.
+// The decode step (one token per sequence, e.g. 32 x 8 x 128: 128 KiB in all) is a launch and three dependent
+// memory round trips long; fusing saves the second launch and the round trip of the rotated K through memory.
+#include "rope_paged_caching_amd.h"
+#include "../../../handle.h"
+#include "../../../../utils/check.h"
+#include <cstdint>
+#include <hip/hip_runtime.h>
+
+namespace op::rope_paged_caching::amd {
+
+namespace {
+
+struct Args {
+    void *k_cache;
+    void *v_cache;
+    const void *k;
+    const void *v;
+    const int64_t *slot_mapping;
+    const void *pos_ids;
+    const void *sin_table;
+    const void *cos_table;
+    int64_t num_tokens;
+    int64_t num_slots; // num_blocks * block_size; slots at or beyond it are ignored
+    int64_t table_len;
+    int32_t num_kv_heads;
+    int32_t block_size;
+    int32_t block_shift; // log2(block_size) when it is a power of two, else -1
+    int32_t head_size;
+    int32_t value_size;
+    int32_t pos_bytes;   // 1, 2, 4 or 8
+    int32_t pos_signed;
+    int32_t neox;        // pairs half a vector apart (GPT_NEOX) or neighbouring (GPT_J)
+    // element strides
+    int64_t k_src_token_stride, v_src_token_stride;
+    int64_t k_block_stride, k_head_stride, k_slot_stride;
+    int64_t v_block_stride, v_head_stride, v_slot_stride;
+};
+
+struct F16 {
+    using storage = _Float16;
+};
+struct BF16 {
+    using storage = __bf16;
+};
+struct F32 {
+    using storage = float;
+};
+
+__device__ __forceinline__ int64_t loadPosition(const Args &a, int64_t i) {
+    switch (a.pos_bytes) {
+    case 1: return a.pos_signed ? static_cast<const int8_t *>(a.pos_ids)[i] : static_cast<const uint8_t *>(a.pos_ids)[i];
+    case 2: return a.pos_signed ? static_cast<const int16_t *>(a.pos_ids)[i] : static_cast<const uint16_t *>(a.pos_ids)[i];
+    case 4: return a.pos_signed ? static_cast<const int32_t *>(a.pos_ids)[i] : static_cast<const uint32_t *>(a.pos_ids)[i];
+    default: {
+        const int64_t p = static_cast<const int64_t *>(a.pos_ids)[i];
+        return (!a.pos_signed && p < 0) ? INT64_MAX : p; // an unsigned value beyond 2^63: past any table
+    }
+    }
+}
+
+// One pair: every product and the sum rounded to fp32 on its own (no fused multiply-add), as the reference's CPU
+// statement computes it, then one rounding to the storage dtype.
+template <typename S>
+__device__ __forceinline__ void rotatePair(S x0, S x1, S sin_, S cos_, S &y0, S &y1) {
+#pragma clang fp contract(off)
+    const float a = static_cast<float>(x0), b = static_cast<float>(x1);
+    const float s = static_cast<float>(sin_), c = static_cast<float>(cos_);
+    const float ac = a * c, bs = b * s, as = a * s, bc = b * c;
+    y0 = static_cast<S>(ac - bs);
+    y1 = static_cast<S>(as + bc);
+}
+
+template <typename S>
+struct Unit16 {
+    static constexpr int kElements = 16 / sizeof(S);
+    S e[kElements];
+};
+
+// VEC: 16-byte units (see the head of the file); else one pair / one element per step.
+template <typename T, bool VEC>
+__global__ void __launch_bounds__(256) ropeScatterKernel(Args a) {
+    using S = typename T::storage;
+    using U = Unit16<S>;
+    constexpr int kPer = U::kElements;
+    const int64_t token = static_cast<int64_t>(blockIdx.x) * blockDim.z + threadIdx.z;
+    if (token >= a.num_tokens) {
+        return;
+    }
+    const int64_t slot = a.slot_mapping[token];
+    int64_t pos = loadPosition(a, token);
+    // Negative = padding (paged_caching kernel.cuh:61-63). Slots past the pool would be an out-of-bounds
+    // write in the reference; here they are dropped.
+    if (slot < 0 || slot >= a.num_slots) {
+        return;
+    }
+    pos = pos < 0 ? 0 : (pos >= a.table_len ? a.table_len - 1 : pos);
+    int64_t page, row;
+    if (a.block_shift >= 0) {
+        page = slot >> a.block_shift;
+        row = slot & (a.block_size - 1);
+    } else {
+        page = slot / a.block_size;
+        row = slot % a.block_size;
+    }
+    const int table_dim = a.head_size / 2;
+    const S *sin_row = static_cast<const S *>(a.sin_table) + pos * table_dim;
+    const S *cos_row = static_cast<const S *>(a.cos_table) + pos * table_dim;
+
+    for (int head = threadIdx.y; head < a.num_kv_heads; head += blockDim.y) {
+        const S *k_src = static_cast<const S *>(a.k) + token * a.k_src_token_stride + static_cast<int64_t>(head) * a.head_size;
+        const S *v_src = static_cast<const S *>(a.v) + token * a.v_src_token_stride + static_cast<int64_t>(head) * a.value_size;
+        S *k_dst = static_cast<S *>(a.k_cache) + page * a.k_block_stride + head * a.k_head_stride + row * a.k_slot_stride;
+        S *v_dst = static_cast<S *>(a.v_cache) + page * a.v_block_stride + head * a.v_head_stride + row * a.v_slot_stride;
+        if constexpr (VEC) {
+            // unit u of the rotation covers pairs [u * kPer, (u + 1) * kPer)
+            for (int u = threadIdx.x; u < table_dim / kPer; u += blockDim.x) {
+                const int first = a.neox ? u * kPer : 2 * u * kPer;                 // elements of the first unit
+                const int second = a.neox ? table_dim + u * kPer : 2 * u * kPer + kPer;
+                const U x_lo = *reinterpret_cast<const U *>(k_src + first);
+                const U x_hi = *reinterpret_cast<const U *>(k_src + second);
+                const U sn = *reinterpret_cast<const U *>(sin_row + u * kPer);
+                const U cs = *reinterpret_cast<const U *>(cos_row + u * kPer);
+                U y_lo, y_hi;
+                if (a.neox) {
+#pragma unroll
+                    for (int i = 0; i < kPer; ++i) {
+                        rotatePair(x_lo.e[i], x_hi.e[i], sn.e[i], cs.e[i], y_lo.e[i], y_hi.e[i]);
+                    }
+                } else {
+                    // the 2 kPer elements are kPer neighbouring pairs: pair i = elements 2 i, 2 i + 1
+#pragma unroll
+                    for (int i = 0; i < kPer / 2; ++i) {
+                        rotatePair(x_lo.e[2 * i], x_lo.e[2 * i + 1], sn.e[i], cs.e[i], y_lo.e[2 * i], y_lo.e[2 * i + 1]);
+                        rotatePair(x_hi.e[2 * i], x_hi.e[2 * i + 1], sn.e[kPer / 2 + i], cs.e[kPer / 2 + i], y_hi.e[2 * i],
+                                   y_hi.e[2 * i + 1]);
+                    }
+                }
+                *reinterpret_cast<U *>(k_dst + first) = y_lo;
+                *reinterpret_cast<U *>(k_dst + second) = y_hi;
+            }
+            for (int u = threadIdx.x; u < a.value_size / kPer; u += blockDim.x) {
+                *reinterpret_cast<U *>(v_dst + u * kPer) = *reinterpret_cast<const U *>(v_src + u * kPer);
+            }
+        } else {
+            for (int j = threadIdx.x; j < table_dim; j += blockDim.x) {
+                const int first = a.neox ? j : 2 * j;
+                const int second = a.neox ? j + table_dim : 2 * j + 1;
+                S y0, y1;
+                rotatePair(k_src[first], k_src[second], sin_row[j], cos_row[j], y0, y1);
+                k_dst[first] = y0;
+                k_dst[second] = y1;
+            }
+            for (int j = threadIdx.x; j < a.value_size; j += blockDim.x) {
+                v_dst[j] = v_src[j];
+            }
+        }
+    }
+}
+
+int ceilPow2(int x) {
+    int p = 1;
+    while (p < x) {
+        p <<= 1;
+    }
+    return p;
+}
+
+bool multipleOf16(uint64_t x) { return (x & 15u) == 0; }
+
+template <typename T>
+void launch(const Args &a, bool vec, int row_steps, hipStream_t stream) {
+    // 256-thread box: x = steps along a row, y = heads, z = tokens
+    int bx = ceilPow2(row_steps);
+    bx = bx > 64 ? 64 : bx;
+    int by = ceilPow2(a.num_kv_heads);
+    by = by > 256 / bx ? 256 / bx : by;
+    const int bz = 256 / (bx * by);
+    const dim3 block(bx, by, bz);
+    const dim3 grid(static_cast<unsigned>((a.num_tokens + bz - 1) / bz));
+    if (vec) {
+        ropeScatterKernel<T, true><<<grid, block, 0, stream>>>(a);
+    } else {
+        ropeScatterKernel<T, false><<<grid, block, 0, stream>>>(a);
+    }
+}
+
+} // namespace
+
+struct Descriptor::Opaque {};
+
+Descriptor::~Descriptor() { delete _opaque; }
+
+infiniStatus_t Descriptor::create(infiniopHandle_t handle, Descriptor **desc_ptr, infiniopTensorDescriptor_t k_cache_desc,
+                                  infiniopTensorDescriptor_t v_cache_desc, infiniopTensorDescriptor_t k_desc,
+                                  infiniopTensorDescriptor_t v_desc, infiniopTensorDescriptor_t slot_mapping_desc,
+                                  infiniopTensorDescriptor_t pos_ids_desc, infiniopTensorDescriptor_t sin_table_desc,
+                                  infiniopTensorDescriptor_t cos_table_desc, infiniopRoPEAlgo_t algo) {
+    auto info = RoPEPagedCachingInfo::create(k_cache_desc, v_cache_desc, k_desc, v_desc, slot_mapping_desc, pos_ids_desc,
+                                             sin_table_desc, cos_table_desc, algo);
+    CHECK_RESULT(info);
+    *desc_ptr = new Descriptor(new Opaque{}, info.take(), 0, handle->device, handle->device_id);
+    return INFINI_STATUS_SUCCESS;
+}
+
+infiniStatus_t Descriptor::calculate(void *workspace, size_t workspace_size, void *k_cache, void *v_cache, const void *k,
+                                     const void *v, const void *slot_mapping, const void *pos_ids, const void *sin_table,
+                                     const void *cos_table, void *stream_) const {
+    (void)workspace;
+    (void)workspace_size;
+    const auto &in = _info.scatter;
+    if (in.num_tokens == 0 || in.num_kv_heads == 0 || (in.head_size == 0 && in.v_head_size == 0)) {
+        return INFINI_STATUS_SUCCESS;
+    }
+    if (k_cache == nullptr || v_cache == nullptr || k == nullptr || v == nullptr || slot_mapping == nullptr
+        || pos_ids == nullptr || sin_table == nullptr || cos_table == nullptr) {
+        return INFINI_STATUS_NULL_POINTER;
+    }
+    if (_info.table_len == 0 && in.head_size > 0) {
+        return INFINI_STATUS_BAD_PARAM; // no row of the tables to rotate with
+    }
+    int current_device = -1;
+    if (hipGetDevice(&current_device) != hipSuccess || current_device != device_id) {
+        return INFINI_STATUS_BAD_PARAM;
+    }
+
+    Args a{};
+    a.k_cache = k_cache;
+    a.v_cache = v_cache;
+    a.k = k;
+    a.v = v;
+    a.slot_mapping = static_cast<const int64_t *>(slot_mapping);
+    a.pos_ids = pos_ids;
+    a.sin_table = sin_table;
+    a.cos_table = cos_table;
+    a.num_tokens = static_cast<int64_t>(in.num_tokens);
+    a.num_slots = static_cast<int64_t>(in.num_blocks) * static_cast<int64_t>(in.block_size);
+    a.table_len = static_cast<int64_t>(_info.table_len);
+    a.num_kv_heads = static_cast<int32_t>(in.num_kv_heads);
+    a.block_size = static_cast<int32_t>(in.block_size);
+    a.block_shift = -1;
+    if (in.block_size > 0 && (in.block_size & (in.block_size - 1)) == 0) {
+        a.block_shift = __builtin_ctzll(in.block_size);
+    }
+    a.head_size = static_cast<int32_t>(in.head_size);
+    a.value_size = static_cast<int32_t>(in.v_head_size);
+    a.pos_bytes = static_cast<int32_t>(infiniSizeOf(_info.pos_dtype));
+    a.pos_signed = _info.pos_dtype == INFINI_DTYPE_I8 || _info.pos_dtype == INFINI_DTYPE_I16
+                || _info.pos_dtype == INFINI_DTYPE_I32 || _info.pos_dtype == INFINI_DTYPE_I64;
+    a.neox = _info.algo == INFINIOP_ROPE_ALGO_GPT_NEOX;
+    a.k_src_token_stride = in.k_src_stride;
+    a.v_src_token_stride = in.v_src_stride;
+    a.k_block_stride = in.k_cache_block_stride;
+    a.k_head_stride = in.k_cache_head_stride;
+    a.k_slot_stride = in.k_cache_slot_stride;
+    a.v_block_stride = in.v_cache_block_stride;
+    a.v_head_stride = in.v_cache_head_stride;
+    a.v_slot_stride = in.v_cache_slot_stride;
+
+    // 16-byte units when every size, stride and base address allows them
+    const uint64_t es = infiniSizeOf(in.dtype);
+    auto bytes = [es](ptrdiff_t elements) { return static_cast<uint64_t>(elements) * es; };
+    const int per = static_cast<int>(16 / es);
+    bool vec = (_info.table_dim % per) == 0 && (in.v_head_size % per) == 0;
+    for (uint64_t quantity : {bytes(in.head_size), bytes(in.v_head_size), bytes(in.k_src_stride), bytes(in.v_src_stride),
+                              bytes(in.k_cache_block_stride), bytes(in.k_cache_head_stride), bytes(in.k_cache_slot_stride),
+                              bytes(in.v_cache_block_stride), bytes(in.v_cache_head_stride), bytes(in.v_cache_slot_stride),
+                              static_cast<uint64_t>(reinterpret_cast<uintptr_t>(k_cache)),
+                              static_cast<uint64_t>(reinterpret_cast<uintptr_t>(v_cache)),
+                              static_cast<uint64_t>(reinterpret_cast<uintptr_t>(k)),
+                              static_cast<uint64_t>(reinterpret_cast<uintptr_t>(v)),
+                              static_cast<uint64_t>(reinterpret_cast<uintptr_t>(sin_table)),
+                              static_cast<uint64_t>(reinterpret_cast<uintptr_t>(cos_table)),
+                              bytes(static_cast<ptrdiff_t>(_info.table_dim))}) {
+        vec = vec && multipleOf16(quantity);
+    }
+    const int rotate_steps = static_cast<int>(vec ? _info.table_dim / per : _info.table_dim);
+    const int copy_steps = static_cast<int>(vec ? in.v_head_size / per : in.v_head_size);
+    const int row_steps = rotate_steps > copy_steps ? rotate_steps : copy_steps;
+    auto stream = static_cast<hipStream_t>(stream_);
+    switch (in.dtype) {
+    case INFINI_DTYPE_F16: launch<F16>(a, vec, row_steps > 0 ? row_steps : 1, stream); break;
+    case INFINI_DTYPE_BF16: launch<BF16>(a, vec, row_steps > 0 ? row_steps : 1, stream); break;
+    case INFINI_DTYPE_F32: launch<F32>(a, vec, row_steps > 0 ? row_steps : 1, stream); break;
+    default: return INFINI_STATUS_BAD_TENSOR_DTYPE;
+    }
+    return hipGetLastError() == hipSuccess ? INFINI_STATUS_SUCCESS : INFINI_STATUS_INTERNAL_ERROR;
+}
+
+} // namespace op::rope_paged_caching::amd

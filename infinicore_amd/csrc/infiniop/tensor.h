@@ -20,6 +20,17 @@ struct InfiniopTensorDescriptor {
     size_t dim(size_t i) const { return _shape[i]; }
     const std::vector<ptrdiff_t> &strides() const { return _strides; }
     ptrdiff_t stride(size_t i) const { return _strides[i]; }
+    // packed row-major strides (dimensions of extent 1 may carry any stride)
+    bool isContiguous() const {
+        ptrdiff_t expected = 1;
+        for (size_t i = _shape.size(); i-- > 0;) {
+            if (_shape[i] != 1 && _strides[i] != expected) {
+                return false;
+            }
+            expected *= static_cast<ptrdiff_t>(_shape[i]);
+        }
+        return true;
+    }
     size_t numel() const {
         size_t n = 1;
         for (size_t d : _shape) {

@@ -16,7 +16,7 @@
 -- The sources are the ones under infinicore_amd/csrc of this repository, copied to the matching
 -- places of the reference tree (src/infinirt/amd, src/infiniop/devices/amd,
 -- src/infiniop/ops/paged_attention/amd, src/infiniop/ops/paged_attention_prefill/amd,
--- src/infiniop/ops/paged_caching/amd, src/infiniop/ops/kv_caching/amd).
+-- src/infiniop/ops/paged_caching/amd, src/infiniop/ops/kv_caching/amd, src/infiniop/ops/rope_paged_caching/amd).
 -- xmake is not installed in the environment this file was written in; the Makefile next to it builds
 -- the same objects with the same flags and is what the tests use.
 
@@ -86,6 +86,7 @@ target("infiniop-amd")
     add_cxflags("-fPIC")
     add_files("../src/infiniop/devices/amd/*.cc")
     add_files("../src/infiniop/ops/kv_caching/amd/*.hip")
+    add_files("../src/infiniop/ops/rope_paged_caching/amd/*.hip")
     -- the scatter kernel gets its first 14 argument words in scalar registers at wavefront start
     add_files("../src/infiniop/ops/paged_caching/amd/*.hip", {cxflags = {"-mllvm", "-amdgpu-kernarg-preload-count=14"}})
     -- the attention kernels keep their matrix-instruction accumulators in ordinary vector registers

@@ -45,14 +45,23 @@ class InfiniDevice:
 
 class InfiniDtype:
     INVALID = 0
+    I8 = 3
+    I16 = 4
     I32 = 5
     I64 = 6
     U8 = 7
+    U16 = 8
     U32 = 9
+    U64 = 10
     F16 = 12
     F32 = 13
     F64 = 14
     BF16 = 19
+
+
+class RoPEAlgo:
+    GPT_J = 0     # pairs are neighbours: (2j, 2j + 1)
+    GPT_NEOX = 1  # pairs are half a vector apart: (j, j + d / 2)
 
 
 class Handle(Structure):
@@ -164,6 +173,10 @@ def _open():
     _declare(op, "infiniopGetPagedCachingWorkspaceSize", [D, POINTER(c_size_t)])
     _declare(op, "infiniopPagedCaching", [D, vp, c_size_t, vp, vp, vp, vp, vp, vp])
     _declare(op, "infiniopDestroyPagedCachingDescriptor", [D])
+    _declare(op, "infiniopCreateRoPEPagedCachingDescriptor", [infiniopHandle_t, POINTER(D), T, T, T, T, T, T, T, T, c_int])
+    _declare(op, "infiniopGetRoPEPagedCachingWorkspaceSize", [D, POINTER(c_size_t)])
+    _declare(op, "infiniopRoPEPagedCaching", [D, vp, c_size_t, vp, vp, vp, vp, vp, vp, vp, vp, vp])
+    _declare(op, "infiniopDestroyRoPEPagedCachingDescriptor", [D])
     _declare(op, "infiniopCreateKVCachingDescriptor", [infiniopHandle_t, POINTER(D), T, T, T, T, T])
     _declare(op, "infiniopGetKVCachingWorkspaceSize", [D, POINTER(c_size_t)])
     _declare(op, "infiniopKVCaching", [D, vp, c_size_t, vp, vp, vp, vp, vp, vp])

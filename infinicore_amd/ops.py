@@ -28,6 +28,10 @@ _TORCH_TO_INFINI = {
     torch.int32: InfiniDtype.I32,
     torch.uint32: InfiniDtype.U32,
     torch.uint8: InfiniDtype.U8,
+    torch.int8: InfiniDtype.I8,
+    torch.int16: InfiniDtype.I16,
+    torch.uint16: InfiniDtype.U16,
+    torch.uint64: InfiniDtype.U64,
 }
 
 _PLAN_CACHE_CAPACITY = 100  # the reference keeps a thread-local LRU of 100 descriptors per operator
@@ -230,6 +234,43 @@ def paged_caching(k_cache, v_cache, k, v, slot_mapping):
             _ptr(v), _ptr(slot_mapping), _stream_ptr(index),
         ),
         "infiniopPagedCaching",
+    )
+    return k_cache, v_cache
+
+
+def rope_paged_caching(k_cache, v_cache, k, v, slot_mapping, pos_ids, sin_table, cos_table, algo: int = lib.RoPEAlgo.GPT_NEOX):
+    """Rotate ``k`` [num_tokens, num_kv_heads, head_size] by the rows ``pos_ids`` of the sin / cos tables
+    [table_len, head_size / 2] and scatter it, and ``v`` unchanged, into their slots of the paged pools, in one
+    launch; returns the pools. The result of the reference's ``rope`` followed by ``paged_caching``
+    (python/infinicore/ops/paged_caching.py:5-15 for the scatter's argument order)."""
+    index = _device_index(k)
+    tensors = (k_cache, v_cache, k, v, slot_mapping, pos_ids, sin_table, cos_table)
+    key = ("rope_paged_caching", index, _stream_key(index), int(algo), *(_meta(t) for t in tensors))
+
+    def make():
+        handle = _handle_for(index)
+        descs = [_describe(t) for t in tensors]
+        op = lib.infiniopOperatorDescriptor_t()
+        try:
+            check_error(
+                LIBINFINIOP.infiniopCreateRoPEPagedCachingDescriptor(handle, ctypes.byref(op), *descs, int(algo)),
+                "infiniopCreateRoPEPagedCachingDescriptor",
+            )
+        finally:
+            for d in descs:
+                lib.destroy_tensor_descriptor(d)
+        size = c_size_t(0)
+        check_error(LIBINFINIOP.infiniopGetRoPEPagedCachingWorkspaceSize(op, ctypes.byref(size)))
+        return _Plan(op, LIBINFINIOP.infiniopDestroyRoPEPagedCachingDescriptor, size.value, k.device)
+
+    plan = _cached_plan(key, make)
+    lib.set_device(InfiniDevice.AMD, index)
+    check_error(
+        LIBINFINIOP.infiniopRoPEPagedCaching(
+            plan.descriptor, _ptr(plan.workspace), plan.workspace_bytes, _ptr(k_cache), _ptr(v_cache), _ptr(k),
+            _ptr(v), _ptr(slot_mapping), _ptr(pos_ids), _ptr(sin_table), _ptr(cos_table), _stream_ptr(index),
+        ),
+        "infiniopRoPEPagedCaching",
     )
     return k_cache, v_cache
 

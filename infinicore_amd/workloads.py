@@ -93,6 +93,15 @@ CACHING_CONFIGS = {
 }
 
 
+# rotary embedding of K fused with the scatter (infiniopRoPEPagedCaching): the decode step's producer (one token per
+# sequence) and a prefill chunk; positions drawn from a table of 8192 rows, pairs half a vector apart (GPT-NeoX)
+ROPE_CACHING_TABLE_LEN = 8192
+ROPE_CACHING_CONFIGS = {
+    "r1_rope_scatter_decode_step": CachingConfig("r1_rope_scatter_decode_step", torch.bfloat16, 32, 8, 128, 16, 65536, 0.0, seed=401),
+    "r2_rope_scatter_prefill_chunk": CachingConfig("r2_rope_scatter_prefill_chunk", torch.bfloat16, 4096, 8, 128, 16, 65536, 0.05, seed=402),
+}
+
+
 @dataclass
 class KVCachingConfig:
     """Append to contiguous (non-paged) caches: ``new_tokens`` tokens per sequence behind random past lengths."""
@@ -273,6 +282,29 @@ def make_caching_inputs(cfg: CachingConfig) -> CachingInputs:
     k_cache = torch.full(shape, -777.0, dtype=cfg.dtype)
     v_cache = torch.full(shape, 555.0, dtype=cfg.dtype)
     return CachingInputs(cfg, k, v, k_cache, v_cache, torch.from_numpy(slots))
+
+
+def make_rope_tables(table_len: int, head_size: int, dtype: torch.dtype, theta: float = 10000.0):
+    """sin / cos tables [table_len, head_size / 2] as the reference's RoPE test builds them
+    (test/infiniop/rope.py:124-131)."""
+    freqs = 1.0 / (theta ** (torch.arange(0, head_size, 2).float() / head_size))
+    angles = torch.outer(torch.arange(table_len).float(), freqs)
+    return torch.sin(angles).to(dtype), torch.cos(angles).to(dtype)
+
+
+def make_rope_caching_inputs(cfg: CachingConfig):
+    """The scatter's inputs plus one position per token and the tables: (CachingInputs, pos_ids, sin, cos)."""
+    inp = make_caching_inputs(cfg)
+    rng = np.random.default_rng([cfg.seed, 13])
+    pos = torch.from_numpy(rng.integers(0, ROPE_CACHING_TABLE_LEN, cfg.num_tokens).astype(np.int64))
+    sin, cos = make_rope_tables(ROPE_CACHING_TABLE_LEN, cfg.head_size, cfg.dtype)
+    return inp, pos, sin, cos
+
+
+def rope_caching_algorithmic_bytes(cfg: CachingConfig, slot_mapping) -> int:
+    """The scatter's bytes plus one position and one row of each table per token."""
+    e = 2 if cfg.dtype in (torch.float16, torch.bfloat16) else 4
+    return caching_algorithmic_bytes(cfg, slot_mapping) + cfg.num_tokens * (8 + 2 * (cfg.head_size // 2) * e)
 
 
 @dataclass

@@ -26,6 +26,10 @@
  *   oracle_paged_caching           src/infiniop/ops/paged_caching/cuda/kernel.cuh:22-89
  *                                  (slot < 0 skipped, page = slot / block_size, row = slot % block_size,
  *                                  source heads packed, element-wise copy)
+ *   oracle_rope_paged_caching      src/infiniop/ops/rope/cpu/rope_cpu.cc:56-98 (pairs (2j, 2j + 1) or (j, j + d / 2),
+ *                                  y0 = x0 cos - x1 sin, y1 = x0 sin + x1 cos in fp32, every product and sum
+ *                                  rounded on its own, one rounding to the storage dtype) followed by the slot
+ *                                  scatter of oracle_paged_caching, without the tensor in between
  *   oracle_kv_caching              src/infiniop/ops/kv_caching/cuda/kernel.cuh:32-58
  *                                  (element (b, h, s, d) of the new tensors goes to cache position
  *                                  past_kv_lengths[b] + s; every dimension of every tensor strided)
@@ -405,6 +409,66 @@ int oracle_paged_caching(void *k_cache_, void *v_cache_, const void *k_, const v
             for (int64_t i = 0; i < s->v_head_size; ++i) {
                 memcpy(v_dst + i * es, v_src + i * es, (size_t)es);
             }
+        }
+    }
+    return 0;
+}
+
+/* Rotary embedding of K (rope_cpu.cc:56-98, one position per token) fused with the slot scatter above.
+ * dtype: ORACLE_DTYPE_F16 / BF16, or 2 for fp32. neox: pairs half a vector apart, else neighbouring. A position
+ * outside the tables uses the nearest row (the reference reads out of bounds); returns -1 for arguments it
+ * cannot take. */
+int oracle_rope_paged_caching(void *k_cache_, void *v_cache_, const void *k_, const void *v_, const int64_t *slot_mapping,
+                              const int64_t *pos_ids, const void *sin_table_, const void *cos_table_, int64_t table_len,
+                              int dtype, int neox, const oracle_caching_shape *s) {
+    const int64_t es = dtype == 2 ? 4 : 2;
+    if (s->block_size <= 0 || s->elem_size != es || (s->head_size & 1) || table_len <= 0 || dtype < 0 || dtype > 2) {
+        return -1;
+    }
+    char *k_cache = (char *)k_cache_, *v_cache = (char *)v_cache_;
+    const char *k = (const char *)k_, *v = (const char *)v_;
+    const char *sin_table = (const char *)sin_table_, *cos_table = (const char *)cos_table_;
+    const int64_t half = s->head_size / 2;
+    for (int64_t tok = 0; tok < s->num_tokens; ++tok) {
+        const int64_t slot = slot_mapping[tok];
+        if (slot < 0) {
+            continue;
+        }
+        int64_t pos = pos_ids[tok];
+        pos = pos < 0 ? 0 : (pos >= table_len ? table_len - 1 : pos);
+        const int64_t page = slot / s->block_size, row = slot % s->block_size;
+        for (int64_t head = 0; head < s->num_kv_heads; ++head) {
+            const char *k_src = k + (tok * s->k_src_stride + head * s->head_size) * es;
+            const char *v_src = v + (tok * s->v_src_stride + head * s->v_head_size) * es;
+            char *k_dst = k_cache + (page * s->k_cache_block_stride + head * s->k_cache_head_stride + row * s->k_cache_slot_stride) * es;
+            char *v_dst = v_cache + (page * s->v_cache_block_stride + head * s->v_cache_head_stride + row * s->v_cache_slot_stride) * es;
+            for (int64_t j = 0; j < half; ++j) {
+                const int64_t p0 = neox ? j : 2 * j, p1 = neox ? j + half : 2 * j + 1;
+                float x0, x1, sn, cs;
+                if (dtype == 2) {
+                    memcpy(&x0, k_src + p0 * 4, 4);
+                    memcpy(&x1, k_src + p1 * 4, 4);
+                    memcpy(&sn, sin_table + (pos * half + j) * 4, 4);
+                    memcpy(&cs, cos_table + (pos * half + j) * 4, 4);
+                } else {
+                    x0 = load_elem((const uint16_t *)(k_src + p0 * 2), dtype);
+                    x1 = load_elem((const uint16_t *)(k_src + p1 * 2), dtype);
+                    sn = load_elem((const uint16_t *)(sin_table + (pos * half + j) * 2), dtype);
+                    cs = load_elem((const uint16_t *)(cos_table + (pos * half + j) * 2), dtype);
+                }
+                /* four products and two sums, each rounded to fp32 (no fused multiply-add) */
+                volatile float x0c = x0 * cs, x1s = x1 * sn, x0s = x0 * sn, x1c = x1 * cs;
+                const float y0 = x0c - x1s, y1 = x0s + x1c;
+                if (dtype == 2) {
+                    memcpy(k_dst + p0 * 4, &y0, 4);
+                    memcpy(k_dst + p1 * 4, &y1, 4);
+                } else {
+                    const uint16_t b0 = store_elem(y0, dtype), b1 = store_elem(y1, dtype);
+                    memcpy(k_dst + p0 * 2, &b0, 2);
+                    memcpy(k_dst + p1 * 2, &b1, 2);
+                }
+            }
+            memcpy(v_dst, v_src, (size_t)(s->v_head_size * es));
         }
     }
     return 0;

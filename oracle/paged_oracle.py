@@ -80,6 +80,9 @@ def load():
         lib.oracle_paged_attention_prefill.restype = c_int
         lib.oracle_paged_caching.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, POINTER(CachingShape)]
         lib.oracle_paged_caching.restype = c_int
+        lib.oracle_rope_paged_caching.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                                  c_void_p, c_int64, c_int, c_int, POINTER(CachingShape)]
+        lib.oracle_rope_paged_caching.restype = c_int
         lib.oracle_kv_caching.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, POINTER(KVCachingShape)]
         lib.oracle_kv_caching.restype = c_int
         lib.oracle_to_float.argtypes = [ctypes.c_uint16, c_int]
@@ -189,6 +192,46 @@ def paged_caching(k_cache, v_cache, k, v, slot_mapping):
     if rc != 0:
         raise ValueError("oracle rejected the arguments")
     return k_cache, v_cache
+
+
+def rope_paged_caching(k_cache, v_cache, k, v, slot_mapping, pos_ids, sin_table, cos_table, neox: bool):
+    """C oracle rotary embedding of K fused with the scatter of K and V; writes into the caches in place and
+    returns them. ``neox``: pairs half a vector apart (GPT-NeoX), else neighbouring (GPT-J)."""
+    lib = load()
+    slot_mapping = _cpu(slot_mapping).to(torch.int64).contiguous()
+    pos_ids = _cpu(pos_ids).to(torch.int64).contiguous()
+    sin_table, cos_table = _cpu(sin_table).contiguous(), _cpu(cos_table).contiguous()
+    code = {torch.float16: 0, torch.bfloat16: 1, torch.float32: 2}[k.dtype]
+    s = CachingShape(
+        k.element_size(), slot_mapping.shape[0], k.shape[1], k.shape[2], v.shape[2], k_cache.shape[2],
+        k.stride(0), v.stride(0), k_cache.stride(0), v_cache.stride(0),
+        k_cache.stride(1), v_cache.stride(1), k_cache.stride(2), v_cache.stride(2),
+    )
+    rc = lib.oracle_rope_paged_caching(_cpu(k_cache).data_ptr(), _cpu(v_cache).data_ptr(), _cpu(k).data_ptr(),
+                                       _cpu(v).data_ptr(), slot_mapping.data_ptr(), pos_ids.data_ptr(), sin_table.data_ptr(),
+                                       cos_table.data_ptr(), sin_table.shape[0], code, int(bool(neox)), ctypes.byref(s))
+    if rc != 0:
+        raise ValueError("oracle rejected the arguments")
+    return k_cache, v_cache
+
+
+def torch_reference_rope(x, pos_ids, sin_table, cos_table, neox: bool):
+    """The expected-value function of the reference's RoPE test on the CPU (test/infiniop/rope.py:84-121), restated:
+    operands widened to fp32, ``t1 * cos - t2 * sin`` and ``t1 * sin + t2 * cos`` as separate tensor operations, one
+    cast back. ``x`` is [tokens, heads, d]; returns the rotated tensor."""
+    sin = sin_table[pos_ids.long()].float().unsqueeze(1)
+    cos = cos_table[pos_ids.long()].float().unsqueeze(1)
+    out = torch.empty_like(x)
+    if neox:
+        half = x.shape[-1] // 2
+        t1, t2 = x[..., :half].float(), x[..., half:].float()
+        out[..., :half] = (t1 * cos - t2 * sin).to(x.dtype)
+        out[..., half:] = (t1 * sin + t2 * cos).to(x.dtype)
+    else:
+        t1, t2 = x[..., 0::2].float(), x[..., 1::2].float()
+        out[..., 0::2] = (t1 * cos - t2 * sin).to(x.dtype)
+        out[..., 1::2] = (t1 * sin + t2 * cos).to(x.dtype)
+    return out
 
 
 def kv_caching(k_cache, v_cache, k, v, past_kv_lengths):

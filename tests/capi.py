@@ -18,6 +18,11 @@ TORCH_TO_INFINI = {
     torch.int64: L.InfiniDtype.I64,
     torch.int32: L.InfiniDtype.I32,
     torch.uint32: L.InfiniDtype.U32,
+    torch.int8: L.InfiniDtype.I8,
+    torch.uint8: L.InfiniDtype.U8,
+    torch.int16: L.InfiniDtype.I16,
+    torch.uint16: L.InfiniDtype.U16,
+    torch.uint64: L.InfiniDtype.U64,
 }
 
 
@@ -132,6 +137,34 @@ def run_paged_caching(handle, k_cache, v_cache, k, v, slot_mapping, stream=None)
     )
     torch.cuda.synchronize()
     L.check_error(L.LIBINFINIOP.infiniopDestroyPagedCachingDescriptor(op))
+    return k_cache, v_cache
+
+
+def create_rope_paged_caching(handle, k_cache, v_cache, k, v, slot_mapping, pos_ids, sin_table, cos_table, algo):
+    descs = [describe(t) for t in (k_cache, v_cache, k, v, slot_mapping, pos_ids, sin_table, cos_table)]
+    op = L.infiniopOperatorDescriptor_t()
+    status = L.LIBINFINIOP.infiniopCreateRoPEPagedCachingDescriptor(handle, ctypes.byref(op), *descs, int(algo))
+    for d in descs:
+        L.destroy_tensor_descriptor(d)
+    return status, op
+
+
+def run_rope_paged_caching(handle, k_cache, v_cache, k, v, slot_mapping, pos_ids, sin_table, cos_table, algo, stream=None):
+    """In place on the device pools; returns them."""
+    status, op = create_rope_paged_caching(handle, k_cache, v_cache, k, v, slot_mapping, pos_ids, sin_table, cos_table, algo)
+    L.check_error(status, "infiniopCreateRoPEPagedCachingDescriptor")
+    size = c_size_t(123)
+    L.check_error(L.LIBINFINIOP.infiniopGetRoPEPagedCachingWorkspaceSize(op, ctypes.byref(size)))
+    assert size.value == 0
+    torch.cuda.synchronize()
+    L.check_error(
+        L.LIBINFINIOP.infiniopRoPEPagedCaching(op, c_void_p(0), 0, ptr(k_cache), ptr(v_cache), ptr(k), ptr(v),
+                                               ptr(slot_mapping), ptr(pos_ids), ptr(sin_table), ptr(cos_table),
+                                               c_void_p(stream or 0)),
+        "infiniopRoPEPagedCaching",
+    )
+    torch.cuda.synchronize()
+    L.check_error(L.LIBINFINIOP.infiniopDestroyRoPEPagedCachingDescriptor(op))
     return k_cache, v_cache
 
 
