@@ -300,6 +300,12 @@ infiniStatus_t Descriptor::launch(void *workspace, void *out, const void *q, con
         a.seq_pieces = reinterpret_cast<int2 *>(ws + plan.acc_bytes + 2 * plan.ml_bytes);
         a.seg_flags = reinterpret_cast<unsigned long long *>(ws + plan.acc_bytes + 2 * plan.ml_bytes + plan.pieces_bytes);
         a.token = nextToken();
+        // the 64-head latent-attention kernel plans its units per call from the actual lengths and leaves the
+        // partition size it chose in the first word of the pieces region, for the merge kernel
+        if (plan.latent_wide && !plan.partition_forced && in.num_seqs <= 256 && plan.tiled && aligned16(out) && aligned16(q)
+            && aligned16(k_cache) && aligned16(v_cache)) {
+            a.chosen_partition = reinterpret_cast<int32_t *>(ws + plan.acc_bytes + 2 * plan.ml_bytes);
+        }
     }
     a.scale_log2 = in.scale * kLog2e;
     a.num_seqs = static_cast<int32_t>(in.num_seqs);

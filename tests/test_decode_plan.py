@@ -11,12 +11,12 @@ ROOT = Path(__file__).resolve().parents[1]
 KNOBS = ("INFINIOP_AMD_PA_KERNEL", "INFINIOP_AMD_PA_SCHEDULE", "INFINIOP_AMD_PA_LATENT_KERNEL",
          "INFINIOP_AMD_PA_PARTITION", "INFINIOP_AMD_PA_WAVES_PER_CU")
 FIELDS = ("tiled", "balanced", "latent_wide", "partition_tokens", "max_partitions", "fallback_partition_tokens",
-          "fallback_max_partitions", "waves_per_stream", "workspace_bytes", "launchable")
+          "fallback_max_partitions", "waves_per_stream", "workspace_bytes", "launchable", "acc_bytes", "ml_bytes")
 
 
-@pytest.fixture(scope="module")
-def probe(tmp_path_factory):
-    out = tmp_path_factory.mktemp("plan") / "libplanprobe.so"
+def build_probe(directory):
+    """Compiles tests/plan_probe.cc with the host compiler; returns plan(num_seqs, num_heads, ...) -> dict."""
+    out = directory / "libplanprobe.so"
     subprocess.run(["g++", "-std=c++17", "-O1", "-shared", "-fPIC", f"-I{ROOT / 'include'}",
                     f"-I{ROOT / 'infinicore_amd' / 'csrc'}", str(ROOT / "tests" / "plan_probe.cc"), "-o", str(out)],
                    check=True, capture_output=True, text=True)
@@ -33,6 +33,11 @@ def probe(tmp_path_factory):
         return dict(zip(FIELDS, res))
 
     return plan
+
+
+@pytest.fixture(scope="module")
+def probe(tmp_path_factory):
+    return build_probe(tmp_path_factory.mktemp("plan"))
 
 
 @pytest.fixture(autouse=True)

@@ -356,6 +356,30 @@ def test_mla_empty_and_negative_lengths_in_the_per_call_plan(gpu_handle, oracle)
     assert_close(out, want, "mla_empty")
 
 
+def test_mla_per_call_plan_is_in_use(gpu_handle, tmp_path):
+    """The 64-head kernel chooses its partition size per call from the actual lengths and leaves it in the
+    workspace for the merge kernel (first word behind the partial results): after a call that word holds a
+    size the plan can produce, not the bytes the workspace was filled with."""
+    from test_decode_plan import build_probe
+
+    inp = workloads.make_decode_inputs(mla("mla_planned", torch.bfloat16, 8, 128, 16, 600, 2500, seed=465))
+    q, k, v, bt, sl = to_device(inp)
+    out = torch.zeros((8, 128, 512), dtype=torch.bfloat16, device=DEV)
+    status, op = create_paged_attention(gpu_handle, out, q, k, v, bt, sl, None, inp.scale)
+    assert status == 0
+    size = workspace_size_attention(op)
+    ws = torch.full((size,), 0xFF, dtype=torch.uint8, device=DEV)
+    assert ws.data_ptr() % 256 == 0
+    L.check_error(L.LIBINFINIOP.infiniopPagedAttention(op, ptr(ws), size, ptr(out), ptr(q), ptr(k), ptr(v), ptr(bt), ptr(sl), None, None))
+    torch.cuda.synchronize()
+    L.check_error(L.LIBINFINIOP.infiniopDestroyPagedAttentionDescriptor(op))
+    plan = build_probe(tmp_path)(8, 128, 1, 576, 16, bt.shape[1], value_size=512, num_blocks=k.shape[0])
+    assert plan["latent_wide"] and plan["workspace_bytes"] == size
+    offset = plan["acc_bytes"] + 2 * plan["ml_bytes"]
+    chosen = int(ws[offset:offset + 4].view(torch.int32).item())
+    assert 128 <= chosen <= 1024 and chosen % 64 == 0, chosen
+
+
 def test_mla_more_sequences_than_the_per_call_plan_handles(gpu_handle, oracle):
     """More than 256 sequences: fixed partitions on the three-dimensional grid."""
     run_case(gpu_handle, oracle, workloads.make_decode_inputs(mla("mla_b300", torch.bfloat16, 300, 32, 16, 1, 400, seed=470)))
