@@ -37,16 +37,28 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E
 MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 / fp16 matrix peak
 
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
-# file, each scaled by what the same counter reads for a 256 MiB copy (summaries and commands: profiles/).
-# Counters cannot be read from inside this process, so the figures are recorded here, per workload.
-MEASURED_TRAFFIC_BYTES = {
-    "c2_llama3_8b_b32": 322_300_000,       # decodeBalancedKernel: 319.7 MB fetched + 2.6 MB written
-    "m1_mla_16_heads_b32": 155_000_000,    # decodeMlaWideKernel<.., 1>: 146.4 MB fetched + 8.6 MB written
-    "m2_mla_128_heads_b32": 215_500_000,   # decodeMlaWideKernel: 184.1 MB fetched + 31.4 MB written
-    "c5_prefill_scatter": 32_100_000,      # pagedCachingScatterKernel: 16.2 MB fetched + 15.9 MB written
-    "k2_append_prefill_chunk": 33_600_000, # kvCachingAppendKernel: 16.8 MB fetched + 16.8 MB written
-    "p3_llama3_8b_chunked": 451_500_000,   # prefillTiledKernel: fetched (writes: the 44 MB output)
+# file, each scaled by what the same counter reads for a 256 MiB copy. Counters cannot be read from inside
+# this process, so the figures are recorded here per workload, each with the summary under profiles/ that
+# holds the command and the raw counter values, and the commit whose kernel sources were measured (a later
+# change to that kernel makes the figure stale until it is collected again).
+MEASURED_TRAFFIC = {
+    # workload: (bytes, summary under profiles/, commit of the measured kernel)
+    "c2_llama3_8b_b32": (322_300_000, "decode_balanced_c2_llama3_8b_b32_hbm_traffic.md", "869e7ad"),
+    "m1_mla_16_heads_b32": (153_500_000, "decode_mla_m1_m2_kernel_stats_and_traffic.md", "869e7ad"),
+    "m2_mla_128_heads_b32": (215_400_000, "decode_mla_m1_m2_kernel_stats_and_traffic.md", "869e7ad"),
+    "c5_prefill_scatter": (32_100_000, "paged_caching_c5_prefill_scatter_kernel_stats_and_traffic.md", "a636ea0"),
+    "k2_append_prefill_chunk": (33_600_000, "kv_caching_k2_append_prefill_chunk_kernel_stats_and_traffic.md", "f6351eb"),
+    "r2_rope_scatter_prefill_chunk": (33_550_000, "rope_paged_caching_r1_r2_kernel_stats_and_traffic.md", "fa02f8a"),
+    "p3_llama3_8b_chunked": (451_500_000, "prefill_tiled_p3_llama3_8b_chunked_counters.md", "a4c5528"),  # fetched only
 }
+
+
+def traffic_fields(workload):
+    """``roofline.traffic`` and where the figure comes from (both None for a workload without a counter run)."""
+    if workload not in MEASURED_TRAFFIC:
+        return {"traffic": None, "traffic_source": None}
+    nbytes, summary, commit = MEASURED_TRAFFIC[workload]
+    return {"traffic": nbytes, "traffic_source": {"profile": "profiles/" + summary, "kernel_commit": commit}}
 
 
 def parse_args():
@@ -171,7 +183,7 @@ def run_prefill(args, torch, L, workloads, dev):
             "peak": MFMA_PEAK_TFLOPS,
             "unit": "TFLOP/s",
             "frac": round(tflops_dev / MFMA_PEAK_TFLOPS, 4),
-            "traffic": MEASURED_TRAFFIC_BYTES.get(cfg.name),
+            **traffic_fields(cfg.name),
             "us_per_call_device": round(us_dev, 2),
             "note": "achieved = flops per call / device time per call (events on the kernel's stream); one kernel per call",
         },
@@ -351,7 +363,7 @@ def run_caching(args, torch, L, workloads, dev):
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": round(algo_bytes / (us_dev * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
-            "traffic": MEASURED_TRAFFIC_BYTES.get(cfg.name),
+            **traffic_fields(cfg.name),
             "us_per_call_device": round(us_dev, 2),
             "note": "achieved = algorithmic bytes / device time per call (events on the kernel's stream, back-to-back "
                     "launches); 32 MB per call is 4 us of traffic at 8 TB/s, the size of a kernel launch",
@@ -520,7 +532,7 @@ def main():
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": round(gbps_dev / HBM_PEAK_GBPS, 4),
-            "traffic": MEASURED_TRAFFIC_BYTES.get(cfg.name),
+            **traffic_fields(cfg.name),
             "us_per_call_device": round(us_dev, 2),
             "note": "achieved = algorithmic bytes / device time per CALL (events on the kernels' stream bracket the "
                     "decode kernel and the small segment-merge kernel that follows it); traffic = HBM bytes of the "

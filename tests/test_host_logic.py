@@ -27,6 +27,24 @@ def test_bench_refuses_to_run_without_a_gpu():
     assert proc.returncode != 0 and proc.stdout.strip() == ""  # no CPU fallback, no JSON line
 
 
+def test_every_recorded_traffic_figure_names_a_workload_and_a_committed_profile_summary():
+    import importlib.util
+
+    spec = importlib.util.spec_from_file_location("bench_module", ROOT / "bench.py")
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    known = (set(workloads.DECODE_CONFIGS) | set(workloads.CACHING_CONFIGS) | set(workloads.KV_CACHING_CONFIGS)
+             | set(workloads.ROPE_CACHING_CONFIGS) | set(workloads.PREFILL_CONFIGS))
+    for name, (nbytes, summary, commit) in bench.MEASURED_TRAFFIC.items():
+        assert name in known
+        assert nbytes > 0 and len(commit) >= 7
+        text = (ROOT / "profiles" / summary).read_text()
+        assert "FETCH_SIZE" in text and "rocprofv3 --pmc" in text
+        fields = bench.traffic_fields(name)
+        assert fields["traffic"] == nbytes and fields["traffic_source"]["profile"] == "profiles/" + summary
+    assert bench.traffic_fields("no_such_workload") == {"traffic": None, "traffic_source": None}
+
+
 @pytest.mark.parametrize("name", sorted(workloads.DECODE_CONFIGS))
 def test_decode_workloads_are_reproducible_and_consistent(name):
     cfg = workloads.DECODE_CONFIGS[name]
