@@ -348,13 +348,17 @@ __device__ __forceinline__ void softmaxStepPair(f32x4 (&o)[COLS], float &m, floa
 struct WidePlan {
     int partition_tokens;
     int seq, part, stream; // this workgroup's unit; seq < 0: none
+    int len;               // length of that sequence, clamped to [0, what its block-table row can hold]
 };
 
 template <typename Tindex>
 __device__ __forceinline__ WidePlan planWide(const DecodeArgs &a, int lane, int streams, int linear_id) {
-    WidePlan plan{a.partition_tokens, -1, 0, 0};
+    WidePlan plan{a.partition_tokens, -1, 0, 0, 0};
     const int64_t max_len = static_cast<int64_t>(a.max_blocks_per_seq) << a.block_shift;
-    int lens[4]; // the lengths once, up to four per lane (one round of independent loads)
+    // Lanes hold up to four lengths each; a batch of at most 64 sequences fills one of the four slots, and
+    // the arithmetic on the empty ones (three quarters of the search below) is skipped: wave-uniform tests.
+    const int slots = (a.num_seqs + 63) >> 6;
+    int lens[4]; // the lengths once (one round of independent loads)
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         int64_t len = 0;
@@ -373,6 +377,9 @@ __device__ __forceinline__ WidePlan planWide(const DecodeArgs &a, int lane, int 
         int x = 0;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
+            if (i >= slots) {
+                break;
+            }
             const float lf = static_cast<float>(lens[i]);
             float q = floorf(lf * inv);
             q = q * pf > lf ? q - 1.0f : q;          // one too many
@@ -398,6 +405,9 @@ __device__ __forceinline__ WidePlan planWide(const DecodeArgs &a, int lane, int 
     int running = 0;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
+        if (i >= slots) {
+            break;
+        }
         const int k = (lens[i] + p - 1) / p;
         const int incl = waveInclusiveSum(k) + running;
         const unsigned long long hit = __builtin_amdgcn_ballot_w64(incl > u);
@@ -405,6 +415,7 @@ __device__ __forceinline__ WidePlan planWide(const DecodeArgs &a, int lane, int 
             const int first = __builtin_ctzll(hit);
             plan.seq = 64 * i + first;
             plan.part = u - (__builtin_amdgcn_readlane(incl, first) - __builtin_amdgcn_readlane(k, first));
+            plan.len = __builtin_amdgcn_readlane(lens[i], first);
         }
         running = __builtin_amdgcn_readlane(incl, 63);
     }
@@ -443,6 +454,7 @@ __global__ void __launch_bounds__(kMlaWideThreads, 2) decodeMlaWideKernel(Decode
     // Which (sequence, partition, KV head x group of four head chunks) this workgroup works on. Everything
     // up to the first barrier depends on the workgroup only, so all wavefronts leave together.
     int seq, part, stream, partition_tokens;
+    int len; // of the sequence, clamped to what its block-table row can hold
     if (a.chosen_partition != nullptr) {
         // planned per call (see planWide): one-dimensional grid
         const WidePlan plan = planWide<Tindex>(a, lane, a.num_kv_heads * groups_of_chunks, static_cast<int>(blockIdx.x));
@@ -457,12 +469,16 @@ __global__ void __launch_bounds__(kMlaWideThreads, 2) decodeMlaWideKernel(Decode
         part = __builtin_amdgcn_readfirstlane(plan.part);
         stream = __builtin_amdgcn_readfirstlane(plan.stream);
         partition_tokens = __builtin_amdgcn_readfirstlane(plan.partition_tokens);
+        len = __builtin_amdgcn_readfirstlane(plan.len); // the plan has read it already: no second round trip
     } else {
         // fixed partitions on a three-dimensional grid, rotated as in decodeMlaKernel
         seq = blockIdx.z;
         part = static_cast<int>((blockIdx.x + blockIdx.z) % gridDim.x);
         stream = blockIdx.y;
         partition_tokens = a.partition_tokens;
+        const int64_t len64 = loadIndex<Tindex>(a.seq_lens, seq);
+        const int64_t max_len = static_cast<int64_t>(a.max_blocks_per_seq) << a.block_shift;
+        len = static_cast<int>(len64 < max_len ? len64 : max_len);
     }
     const int kv_head = stream / groups_of_chunks;
     const int chunk_group = stream - kv_head * groups_of_chunks;
@@ -473,9 +489,6 @@ __global__ void __launch_bounds__(kMlaWideThreads, 2) decodeMlaWideKernel(Decode
     const int own_steps = kOne ? ((wave >> 1) < 2 ? 5 : 4) : kHalfSteps;
     const int th = wave & 1; // CHUNKS = 1: the token half whose scores this wavefront computes
 
-    const int64_t len64 = loadIndex<Tindex>(a.seq_lens, seq);
-    const int64_t max_len = static_cast<int64_t>(a.max_blocks_per_seq) << a.block_shift;
-    const int len = static_cast<int>(len64 < max_len ? len64 : max_len);
     const int start = part * partition_tokens;
     if (len <= 0 || start >= len) {
         return;
