@@ -218,6 +218,31 @@ def test_alibi(gpu_handle, oracle, monkeypatch, dtype, kernel):
     run_case(gpu_handle, oracle, workloads.make_prefill_inputs(cfg), alibi=slopes)
 
 
+@pytest.mark.parametrize("seed", range(16))
+def test_random_shapes_row_blocks_and_dtypes(gpu_handle, oracle, monkeypatch, seed):
+    """Every knob drawn at random from one seed: head size, group size, page size, batch, new-token and history
+    ranges, dtype, index dtype, ALiBi and rows per workgroup."""
+    rng = np.random.default_rng(2000 + seed)
+    D = int(rng.choice([64, 128, 128, 192, 256]))
+    Hkv = int(rng.choice([1, 2, 4]))
+    group = int(rng.choice([1, 2, 3, 4, 7]))
+    bs = int(rng.choice([8, 16, 16, 32, 64]))
+    B = int(rng.choice([1, 3, 9]))
+    new = (1, int(rng.choice([1, 20, 150, 400])))
+    history = (0, int(rng.choice([0, 50, 700])))
+    dtype = [torch.float16, torch.bfloat16][rng.integers(0, 2)]
+    idx = [torch.int64, torch.int32, torch.uint32][rng.integers(0, 3)]
+    groups = ["1", "2"][rng.integers(0, 2)]
+    use_alibi = bool(rng.integers(0, 2))
+    monkeypatch.setenv("INFINIOP_AMD_PREFILL_GROUPS", groups)
+    H = Hkv * group
+    cfg = prefill_config(f"sweep{seed}", dtype, B, H, Hkv, D, bs, new, history, seed=800 + seed)
+    slopes = torch.tensor(rng.uniform(0.001, 0.3, H), dtype=torch.float32) if use_alibi else None
+    print(f"sweep {seed}: D={D} H={H}/{Hkv} bs={bs} B={B} new={new} history={history} {dtype} {idx} rows/wg={groups} "
+          f"alibi={use_alibi}", flush=True)
+    run_case(gpu_handle, oracle, workloads.make_prefill_inputs(cfg), alibi=slopes, index_dtype=idx)
+
+
 # ---- edge cases ---------------------------------------------------------------------------------------------
 
 def test_one_new_token_per_sequence_equals_decode(gpu_handle, oracle):
