@@ -81,4 +81,47 @@ __INFINI_C __export infiniStatus_t infiniopRoPEPagedCaching(
 __INFINI_C __export infiniStatus_t infiniopDestroyRoPEPagedCachingDescriptor(
     infiniopRoPEPagedCachingDescriptor_t desc);
 
+/*
+ * The same with the rotation of the query in the launch as well: the whole producer step in front of a decode
+ * call, which the reference runs as infiniopRoPE on q, infiniopRoPE on k and infiniopPagedCaching.
+ *   q      [num_tokens, num_heads, head_size]  same dtype as k, any token / head strides, last dimension packed
+ *   q_out  [num_tokens, num_heads, head_size]  same dtype; may be q itself (rotation in place)
+ *   q_out[i][h] = rotation of q[i][h] by row pos_ids[i] of the tables, for EVERY token i - also those whose slot is
+ *   negative (padding): only the cache writes are skipped for them.
+ * q, k and v may be slices of one fused projection output (their token strides are taken from the descriptors).
+ * The descriptor is of the same type as above: infiniopGetRoPEPagedCachingWorkspaceSize and
+ * infiniopDestroyRoPEPagedCachingDescriptor serve both; each descriptor is run with the entry point that
+ * matches the way it was created (the other one answers BAD_PARAM).
+ */
+__INFINI_C __export infiniStatus_t infiniopCreateRoPEQKPagedCachingDescriptor(
+    infiniopHandle_t handle,
+    infiniopRoPEPagedCachingDescriptor_t *desc_ptr,
+    infiniopTensorDescriptor_t q_out_desc,
+    infiniopTensorDescriptor_t q_desc,
+    infiniopTensorDescriptor_t k_cache_desc,
+    infiniopTensorDescriptor_t v_cache_desc,
+    infiniopTensorDescriptor_t k_desc,
+    infiniopTensorDescriptor_t v_desc,
+    infiniopTensorDescriptor_t slot_mapping_desc,
+    infiniopTensorDescriptor_t pos_ids_desc,
+    infiniopTensorDescriptor_t sin_table_desc,
+    infiniopTensorDescriptor_t cos_table_desc,
+    infiniopRoPEAlgo_t algo);
+
+__INFINI_C __export infiniStatus_t infiniopRoPEQKPagedCaching(
+    infiniopRoPEPagedCachingDescriptor_t desc,
+    void *workspace,
+    size_t workspace_size,
+    void *q_out,
+    const void *q,
+    void *k_cache,
+    void *v_cache,
+    const void *k,
+    const void *v,
+    const void *slot_mapping,
+    const void *pos_ids,
+    const void *sin_table,
+    const void *cos_table,
+    void *stream);
+
 #endif

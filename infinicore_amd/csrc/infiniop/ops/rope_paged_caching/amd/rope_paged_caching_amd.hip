@@ -47,6 +47,18 @@ struct Args {
     int64_t v_block_stride, v_head_stride, v_slot_stride;
 };
 
+// The query rotated in the same launch: a second argument block, which the kernels without a query do not carry
+// (their argument block is then no longer than the scatter alone needs; a longer one costs them 9 % at 4 096 tokens).
+template <bool QUERY>
+struct QueryArgs {};
+template <>
+struct QueryArgs<true> {
+    void *q_out;
+    const void *q;
+    int32_t num_q_heads;
+    int64_t q_token_stride, q_head_stride, q_out_token_stride, q_out_head_stride;
+};
+
 struct F16 {
     using storage = _Float16;
 };
@@ -87,9 +99,56 @@ struct Unit16 {
     S e[kElements];
 };
 
-// VEC: 16-byte units (see the head of the file); else one pair / one element per step.
-template <typename T, bool VEC>
-__global__ void __launch_bounds__(256) ropeScatterKernel(Args a) {
+// One vector of 2 * table_dim elements rotated from src to dst (dst may be src: a thread reads both halves of its
+// pairs before it writes them). VEC: 16-byte units (see the head of the file); else one pair per step.
+template <typename S, bool VEC>
+__device__ __forceinline__ void rotateRow(const S *src, S *dst, const S *sin_row, const S *cos_row, int table_dim, bool neox,
+                                          int step0, int step) {
+    using U = Unit16<S>;
+    constexpr int kPer = U::kElements;
+    if constexpr (VEC) {
+        // unit u of the rotation covers pairs [u * kPer, (u + 1) * kPer)
+        for (int u = step0; u < table_dim / kPer; u += step) {
+            const int first = neox ? u * kPer : 2 * u * kPer;                 // elements of the first unit
+            const int second = neox ? table_dim + u * kPer : 2 * u * kPer + kPer;
+            const U x_lo = *reinterpret_cast<const U *>(src + first);
+            const U x_hi = *reinterpret_cast<const U *>(src + second);
+            const U sn = *reinterpret_cast<const U *>(sin_row + u * kPer);
+            const U cs = *reinterpret_cast<const U *>(cos_row + u * kPer);
+            U y_lo, y_hi;
+            if (neox) {
+#pragma unroll
+                for (int i = 0; i < kPer; ++i) {
+                    rotatePair(x_lo.e[i], x_hi.e[i], sn.e[i], cs.e[i], y_lo.e[i], y_hi.e[i]);
+                }
+            } else {
+                // the 2 kPer elements are kPer neighbouring pairs: pair i = elements 2 i, 2 i + 1
+#pragma unroll
+                for (int i = 0; i < kPer / 2; ++i) {
+                    rotatePair(x_lo.e[2 * i], x_lo.e[2 * i + 1], sn.e[i], cs.e[i], y_lo.e[2 * i], y_lo.e[2 * i + 1]);
+                    rotatePair(x_hi.e[2 * i], x_hi.e[2 * i + 1], sn.e[kPer / 2 + i], cs.e[kPer / 2 + i], y_hi.e[2 * i],
+                               y_hi.e[2 * i + 1]);
+                }
+            }
+            *reinterpret_cast<U *>(dst + first) = y_lo;
+            *reinterpret_cast<U *>(dst + second) = y_hi;
+        }
+    } else {
+        for (int j = step0; j < table_dim; j += step) {
+            const int first = neox ? j : 2 * j;
+            const int second = neox ? j + table_dim : 2 * j + 1;
+            S y0, y1;
+            rotatePair(src[first], src[second], sin_row[j], cos_row[j], y0, y1);
+            dst[first] = y0;
+            dst[second] = y1;
+        }
+    }
+}
+
+// Thread box: x = steps along a row, y = heads (the KV heads first, then the query heads if the query is rotated
+// too: QUERY), z = tokens.
+template <typename T, bool VEC, bool QUERY>
+__device__ __forceinline__ void ropeScatter(const Args &a, const QueryArgs<QUERY> &qa) {
     using S = typename T::storage;
     using U = Unit16<S>;
     constexpr int kPer = U::kElements;
@@ -97,11 +156,18 @@ __global__ void __launch_bounds__(256) ropeScatterKernel(Args a) {
     if (token >= a.num_tokens) {
         return;
     }
+    // the box once, up front: read inside the loops below, its extents become a memory load per head
+    const int x0 = threadIdx.x, x_step = blockDim.x, y0 = threadIdx.y, y_step = blockDim.y;
     const int64_t slot = a.slot_mapping[token];
     int64_t pos = loadPosition(a, token);
     // Negative = padding (paged_caching kernel.cuh:61-63). Slots past the pool would be an out-of-bounds
-    // write in the reference; here they are dropped.
-    if (slot < 0 || slot >= a.num_slots) {
+    // write in the reference; here they are dropped. The query of such a token is rotated all the same.
+    const bool cached = slot >= 0 && slot < a.num_slots;
+    int num_q_heads = 0;
+    if constexpr (QUERY) {
+        num_q_heads = qa.num_q_heads;
+    }
+    if (!cached && num_q_heads == 0) {
         return;
     }
     pos = pos < 0 ? 0 : (pos >= a.table_len ? a.table_len - 1 : pos);
@@ -117,55 +183,43 @@ __global__ void __launch_bounds__(256) ropeScatterKernel(Args a) {
     const S *sin_row = static_cast<const S *>(a.sin_table) + pos * table_dim;
     const S *cos_row = static_cast<const S *>(a.cos_table) + pos * table_dim;
 
-    for (int head = threadIdx.y; head < a.num_kv_heads; head += blockDim.y) {
+    for (int head = y0; head < a.num_kv_heads + num_q_heads; head += y_step) {
+        if constexpr (QUERY) {
+            if (head >= a.num_kv_heads) {
+                const int64_t q_head = head - a.num_kv_heads;
+                rotateRow<S, VEC>(static_cast<const S *>(qa.q) + token * qa.q_token_stride + q_head * qa.q_head_stride,
+                                  static_cast<S *>(qa.q_out) + token * qa.q_out_token_stride + q_head * qa.q_out_head_stride,
+                                  sin_row, cos_row, table_dim, a.neox != 0, x0, x_step);
+                continue;
+            }
+        }
+        if (QUERY && !cached) {
+            continue;
+        }
         const S *k_src = static_cast<const S *>(a.k) + token * a.k_src_token_stride + static_cast<int64_t>(head) * a.head_size;
         const S *v_src = static_cast<const S *>(a.v) + token * a.v_src_token_stride + static_cast<int64_t>(head) * a.value_size;
         S *k_dst = static_cast<S *>(a.k_cache) + page * a.k_block_stride + head * a.k_head_stride + row * a.k_slot_stride;
         S *v_dst = static_cast<S *>(a.v_cache) + page * a.v_block_stride + head * a.v_head_stride + row * a.v_slot_stride;
+        rotateRow<S, VEC>(k_src, k_dst, sin_row, cos_row, table_dim, a.neox != 0, x0, x_step);
         if constexpr (VEC) {
-            // unit u of the rotation covers pairs [u * kPer, (u + 1) * kPer)
-            for (int u = threadIdx.x; u < table_dim / kPer; u += blockDim.x) {
-                const int first = a.neox ? u * kPer : 2 * u * kPer;                 // elements of the first unit
-                const int second = a.neox ? table_dim + u * kPer : 2 * u * kPer + kPer;
-                const U x_lo = *reinterpret_cast<const U *>(k_src + first);
-                const U x_hi = *reinterpret_cast<const U *>(k_src + second);
-                const U sn = *reinterpret_cast<const U *>(sin_row + u * kPer);
-                const U cs = *reinterpret_cast<const U *>(cos_row + u * kPer);
-                U y_lo, y_hi;
-                if (a.neox) {
-#pragma unroll
-                    for (int i = 0; i < kPer; ++i) {
-                        rotatePair(x_lo.e[i], x_hi.e[i], sn.e[i], cs.e[i], y_lo.e[i], y_hi.e[i]);
-                    }
-                } else {
-                    // the 2 kPer elements are kPer neighbouring pairs: pair i = elements 2 i, 2 i + 1
-#pragma unroll
-                    for (int i = 0; i < kPer / 2; ++i) {
-                        rotatePair(x_lo.e[2 * i], x_lo.e[2 * i + 1], sn.e[i], cs.e[i], y_lo.e[2 * i], y_lo.e[2 * i + 1]);
-                        rotatePair(x_hi.e[2 * i], x_hi.e[2 * i + 1], sn.e[kPer / 2 + i], cs.e[kPer / 2 + i], y_hi.e[2 * i],
-                                   y_hi.e[2 * i + 1]);
-                    }
-                }
-                *reinterpret_cast<U *>(k_dst + first) = y_lo;
-                *reinterpret_cast<U *>(k_dst + second) = y_hi;
-            }
-            for (int u = threadIdx.x; u < a.value_size / kPer; u += blockDim.x) {
+            for (int u = x0; u < a.value_size / kPer; u += x_step) {
                 *reinterpret_cast<U *>(v_dst + u * kPer) = *reinterpret_cast<const U *>(v_src + u * kPer);
             }
         } else {
-            for (int j = threadIdx.x; j < table_dim; j += blockDim.x) {
-                const int first = a.neox ? j : 2 * j;
-                const int second = a.neox ? j + table_dim : 2 * j + 1;
-                S y0, y1;
-                rotatePair(k_src[first], k_src[second], sin_row[j], cos_row[j], y0, y1);
-                k_dst[first] = y0;
-                k_dst[second] = y1;
-            }
-            for (int j = threadIdx.x; j < a.value_size; j += blockDim.x) {
+            for (int j = x0; j < a.value_size; j += x_step) {
                 v_dst[j] = v_src[j];
             }
         }
     }
+}
+
+template <typename T, bool VEC>
+__global__ void __launch_bounds__(256) ropeScatterKernel(Args a) {
+    ropeScatter<T, VEC, false>(a, QueryArgs<false>{});
+}
+template <typename T, bool VEC>
+__global__ void __launch_bounds__(256) ropeScatterQueryKernel(Args a, QueryArgs<true> qa) {
+    ropeScatter<T, VEC, true>(a, qa);
 }
 
 int ceilPow2(int x) {
@@ -179,16 +233,22 @@ int ceilPow2(int x) {
 bool multipleOf16(uint64_t x) { return (x & 15u) == 0; }
 
 template <typename T>
-void launch(const Args &a, bool vec, int row_steps, hipStream_t stream) {
+void launch(const Args &a, const QueryArgs<true> &qa, bool vec, int row_steps, hipStream_t stream) {
     // 256-thread box: x = steps along a row, y = heads, z = tokens
     int bx = ceilPow2(row_steps);
     bx = bx > 64 ? 64 : bx;
-    int by = ceilPow2(a.num_kv_heads);
+    int by = ceilPow2(a.num_kv_heads + qa.num_q_heads);
     by = by > 256 / bx ? 256 / bx : by;
     const int bz = 256 / (bx * by);
     const dim3 block(bx, by, bz);
     const dim3 grid(static_cast<unsigned>((a.num_tokens + bz - 1) / bz));
-    if (vec) {
+    if (qa.num_q_heads > 0) {
+        if (vec) {
+            ropeScatterQueryKernel<T, true><<<grid, block, 0, stream>>>(a, qa);
+        } else {
+            ropeScatterQueryKernel<T, false><<<grid, block, 0, stream>>>(a, qa);
+        }
+    } else if (vec) {
         ropeScatterKernel<T, true><<<grid, block, 0, stream>>>(a);
     } else {
         ropeScatterKernel<T, false><<<grid, block, 0, stream>>>(a);
@@ -205,22 +265,31 @@ infiniStatus_t Descriptor::create(infiniopHandle_t handle, Descriptor **desc_ptr
                                   infiniopTensorDescriptor_t v_cache_desc, infiniopTensorDescriptor_t k_desc,
                                   infiniopTensorDescriptor_t v_desc, infiniopTensorDescriptor_t slot_mapping_desc,
                                   infiniopTensorDescriptor_t pos_ids_desc, infiniopTensorDescriptor_t sin_table_desc,
-                                  infiniopTensorDescriptor_t cos_table_desc, infiniopRoPEAlgo_t algo) {
+                                  infiniopTensorDescriptor_t cos_table_desc, infiniopRoPEAlgo_t algo, bool with_query,
+                                  infiniopTensorDescriptor_t q_out_desc, infiniopTensorDescriptor_t q_desc) {
     auto info = RoPEPagedCachingInfo::create(k_cache_desc, v_cache_desc, k_desc, v_desc, slot_mapping_desc, pos_ids_desc,
-                                             sin_table_desc, cos_table_desc, algo);
+                                             sin_table_desc, cos_table_desc, algo, with_query, q_out_desc, q_desc);
     CHECK_RESULT(info);
     *desc_ptr = new Descriptor(new Opaque{}, info.take(), 0, handle->device, handle->device_id);
     return INFINI_STATUS_SUCCESS;
 }
 
-infiniStatus_t Descriptor::calculate(void *workspace, size_t workspace_size, void *k_cache, void *v_cache, const void *k,
-                                     const void *v, const void *slot_mapping, const void *pos_ids, const void *sin_table,
-                                     const void *cos_table, void *stream_) const {
+infiniStatus_t Descriptor::calculate(void *workspace, size_t workspace_size, void *q_out, const void *q, void *k_cache,
+                                     void *v_cache, const void *k, const void *v, const void *slot_mapping,
+                                     const void *pos_ids, const void *sin_table, const void *cos_table, void *stream_) const {
     (void)workspace;
     (void)workspace_size;
     const auto &in = _info.scatter;
-    if (in.num_tokens == 0 || in.num_kv_heads == 0 || (in.head_size == 0 && in.v_head_size == 0)) {
+    const bool rotates_query = _info.has_query && _info.num_q_heads > 0 && in.head_size > 0;
+    const bool caches = in.num_kv_heads > 0 && (in.head_size > 0 || in.v_head_size > 0);
+    if (in.num_tokens == 0 || (!caches && !rotates_query)) {
         return INFINI_STATUS_SUCCESS;
+    }
+    if (rotates_query && (q_out == nullptr || q == nullptr)) {
+        return INFINI_STATUS_NULL_POINTER;
+    }
+    if (in.num_kv_heads + (rotates_query ? _info.num_q_heads : 0) > 0x7fffffff) {
+        return INFINI_STATUS_BAD_TENSOR_SHAPE;
     }
     if (k_cache == nullptr || v_cache == nullptr || k == nullptr || v == nullptr || slot_mapping == nullptr
         || pos_ids == nullptr || sin_table == nullptr || cos_table == nullptr) {
@@ -243,6 +312,14 @@ infiniStatus_t Descriptor::calculate(void *workspace, size_t workspace_size, voi
     a.pos_ids = pos_ids;
     a.sin_table = sin_table;
     a.cos_table = cos_table;
+    QueryArgs<true> qa{};
+    qa.q_out = q_out;
+    qa.q = q;
+    qa.num_q_heads = rotates_query ? static_cast<int32_t>(_info.num_q_heads) : 0;
+    qa.q_token_stride = _info.q_token_stride;
+    qa.q_head_stride = _info.q_head_stride;
+    qa.q_out_token_stride = _info.q_out_token_stride;
+    qa.q_out_head_stride = _info.q_out_head_stride;
     a.num_tokens = static_cast<int64_t>(in.num_tokens);
     a.num_slots = static_cast<int64_t>(in.num_blocks) * static_cast<int64_t>(in.block_size);
     a.table_len = static_cast<int64_t>(_info.table_len);
@@ -284,14 +361,21 @@ infiniStatus_t Descriptor::calculate(void *workspace, size_t workspace_size, voi
                               bytes(static_cast<ptrdiff_t>(_info.table_dim))}) {
         vec = vec && multipleOf16(quantity);
     }
+    if (rotates_query) {
+        for (uint64_t quantity : {bytes(_info.q_token_stride), bytes(_info.q_head_stride), bytes(_info.q_out_token_stride),
+                                  bytes(_info.q_out_head_stride), static_cast<uint64_t>(reinterpret_cast<uintptr_t>(q)),
+                                  static_cast<uint64_t>(reinterpret_cast<uintptr_t>(q_out))}) {
+            vec = vec && multipleOf16(quantity);
+        }
+    }
     const int rotate_steps = static_cast<int>(vec ? _info.table_dim / per : _info.table_dim);
     const int copy_steps = static_cast<int>(vec ? in.v_head_size / per : in.v_head_size);
     const int row_steps = rotate_steps > copy_steps ? rotate_steps : copy_steps;
     auto stream = static_cast<hipStream_t>(stream_);
     switch (in.dtype) {
-    case INFINI_DTYPE_F16: launch<F16>(a, vec, row_steps > 0 ? row_steps : 1, stream); break;
-    case INFINI_DTYPE_BF16: launch<BF16>(a, vec, row_steps > 0 ? row_steps : 1, stream); break;
-    case INFINI_DTYPE_F32: launch<F32>(a, vec, row_steps > 0 ? row_steps : 1, stream); break;
+    case INFINI_DTYPE_F16: launch<F16>(a, qa, vec, row_steps > 0 ? row_steps : 1, stream); break;
+    case INFINI_DTYPE_BF16: launch<BF16>(a, qa, vec, row_steps > 0 ? row_steps : 1, stream); break;
+    case INFINI_DTYPE_F32: launch<F32>(a, qa, vec, row_steps > 0 ? row_steps : 1, stream); break;
     default: return INFINI_STATUS_BAD_TENSOR_DTYPE;
     }
     return hipGetLastError() == hipSuccess ? INFINI_STATUS_SUCCESS : INFINI_STATUS_INTERNAL_ERROR;

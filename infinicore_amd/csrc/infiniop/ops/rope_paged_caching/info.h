@@ -16,6 +16,10 @@ struct RoPEPagedCachingInfo {
     size_t table_len;        // rows of the sin / cos tables
     size_t table_dim;        // head_size / 2
     infiniopRoPEAlgo_t algo;
+    // query rotated in the same launch (infiniopCreateRoPEQKPagedCachingDescriptor); else has_query is false
+    bool has_query;
+    size_t num_q_heads;
+    ptrdiff_t q_token_stride, q_head_stride, q_out_token_stride, q_out_head_stride;
 
     static bool isInteger(infiniDtype_t dt) {
         switch (dt) {
@@ -33,7 +37,10 @@ struct RoPEPagedCachingInfo {
                                                       infiniopTensorDescriptor_t slot_mapping_desc,
                                                       infiniopTensorDescriptor_t pos_desc,
                                                       infiniopTensorDescriptor_t sin_desc,
-                                                      infiniopTensorDescriptor_t cos_desc, infiniopRoPEAlgo_t algo) {
+                                                      infiniopTensorDescriptor_t cos_desc, infiniopRoPEAlgo_t algo,
+                                                      bool with_query = false,
+                                                      infiniopTensorDescriptor_t q_out_desc = nullptr,
+                                                      infiniopTensorDescriptor_t q_desc = nullptr) {
         // rope.h:79-82
         if (!pos_desc || !sin_desc || !cos_desc || static_cast<int>(algo) < 0 || algo >= INFINIOP_ROPE_ALGO_COUNT) {
             return INFINI_STATUS_NULL_POINTER;
@@ -70,6 +77,30 @@ struct RoPEPagedCachingInfo {
         }
         if (!sin_desc->isContiguous() || !cos_desc->isContiguous()) {
             return INFINI_STATUS_BAD_TENSOR_STRIDES;
+        }
+        info.has_query = with_query;
+        if (with_query) {
+            // the checks of the reference's RoPE for its x / y pair (rope.h:79-160): both given, dtype of the
+            // tables, [tokens, heads, head_size] with the tokens and head size of k, packed last dimension
+            if (!q_out_desc || !q_desc) {
+                return INFINI_STATUS_NULL_POINTER;
+            }
+            if (q_desc->dtype() != info.scatter.dtype || q_out_desc->dtype() != info.scatter.dtype) {
+                return INFINI_STATUS_BAD_TENSOR_DTYPE;
+            }
+            if (q_desc->ndim() != 3 || q_out_desc->ndim() != 3 || q_desc->dim(0) != info.scatter.num_tokens
+                || q_desc->dim(2) != info.scatter.head_size || q_out_desc->dim(0) != q_desc->dim(0)
+                || q_out_desc->dim(1) != q_desc->dim(1) || q_out_desc->dim(2) != q_desc->dim(2)) {
+                return INFINI_STATUS_BAD_TENSOR_SHAPE;
+            }
+            if (q_desc->stride(2) != 1 || q_out_desc->stride(2) != 1) {
+                return INFINI_STATUS_BAD_TENSOR_STRIDES;
+            }
+            info.num_q_heads = q_desc->dim(1);
+            info.q_token_stride = q_desc->stride(0);
+            info.q_head_stride = q_desc->stride(1);
+            info.q_out_token_stride = q_out_desc->stride(0);
+            info.q_out_head_stride = q_out_desc->stride(1);
         }
         return info;
     }

@@ -20,7 +20,27 @@ __INFINI_C infiniStatus_t infiniopCreateRoPEPagedCachingDescriptor(
     switch (handle->device) {
     case INFINI_DEVICE_AMD:
         return AmdDescriptor::create(handle, reinterpret_cast<AmdDescriptor **>(desc_ptr), k_cache_desc, v_cache_desc,
-                                     k_desc, v_desc, slot_mapping_desc, pos_ids_desc, sin_table_desc, cos_table_desc, algo);
+                                     k_desc, v_desc, slot_mapping_desc, pos_ids_desc, sin_table_desc, cos_table_desc, algo,
+                                     false, nullptr, nullptr);
+    default:
+        return INFINI_STATUS_DEVICE_TYPE_NOT_SUPPORTED;
+    }
+}
+
+__INFINI_C infiniStatus_t infiniopCreateRoPEQKPagedCachingDescriptor(
+    infiniopHandle_t handle, infiniopRoPEPagedCachingDescriptor_t *desc_ptr, infiniopTensorDescriptor_t q_out_desc,
+    infiniopTensorDescriptor_t q_desc, infiniopTensorDescriptor_t k_cache_desc, infiniopTensorDescriptor_t v_cache_desc,
+    infiniopTensorDescriptor_t k_desc, infiniopTensorDescriptor_t v_desc, infiniopTensorDescriptor_t slot_mapping_desc,
+    infiniopTensorDescriptor_t pos_ids_desc, infiniopTensorDescriptor_t sin_table_desc,
+    infiniopTensorDescriptor_t cos_table_desc, infiniopRoPEAlgo_t algo) {
+    if (handle == nullptr || desc_ptr == nullptr) {
+        return INFINI_STATUS_NULL_POINTER;
+    }
+    switch (handle->device) {
+    case INFINI_DEVICE_AMD:
+        return AmdDescriptor::create(handle, reinterpret_cast<AmdDescriptor **>(desc_ptr), k_cache_desc, v_cache_desc,
+                                     k_desc, v_desc, slot_mapping_desc, pos_ids_desc, sin_table_desc, cos_table_desc, algo,
+                                     true, q_out_desc, q_desc);
     default:
         return INFINI_STATUS_DEVICE_TYPE_NOT_SUPPORTED;
     }
@@ -48,8 +68,32 @@ __INFINI_C infiniStatus_t infiniopRoPEPagedCaching(infiniopRoPEPagedCachingDescr
     }
     switch (desc->device_type) {
     case INFINI_DEVICE_AMD:
-        return reinterpret_cast<AmdDescriptor *>(desc)->calculate(workspace, workspace_size, k_cache, v_cache, k, v,
-                                                                  slot_mapping, pos_ids, sin_table, cos_table, stream);
+        if (reinterpret_cast<AmdDescriptor *>(desc)->hasQuery()) {
+            return INFINI_STATUS_BAD_PARAM; // created with a query: run it with infiniopRoPEQKPagedCaching
+        }
+        return reinterpret_cast<AmdDescriptor *>(desc)->calculate(workspace, workspace_size, nullptr, nullptr, k_cache,
+                                                                  v_cache, k, v, slot_mapping, pos_ids, sin_table,
+                                                                  cos_table, stream);
+    default:
+        return INFINI_STATUS_DEVICE_TYPE_NOT_SUPPORTED;
+    }
+}
+
+__INFINI_C infiniStatus_t infiniopRoPEQKPagedCaching(infiniopRoPEPagedCachingDescriptor_t desc, void *workspace,
+                                                     size_t workspace_size, void *q_out, const void *q, void *k_cache,
+                                                     void *v_cache, const void *k, const void *v, const void *slot_mapping,
+                                                     const void *pos_ids, const void *sin_table, const void *cos_table,
+                                                     void *stream) {
+    if (desc == nullptr) {
+        return INFINI_STATUS_NULL_POINTER;
+    }
+    switch (desc->device_type) {
+    case INFINI_DEVICE_AMD:
+        if (!reinterpret_cast<AmdDescriptor *>(desc)->hasQuery()) {
+            return INFINI_STATUS_BAD_PARAM; // created without a query: run it with infiniopRoPEPagedCaching
+        }
+        return reinterpret_cast<AmdDescriptor *>(desc)->calculate(workspace, workspace_size, q_out, q, k_cache, v_cache, k,
+                                                                  v, slot_mapping, pos_ids, sin_table, cos_table, stream);
     default:
         return INFINI_STATUS_DEVICE_TYPE_NOT_SUPPORTED;
     }

@@ -30,8 +30,13 @@
                                      infiniopTensorDescriptor_t slot_mapping_desc,                              \
                                      infiniopTensorDescriptor_t pos_ids_desc,                                   \
                                      infiniopTensorDescriptor_t sin_table_desc,                                 \
-                                     infiniopTensorDescriptor_t cos_table_desc, infiniopRoPEAlgo_t algo);       \
-        infiniStatus_t calculate(void *workspace, size_t workspace_size, void *k_cache, void *v_cache,          \
+                                     infiniopTensorDescriptor_t cos_table_desc, infiniopRoPEAlgo_t algo,        \
+                                     bool with_query, infiniopTensorDescriptor_t q_out_desc,                    \
+                                     infiniopTensorDescriptor_t q_desc);                                        \
+        bool hasQuery() const { return _info.has_query; }                                                       \
+        /* q_out / q: used by descriptors created with a query only */                                          \
+        infiniStatus_t calculate(void *workspace, size_t workspace_size, void *q_out, const void *q,            \
+                                 void *k_cache, void *v_cache,                                                  \
                                  const void *k, const void *v, const void *slot_mapping, const void *pos_ids,   \
                                  const void *sin_table, const void *cos_table, void *stream) const;             \
     };                                                                                                          \

@@ -177,6 +177,8 @@ def _open():
     _declare(op, "infiniopGetRoPEPagedCachingWorkspaceSize", [D, POINTER(c_size_t)])
     _declare(op, "infiniopRoPEPagedCaching", [D, vp, c_size_t, vp, vp, vp, vp, vp, vp, vp, vp, vp])
     _declare(op, "infiniopDestroyRoPEPagedCachingDescriptor", [D])
+    _declare(op, "infiniopCreateRoPEQKPagedCachingDescriptor", [infiniopHandle_t, POINTER(D)] + [T] * 10 + [c_int])
+    _declare(op, "infiniopRoPEQKPagedCaching", [D, vp, c_size_t] + [vp] * 11)
     _declare(op, "infiniopCreateKVCachingDescriptor", [infiniopHandle_t, POINTER(D), T, T, T, T, T])
     _declare(op, "infiniopGetKVCachingWorkspaceSize", [D, POINTER(c_size_t)])
     _declare(op, "infiniopKVCaching", [D, vp, c_size_t, vp, vp, vp, vp, vp, vp])

@@ -238,11 +238,17 @@ def paged_caching(k_cache, v_cache, k, v, slot_mapping):
     return k_cache, v_cache
 
 
-def rope_paged_caching(k_cache, v_cache, k, v, slot_mapping, pos_ids, sin_table, cos_table, algo: int = lib.RoPEAlgo.GPT_NEOX):
+def rope_paged_caching(k_cache, v_cache, k, v, slot_mapping, pos_ids, sin_table, cos_table,
+                       algo: int = lib.RoPEAlgo.GPT_NEOX, *, q=None, q_out=None):
     """Rotate ``k`` [num_tokens, num_kv_heads, head_size] by the rows ``pos_ids`` of the sin / cos tables
     [table_len, head_size / 2] and scatter it, and ``v`` unchanged, into their slots of the paged pools, in one
     launch; returns the pools. The result of the reference's ``rope`` followed by ``paged_caching``
-    (python/infinicore/ops/paged_caching.py:5-15 for the scatter's argument order)."""
+    (python/infinicore/ops/paged_caching.py:5-15 for the scatter's argument order). With ``q``
+    [num_tokens, num_heads, head_size] the query is rotated in the same launch, into ``q_out`` (default: in
+    place), and the call returns ``(k_cache, v_cache, q_out)``."""
+    if q is not None:
+        return _rope_qk_paged_caching(q if q_out is None else q_out, q, k_cache, v_cache, k, v, slot_mapping, pos_ids,
+                                      sin_table, cos_table, algo)
     index = _device_index(k)
     tensors = (k_cache, v_cache, k, v, slot_mapping, pos_ids, sin_table, cos_table)
     key = ("rope_paged_caching", index, _stream_key(index), int(algo), *(_meta(t) for t in tensors))
@@ -273,6 +279,38 @@ def rope_paged_caching(k_cache, v_cache, k, v, slot_mapping, pos_ids, sin_table,
         "infiniopRoPEPagedCaching",
     )
     return k_cache, v_cache
+
+
+def _rope_qk_paged_caching(q_out, q, k_cache, v_cache, k, v, slot_mapping, pos_ids, sin_table, cos_table, algo):
+    index = _device_index(k)
+    tensors = (q_out, q, k_cache, v_cache, k, v, slot_mapping, pos_ids, sin_table, cos_table)
+    key = ("rope_qk_paged_caching", index, _stream_key(index), int(algo), *(_meta(t) for t in tensors))
+
+    def make():
+        handle = _handle_for(index)
+        descs = [_describe(t) for t in tensors]
+        op = lib.infiniopOperatorDescriptor_t()
+        try:
+            check_error(
+                LIBINFINIOP.infiniopCreateRoPEQKPagedCachingDescriptor(handle, ctypes.byref(op), *descs, int(algo)),
+                "infiniopCreateRoPEQKPagedCachingDescriptor",
+            )
+        finally:
+            for d in descs:
+                lib.destroy_tensor_descriptor(d)
+        size = c_size_t(0)
+        check_error(LIBINFINIOP.infiniopGetRoPEPagedCachingWorkspaceSize(op, ctypes.byref(size)))
+        return _Plan(op, LIBINFINIOP.infiniopDestroyRoPEPagedCachingDescriptor, size.value, k.device)
+
+    plan = _cached_plan(key, make)
+    lib.set_device(InfiniDevice.AMD, index)
+    check_error(
+        LIBINFINIOP.infiniopRoPEQKPagedCaching(
+            plan.descriptor, _ptr(plan.workspace), plan.workspace_bytes, *(_ptr(t) for t in tensors), _stream_ptr(index),
+        ),
+        "infiniopRoPEQKPagedCaching",
+    )
+    return k_cache, v_cache, q_out
 
 
 def kv_caching(k_cache, v_cache, k, v, past_kv_lengths):

@@ -99,7 +99,11 @@ ROPE_CACHING_TABLE_LEN = 8192
 ROPE_CACHING_CONFIGS = {
     "r1_rope_scatter_decode_step": CachingConfig("r1_rope_scatter_decode_step", torch.bfloat16, 32, 8, 128, 16, 65536, 0.0, seed=401),
     "r2_rope_scatter_prefill_chunk": CachingConfig("r2_rope_scatter_prefill_chunk", torch.bfloat16, 4096, 8, 128, 16, 65536, 0.05, seed=402),
+    # the same two steps with the query (32 heads) rotated in the launch as well
+    "r3_rope_qk_scatter_decode_step": CachingConfig("r3_rope_qk_scatter_decode_step", torch.bfloat16, 32, 8, 128, 16, 65536, 0.0, seed=403),
+    "r4_rope_qk_scatter_prefill_chunk": CachingConfig("r4_rope_qk_scatter_prefill_chunk", torch.bfloat16, 4096, 8, 128, 16, 65536, 0.05, seed=404),
 }
+ROPE_QUERY_HEADS = {"r3_rope_qk_scatter_decode_step": 32, "r4_rope_qk_scatter_prefill_chunk": 32}
 
 
 @dataclass
@@ -302,9 +306,18 @@ def make_rope_caching_inputs(cfg: CachingConfig):
 
 
 def rope_caching_algorithmic_bytes(cfg: CachingConfig, slot_mapping) -> int:
-    """The scatter's bytes plus one position and one row of each table per token."""
+    """The scatter's bytes plus one position and one row of each table per token, plus the query read once and
+    written once where the workload rotates it too."""
     e = 2 if cfg.dtype in (torch.float16, torch.bfloat16) else 4
-    return caching_algorithmic_bytes(cfg, slot_mapping) + cfg.num_tokens * (8 + 2 * (cfg.head_size // 2) * e)
+    query = 2 * cfg.num_tokens * ROPE_QUERY_HEADS.get(cfg.name, 0) * cfg.head_size * e
+    return caching_algorithmic_bytes(cfg, slot_mapping) + cfg.num_tokens * (8 + 2 * (cfg.head_size // 2) * e) + query
+
+
+def make_rope_query(cfg: CachingConfig):
+    """The query of a workload that rotates it: [num_tokens, ROPE_QUERY_HEADS, head_size]."""
+    rng = np.random.default_rng([cfg.seed, 17])
+    shape = (cfg.num_tokens, ROPE_QUERY_HEADS[cfg.name], cfg.head_size)
+    return torch.from_numpy(rng.standard_normal(shape, dtype=np.float32)).to(cfg.dtype)
 
 
 @dataclass

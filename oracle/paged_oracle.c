@@ -30,6 +30,7 @@
  *                                  y0 = x0 cos - x1 sin, y1 = x0 sin + x1 cos in fp32, every product and sum
  *                                  rounded on its own, one rounding to the storage dtype) followed by the slot
  *                                  scatter of oracle_paged_caching, without the tensor in between
+ *   oracle_rope                    the same rotation on its own, [tokens, heads, d] -> [tokens, heads, d]
  *   oracle_kv_caching              src/infiniop/ops/kv_caching/cuda/kernel.cuh:32-58
  *                                  (element (b, h, s, d) of the new tensors goes to cache position
  *                                  past_kv_lengths[b] + s; every dimension of every tensor strided)
@@ -414,6 +415,60 @@ int oracle_paged_caching(void *k_cache_, void *v_cache_, const void *k_, const v
     return 0;
 }
 
+/* One vector of 2 * half elements rotated by row `pos` of the tables (rope_cpu.cc:71-84): pair j is elements
+ * (2j, 2j + 1), or (j, j + half) for neox; four products and two sums, each rounded to fp32 on its own (no fused
+ * multiply-add), one rounding to the storage dtype. dst may be src. */
+static void rope_vector(char *dst, const char *src, const char *sin_table, const char *cos_table, int64_t pos,
+                        int64_t half, int dtype, int neox) {
+    for (int64_t j = 0; j < half; ++j) {
+        const int64_t p0 = neox ? j : 2 * j, p1 = neox ? j + half : 2 * j + 1;
+        float x0, x1, sn, cs;
+        if (dtype == 2) {
+            memcpy(&x0, src + p0 * 4, 4);
+            memcpy(&x1, src + p1 * 4, 4);
+            memcpy(&sn, sin_table + (pos * half + j) * 4, 4);
+            memcpy(&cs, cos_table + (pos * half + j) * 4, 4);
+        } else {
+            x0 = load_elem((const uint16_t *)(src + p0 * 2), dtype);
+            x1 = load_elem((const uint16_t *)(src + p1 * 2), dtype);
+            sn = load_elem((const uint16_t *)(sin_table + (pos * half + j) * 2), dtype);
+            cs = load_elem((const uint16_t *)(cos_table + (pos * half + j) * 2), dtype);
+        }
+        volatile float x0c = x0 * cs, x1s = x1 * sn, x0s = x0 * sn, x1c = x1 * cs;
+        const float y0 = x0c - x1s, y1 = x0s + x1c;
+        if (dtype == 2) {
+            memcpy(dst + p0 * 4, &y0, 4);
+            memcpy(dst + p1 * 4, &y1, 4);
+        } else {
+            const uint16_t b0 = store_elem(y0, dtype), b1 = store_elem(y1, dtype);
+            memcpy(dst + p0 * 2, &b0, 2);
+            memcpy(dst + p1 * 2, &b1, 2);
+        }
+    }
+}
+
+/* Rotary embedding of x [num_tokens, num_heads, head_size] into y (same shape; y may be x), one position per
+ * token: the reference's RoPE on its own (rope_cpu.cc:56-98), which the fused operator applies to the query.
+ * Strides in elements; the last dimension is packed. Positions outside the tables use the nearest row. */
+int oracle_rope(void *y_, const void *x_, const int64_t *pos_ids, const void *sin_table_, const void *cos_table_,
+                int64_t table_len, int dtype, int neox, int64_t num_tokens, int64_t num_heads, int64_t head_size,
+                int64_t x_token_stride, int64_t x_head_stride, int64_t y_token_stride, int64_t y_head_stride) {
+    const int64_t es = dtype == 2 ? 4 : 2;
+    if ((head_size & 1) || table_len <= 0 || dtype < 0 || dtype > 2) {
+        return -1;
+    }
+    for (int64_t tok = 0; tok < num_tokens; ++tok) {
+        int64_t pos = pos_ids[tok];
+        pos = pos < 0 ? 0 : (pos >= table_len ? table_len - 1 : pos);
+        for (int64_t head = 0; head < num_heads; ++head) {
+            rope_vector((char *)y_ + (tok * y_token_stride + head * y_head_stride) * es,
+                        (const char *)x_ + (tok * x_token_stride + head * x_head_stride) * es,
+                        (const char *)sin_table_, (const char *)cos_table_, pos, head_size / 2, dtype, neox);
+        }
+    }
+    return 0;
+}
+
 /* Rotary embedding of K (rope_cpu.cc:56-98, one position per token) fused with the slot scatter above.
  * dtype: ORACLE_DTYPE_F16 / BF16, or 2 for fp32. neox: pairs half a vector apart, else neighbouring. A position
  * outside the tables uses the nearest row (the reference reads out of bounds); returns -1 for arguments it
@@ -442,32 +497,7 @@ int oracle_rope_paged_caching(void *k_cache_, void *v_cache_, const void *k_, co
             const char *v_src = v + (tok * s->v_src_stride + head * s->v_head_size) * es;
             char *k_dst = k_cache + (page * s->k_cache_block_stride + head * s->k_cache_head_stride + row * s->k_cache_slot_stride) * es;
             char *v_dst = v_cache + (page * s->v_cache_block_stride + head * s->v_cache_head_stride + row * s->v_cache_slot_stride) * es;
-            for (int64_t j = 0; j < half; ++j) {
-                const int64_t p0 = neox ? j : 2 * j, p1 = neox ? j + half : 2 * j + 1;
-                float x0, x1, sn, cs;
-                if (dtype == 2) {
-                    memcpy(&x0, k_src + p0 * 4, 4);
-                    memcpy(&x1, k_src + p1 * 4, 4);
-                    memcpy(&sn, sin_table + (pos * half + j) * 4, 4);
-                    memcpy(&cs, cos_table + (pos * half + j) * 4, 4);
-                } else {
-                    x0 = load_elem((const uint16_t *)(k_src + p0 * 2), dtype);
-                    x1 = load_elem((const uint16_t *)(k_src + p1 * 2), dtype);
-                    sn = load_elem((const uint16_t *)(sin_table + (pos * half + j) * 2), dtype);
-                    cs = load_elem((const uint16_t *)(cos_table + (pos * half + j) * 2), dtype);
-                }
-                /* four products and two sums, each rounded to fp32 (no fused multiply-add) */
-                volatile float x0c = x0 * cs, x1s = x1 * sn, x0s = x0 * sn, x1c = x1 * cs;
-                const float y0 = x0c - x1s, y1 = x0s + x1c;
-                if (dtype == 2) {
-                    memcpy(k_dst + p0 * 4, &y0, 4);
-                    memcpy(k_dst + p1 * 4, &y1, 4);
-                } else {
-                    const uint16_t b0 = store_elem(y0, dtype), b1 = store_elem(y1, dtype);
-                    memcpy(k_dst + p0 * 2, &b0, 2);
-                    memcpy(k_dst + p1 * 2, &b1, 2);
-                }
-            }
+            rope_vector(k_dst, k_src, sin_table, cos_table, pos, half, dtype, neox);
             memcpy(v_dst, v_src, (size_t)(s->v_head_size * es));
         }
     }

@@ -83,6 +83,8 @@ def load():
         lib.oracle_rope_paged_caching.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                                   c_void_p, c_int64, c_int, c_int, POINTER(CachingShape)]
         lib.oracle_rope_paged_caching.restype = c_int
+        lib.oracle_rope.argtypes = [c_void_p] * 5 + [c_int64, c_int, c_int] + [c_int64] * 7
+        lib.oracle_rope.restype = c_int
         lib.oracle_kv_caching.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, POINTER(KVCachingShape)]
         lib.oracle_kv_caching.restype = c_int
         lib.oracle_to_float.argtypes = [ctypes.c_uint16, c_int]
@@ -213,6 +215,25 @@ def rope_paged_caching(k_cache, v_cache, k, v, slot_mapping, pos_ids, sin_table,
     if rc != 0:
         raise ValueError("oracle rejected the arguments")
     return k_cache, v_cache
+
+
+def rope(x, pos_ids, sin_table, cos_table, neox: bool, out=None):
+    """C oracle rotary embedding of ``x`` [tokens, heads, d] (any token / head strides, packed last dimension), one
+    position per token; returns the rotated tensor (``out``, which may be ``x``, or a new packed tensor)."""
+    lib = load()
+    x = _cpu(x)
+    if out is None:
+        out = torch.empty(x.shape, dtype=x.dtype)
+    pos_ids = _cpu(pos_ids).to(torch.int64).contiguous()
+    sin_table, cos_table = _cpu(sin_table).contiguous(), _cpu(cos_table).contiguous()
+    assert x.stride(-1) == 1 and out.stride(-1) == 1 and out.shape == x.shape
+    code = {torch.float16: 0, torch.bfloat16: 1, torch.float32: 2}[x.dtype]
+    rc = lib.oracle_rope(out.data_ptr(), x.data_ptr(), pos_ids.data_ptr(), sin_table.data_ptr(), cos_table.data_ptr(),
+                         sin_table.shape[0], code, int(bool(neox)), x.shape[0], x.shape[1], x.shape[2],
+                         x.stride(0), x.stride(1), out.stride(0), out.stride(1))
+    if rc != 0:
+        raise ValueError("oracle rejected the arguments")
+    return out
 
 
 def torch_reference_rope(x, pos_ids, sin_table, cos_table, neox: bool):

@@ -168,6 +168,36 @@ def run_rope_paged_caching(handle, k_cache, v_cache, k, v, slot_mapping, pos_ids
     return k_cache, v_cache
 
 
+def create_rope_qk_paged_caching(handle, q_out, q, k_cache, v_cache, k, v, slot_mapping, pos_ids, sin_table, cos_table, algo):
+    descs = [describe(t) for t in (q_out, q, k_cache, v_cache, k, v, slot_mapping, pos_ids, sin_table, cos_table)]
+    op = L.infiniopOperatorDescriptor_t()
+    status = L.LIBINFINIOP.infiniopCreateRoPEQKPagedCachingDescriptor(handle, ctypes.byref(op), *descs, int(algo))
+    for d in descs:
+        L.destroy_tensor_descriptor(d)
+    return status, op
+
+
+def run_rope_qk_paged_caching(handle, q_out, q, k_cache, v_cache, k, v, slot_mapping, pos_ids, sin_table, cos_table, algo,
+                              stream=None):
+    """In place on the device pools and q_out; returns (k_cache, v_cache, q_out)."""
+    status, op = create_rope_qk_paged_caching(handle, q_out, q, k_cache, v_cache, k, v, slot_mapping, pos_ids, sin_table,
+                                              cos_table, algo)
+    L.check_error(status, "infiniopCreateRoPEQKPagedCachingDescriptor")
+    size = c_size_t(123)
+    L.check_error(L.LIBINFINIOP.infiniopGetRoPEPagedCachingWorkspaceSize(op, ctypes.byref(size)))
+    assert size.value == 0
+    torch.cuda.synchronize()
+    L.check_error(
+        L.LIBINFINIOP.infiniopRoPEQKPagedCaching(op, c_void_p(0), 0, ptr(q_out), ptr(q), ptr(k_cache), ptr(v_cache), ptr(k),
+                                                 ptr(v), ptr(slot_mapping), ptr(pos_ids), ptr(sin_table), ptr(cos_table),
+                                                 c_void_p(stream or 0)),
+        "infiniopRoPEQKPagedCaching",
+    )
+    torch.cuda.synchronize()
+    L.check_error(L.LIBINFINIOP.infiniopDestroyRoPEPagedCachingDescriptor(op))
+    return k_cache, v_cache, q_out
+
+
 def create_kv_caching(handle, k_cache, v_cache, k, v, past_kv_lengths):
     descs = [describe(t) for t in (k_cache, v_cache, k, v, past_kv_lengths)]
     op = L.infiniopOperatorDescriptor_t()

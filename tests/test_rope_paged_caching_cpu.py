@@ -94,6 +94,73 @@ def test_cpu_device_is_not_supported(lib):
     assert status == 5
 
 
+# ---- the variant that rotates the query in the same launch -----------------------------------------------
+
+def qk_specs(Hq=12, **kw):
+    sp = specs(**kw)
+    ntok, D, dtype = sp["k"][0][0], sp["k"][0][2], sp["k"][2]
+    sp["q"] = ((ntok, Hq, D), None, dtype)
+    sp["q_out"] = ((ntok, Hq, D), None, dtype)
+    return sp
+
+
+def create_qk(lib, handle, sp, algo=NEOX, drop=None):
+    names = ("q_out", "q", "k_cache", "v_cache", "k", "v", "slots", "pos", "sin", "cos")
+    descs = [None if n == drop else lib.create_tensor_descriptor(*sp[n]) for n in names]
+    op = lib.infiniopOperatorDescriptor_t()
+    status = lib.LIBINFINIOP.infiniopCreateRoPEQKPagedCachingDescriptor(handle, ctypes.byref(op), *descs, algo)
+    for d in descs:
+        if d is not None:
+            lib.destroy_tensor_descriptor(d)
+    return status, op
+
+
+QK_CASES = [
+    ("valid", OK, lambda s: s),
+    ("valid: q a slice of a fused projection (token stride wider than its heads)", OK,
+     lambda s: mutate(s, "q", strides=(12 * 64 + 2 * 4 * 64, 64, 1))),
+    ("valid: q_out with padded heads", OK, lambda s: mutate(s, "q_out", strides=(12 * 80, 80, 1))),
+    ("q of another dtype (rope.h:84)", BAD_DTYPE, lambda s: mutate(s, "q", dtype=BF16)),
+    ("q_out of another dtype (rope.h:84)", BAD_DTYPE, lambda s: mutate(s, "q_out", dtype=F32)),
+    ("q rank 2 (rope.h:99)", BAD_SHAPE, lambda s: mutate(s, "q", shape=(6, 12 * 64))),
+    ("q with another token count", BAD_SHAPE, lambda s: mutate(s, "q", shape=(5, 12, 64))),
+    ("q with another head size", BAD_SHAPE, lambda s: mutate(s, "q", shape=(6, 12, 128))),
+    ("q_out with another head count (rope.h:109)", BAD_SHAPE, lambda s: mutate(s, "q_out", shape=(6, 8, 64))),
+    ("q last stride 2 (rope.h:152)", BAD_STRIDES, lambda s: mutate(s, "q", strides=(12 * 128, 128, 2))),
+    ("q_out last stride 2 (rope.h:152)", BAD_STRIDES, lambda s: mutate(s, "q_out", strides=(12 * 128, 128, 2))),
+    ("the scatter's checks still apply: slots not i64 (info.h:47)", BAD_DTYPE, lambda s: mutate(s, "slots", dtype=I32)),
+    ("the table checks still apply (rope.h:143)", BAD_SHAPE, lambda s: mutate(s, "cos", shape=(99, 32))),
+]
+
+
+@pytest.mark.parametrize("what,expected,change", QK_CASES, ids=[c[0] for c in QK_CASES])
+def test_validation_with_query(lib, host_amd_handle, what, expected, change):
+    status, op = create_qk(lib, host_amd_handle, change(qk_specs()))
+    assert status == expected, what
+    if status == OK:
+        size = ctypes.c_size_t(7)
+        lib.check_error(lib.LIBINFINIOP.infiniopGetRoPEPagedCachingWorkspaceSize(op, ctypes.byref(size)))
+        assert size.value == 0
+        lib.check_error(lib.LIBINFINIOP.infiniopDestroyRoPEPagedCachingDescriptor(op))
+
+
+def test_query_operands_must_be_given_and_each_descriptor_runs_with_its_own_entry_point(lib, host_amd_handle):
+    for missing in ("q", "q_out", "k", "pos"):
+        status, _ = create_qk(lib, host_amd_handle, qk_specs(), drop=missing)
+        assert status == NULLP, missing
+    BAD_PARAM = 3
+    nil = ctypes.c_void_p(0)
+    status, with_q = create_qk(lib, host_amd_handle, qk_specs())
+    assert status == OK
+    assert lib.LIBINFINIOP.infiniopRoPEPagedCaching(with_q, nil, 0, *([nil] * 8), nil) == BAD_PARAM
+    status, without_q = create(lib, host_amd_handle, specs())
+    assert status == OK
+    assert lib.LIBINFINIOP.infiniopRoPEQKPagedCaching(without_q, nil, 0, *([nil] * 10), nil) == BAD_PARAM
+    assert lib.LIBINFINIOP.infiniopRoPEQKPagedCaching(None, nil, 0, *([nil] * 10), nil) == NULLP
+    for op in (with_q, without_q):
+        lib.check_error(lib.LIBINFINIOP.infiniopDestroyRoPEPagedCachingDescriptor(op))
+
+
 # ---- the oracle function ------------------------------------------------------------------------------------
 
 def tables(table_len, D, dtype, theta=10000.0):
@@ -207,3 +274,48 @@ def test_oracle_clamps_positions_and_skips_padding(oracle):
     oracle.rope_paged_caching(b_k, b_v, k, v, slots, near, sin, cos, False)
     assert torch.equal(a_k.view(torch.int16), b_k.view(torch.int16))
     assert torch.all(a_k[0, :, 2] == 7) and torch.all(a_k[0, :, 5] == 7)  # padding tokens left their slots alone
+
+
+# ---- the rotation on its own (what the fused operator applies to the query) -------------------------------
+
+@pytest.mark.parametrize("neox", [False, True], ids=["gpt_j", "gpt_neox"])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+def test_rope_oracle_equals_the_torch_rotation_bit_for_bit(oracle, dtype, neox):
+    g = torch.Generator().manual_seed(21)
+    x = torch.randn((19, 5, 64), generator=g).to(dtype)
+    pos = torch.randint(0, 200, (19,), generator=g)
+    sin, cos = tables(200, 64, dtype)
+    got = oracle.rope(x, pos, sin, cos, neox)
+    want = oracle.torch_reference_rope(x, pos, sin, cos, neox)
+    view = torch.int32 if dtype == torch.float32 else torch.int16
+    assert torch.equal(got.view(view), want.view(view))
+
+
+@pytest.mark.parametrize("neox", [False, True], ids=["gpt_j", "gpt_neox"])
+def test_rope_oracle_strided_in_place_and_consistent_with_the_fused_function(oracle, neox):
+    """q as a slice of a fused projection output, rotated in place; and rotating k with this function and then
+    scattering it with the (separately pinned) plain scatter leaves exactly what the fused function leaves."""
+    k_cache, v_cache, k, v, slots, pos, sin, cos = make_case(torch.bfloat16, seed=23)
+    ntok, H, D = k.shape
+    fused = torch.randn((ntok, 7 * D + 2 * H * D)).to(torch.bfloat16)
+    q = fused[:, :7 * D].view(ntok, 7, D)
+    assert not q.is_contiguous()
+    want = oracle.torch_reference_rope(q.clone(), pos, sin, cos, neox)
+    untouched = fused[:, 7 * D:].clone()
+    oracle.rope(q, pos, sin, cos, neox, out=q)
+    assert torch.equal(q.contiguous().view(torch.int16), want.view(torch.int16))
+    assert torch.equal(fused[:, 7 * D:], untouched)
+    two_k, two_v = k_cache.clone(), v_cache.clone()
+    oracle.paged_caching(two_k, two_v, oracle.rope(k, pos, sin, cos, neox), v, slots)
+    oracle.rope_paged_caching(k_cache, v_cache, k, v, slots, pos, sin, cos, neox)
+    assert torch.equal(k_cache.view(torch.int16), two_k.view(torch.int16))
+    assert torch.equal(v_cache.view(torch.int16), two_v.view(torch.int16))
+
+
+def test_rope_oracle_clamps_positions(oracle):
+    g = torch.Generator().manual_seed(25)
+    x = torch.randn((6, 2, 32), generator=g).to(torch.float16)
+    sin, cos = tables(10, 32, torch.float16)
+    far = torch.tensor([0, 9, 12, -4, 10 ** 12, 5])
+    assert torch.equal(oracle.rope(x, far, sin, cos, True).view(torch.int16),
+                       oracle.rope(x, far.clamp(0, 9), sin, cos, True).view(torch.int16))

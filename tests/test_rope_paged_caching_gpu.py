@@ -194,3 +194,107 @@ def test_python_operator_then_attention_sees_the_rotated_keys(gpu_handle, oracle
     _, want = oracle.paged_attention(q, k_pool, v_pool, bt, lens, D ** -0.5, return_fp32=True)
     err = (out.float().cpu() - want).abs()
     assert bool((err <= 1e-2 + 2e-3 * want.abs()).all()), err.max()
+
+
+# ---- the query rotated in the same launch (infiniopRoPEQKPagedCaching) ------------------------------------------
+
+def check_qk(gpu_handle, oracle, case, q, algo, what="", q_out=None, in_place=False):
+    """Pools against the fused oracle function, q_out against the rotation on its own (every token, padding too)."""
+    from capi import run_rope_qk_paged_caching
+
+    print(f"case {what} q {tuple(q.shape)} k {tuple(case[2].shape)} {q.dtype} algo {algo} in_place {in_place}", flush=True)
+    dev = [t.to(DEV) for t in case]
+    q_dev = q.to(DEV)
+    out_dev = q_dev if in_place else (q_out.to(DEV) if q_out is not None else torch.full(q.shape, 5.0, dtype=q.dtype, device=DEV))
+    run_rope_qk_paged_caching(gpu_handle, out_dev, q_dev, *dev, algo)
+    want_k, want_v = case[0].clone(), case[1].clone()
+    oracle.rope_paged_caching(want_k, want_v, *case[2:], algo == NEOX)
+    want_q = oracle.rope(q, case[5], case[6], case[7], algo == NEOX)
+    assert torch.equal(bits(dev[0]), bits(want_k)), f"{what}: K pool differs"
+    assert torch.equal(bits(dev[1]), bits(want_v)), f"{what}: V pool differs"
+    assert torch.equal(bits(out_dev.contiguous()), bits(want_q)), f"{what}: rotated query differs"
+    if not in_place:
+        assert torch.equal(bits(q_dev), bits(q)), f"{what}: the query operand was written"
+    return dev, out_dev
+
+
+@pytest.mark.parametrize("algo", [J, NEOX], ids=["gpt_j", "gpt_neox"])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+def test_query_decode_step(gpu_handle, oracle, dtype, algo):
+    """The Llama-3-8B batch-32 decode step with its 32 query heads."""
+    case = make(dtype, 32, 8, 128, seed=51, pad_every=0)
+    q = torch.randn((32, 32, 128), generator=torch.Generator().manual_seed(52)).to(dtype)
+    check_qk(gpu_handle, oracle, case, q, algo, "decode step with query")
+
+
+@pytest.mark.parametrize("in_place", [False, True])
+@pytest.mark.parametrize("algo", [J, NEOX], ids=["gpt_j", "gpt_neox"])
+def test_query_prefill_chunk_padding_tokens_are_rotated_too(gpu_handle, oracle, algo, in_place):
+    case = make(torch.bfloat16, 1000, 8, 128, NB=1200, seed=53)  # every ninth slot is padding
+    q = torch.randn((1000, 32, 128), generator=torch.Generator().manual_seed(54)).to(torch.bfloat16)
+    check_qk(gpu_handle, oracle, case, q, algo, "prefill chunk with query", in_place=in_place)
+
+
+@pytest.mark.parametrize("Hq,Hkv,D,Dv", [(1, 1, 64, 64), (5, 5, 64, 128), (48, 3, 256, 64), (16, 1, 576, 512), (7, 2, 24, 40)])
+def test_query_head_counts_and_sizes(gpu_handle, oracle, Hq, Hkv, D, Dv):
+    case = make(torch.float16, 77, Hkv, D, Dv=Dv, seed=55 + Hq)
+    q = torch.randn((77, Hq, D), generator=torch.Generator().manual_seed(56)).to(torch.float16)
+    check_qk(gpu_handle, oracle, case, q, NEOX if Hq % 2 else J, f"Hq={Hq} Hkv={Hkv} D={D}/{Dv}")
+
+
+def test_query_key_and_value_as_slices_of_one_projection_output(gpu_handle, oracle):
+    """q, k, v are column slices of one [tokens, (Hq + 2 Hkv) D] tensor, rotated in place / scattered from there."""
+    from capi import run_rope_qk_paged_caching
+
+    ntok, Hq, Hkv, D = 200, 16, 4, 128
+    case = make(torch.bfloat16, ntok, Hkv, D, seed=61)
+    g = torch.Generator().manual_seed(62)
+    fused = torch.randn((ntok, (Hq + 2 * Hkv) * D), generator=g).to(torch.bfloat16)
+    fused[:, Hq * D:(Hq + Hkv) * D] = case[2].reshape(ntok, -1)
+    fused[:, (Hq + Hkv) * D:] = case[3].reshape(ntok, -1)
+    fused_dev = fused.to(DEV)
+    q_dev = fused_dev[:, :Hq * D].view(ntok, Hq, D)
+    k_dev = fused_dev[:, Hq * D:(Hq + Hkv) * D].view(ntok, Hkv, D)
+    v_dev = fused_dev[:, (Hq + Hkv) * D:].view(ntok, Hkv, D)
+    assert not q_dev.is_contiguous() and not k_dev.is_contiguous()
+    dev = [t.to(DEV) for t in case]
+    run_rope_qk_paged_caching(gpu_handle, q_dev, q_dev, dev[0], dev[1], k_dev, v_dev, *dev[4:], NEOX)
+    want_k, want_v = case[0].clone(), case[1].clone()
+    oracle.rope_paged_caching(want_k, want_v, *case[2:], True)
+    want_q = oracle.rope(fused[:, :Hq * D].reshape(ntok, Hq, D), case[5], case[6], case[7], True)
+    assert torch.equal(bits(dev[0]), bits(want_k)) and torch.equal(bits(dev[1]), bits(want_v))
+    assert torch.equal(bits(q_dev.contiguous()), bits(want_q))
+    assert torch.equal(bits(fused_dev[:, Hq * D:].contiguous()), bits(fused[:, Hq * D:].contiguous())), "k / v columns were written"
+
+
+def test_query_unaligned_and_padded_operands_take_the_pair_at_a_time_path(gpu_handle, oracle):
+    from capi import run_rope_qk_paged_caching
+
+    case = make(torch.float16, 50, 3, 64, seed=63)
+    q = torch.randn((50, 6, 64), generator=torch.Generator().manual_seed(64)).to(torch.float16)
+    dev = [t.to(DEV) for t in case]
+    raw = torch.zeros(q.numel() + 1, dtype=q.dtype, device=DEV)
+    q_dev = raw[1:].view(q.shape)  # 2 bytes off a 16-byte boundary
+    q_dev.copy_(q)
+    out_dev = torch.full((50, 6, 72), 5.0, dtype=q.dtype, device=DEV)[:, :, :64]  # padded heads
+    run_rope_qk_paged_caching(gpu_handle, out_dev, q_dev, *dev, J)
+    want_k, want_v = case[0].clone(), case[1].clone()
+    oracle.rope_paged_caching(want_k, want_v, *case[2:], False)
+    assert torch.equal(bits(dev[0]), bits(want_k)) and torch.equal(bits(dev[1]), bits(want_v))
+    assert torch.equal(bits(out_dev.contiguous()), bits(oracle.rope(q, case[5], case[6], case[7], False)))
+
+
+def test_query_python_operator(gpu_handle, oracle):
+    from infinicore_amd import ops
+
+    case = make(torch.bfloat16, 32, 8, 128, seed=65, pad_every=0)
+    q = torch.randn((32, 32, 128), generator=torch.Generator().manual_seed(66)).to(torch.bfloat16)
+    dev = [t.to(DEV) for t in case]
+    q_dev = q.to(DEV)
+    kd, vd, qd = ops.rope_paged_caching(*dev, L.RoPEAlgo.GPT_NEOX, q=q_dev)
+    torch.cuda.synchronize()
+    assert qd is q_dev
+    want_k, want_v = case[0].clone(), case[1].clone()
+    oracle.rope_paged_caching(want_k, want_v, *case[2:], True)
+    assert torch.equal(bits(kd), bits(want_k)) and torch.equal(bits(vd), bits(want_v))
+    assert torch.equal(bits(qd), bits(oracle.rope(q, case[5], case[6], case[7], True)))
