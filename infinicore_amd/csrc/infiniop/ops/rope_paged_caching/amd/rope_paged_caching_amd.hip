@@ -56,6 +56,7 @@ struct QueryArgs<true> {
     void *q_out;
     const void *q;
     int32_t num_q_heads;
+    int32_t threads_per_row; // threads of a token's box that share one query vector (a power of two)
     int64_t q_token_stride, q_head_stride, q_out_token_stride, q_out_head_stride;
 };
 
@@ -183,19 +184,22 @@ __device__ __forceinline__ void ropeScatter(const Args &a, const QueryArgs<QUERY
     const S *sin_row = static_cast<const S *>(a.sin_table) + pos * table_dim;
     const S *cos_row = static_cast<const S *>(a.cos_table) + pos * table_dim;
 
-    for (int head = y0; head < a.num_kv_heads + num_q_heads; head += y_step) {
-        if constexpr (QUERY) {
-            if (head >= a.num_kv_heads) {
-                const int64_t q_head = head - a.num_kv_heads;
-                rotateRow<S, VEC>(static_cast<const S *>(qa.q) + token * qa.q_token_stride + q_head * qa.q_head_stride,
-                                  static_cast<S *>(qa.q_out) + token * qa.q_out_token_stride + q_head * qa.q_out_head_stride,
-                                  sin_row, cos_row, table_dim, a.neox != 0, x0, x_step);
-                continue;
-            }
+    if constexpr (QUERY) {
+        // The query first (its loads depend on nothing the cache writes need). The token's box of x * y threads is
+        // dealt anew: as many threads per vector as the rotation has steps, the others on further heads, so that
+        // e.g. 32 heads of 128 bf16 elements (8 steps each) are one round of a 256-thread box.
+        const int flat = y0 * x_step + x0;
+        const int heads_at_once = (x_step * y_step) / qa.threads_per_row;
+        for (int q_head = flat / qa.threads_per_row; q_head < num_q_heads; q_head += heads_at_once) {
+            rotateRow<S, VEC>(static_cast<const S *>(qa.q) + token * qa.q_token_stride + q_head * qa.q_head_stride,
+                              static_cast<S *>(qa.q_out) + token * qa.q_out_token_stride + q_head * qa.q_out_head_stride,
+                              sin_row, cos_row, table_dim, a.neox != 0, flat & (qa.threads_per_row - 1), qa.threads_per_row);
         }
-        if (QUERY && !cached) {
-            continue;
+        if (!cached) {
+            return;
         }
+    }
+    for (int head = y0; head < a.num_kv_heads; head += y_step) {
         const S *k_src = static_cast<const S *>(a.k) + token * a.k_src_token_stride + static_cast<int64_t>(head) * a.head_size;
         const S *v_src = static_cast<const S *>(a.v) + token * a.v_src_token_stride + static_cast<int64_t>(head) * a.value_size;
         S *k_dst = static_cast<S *>(a.k_cache) + page * a.k_block_stride + head * a.k_head_stride + row * a.k_slot_stride;
@@ -233,13 +237,15 @@ int ceilPow2(int x) {
 bool multipleOf16(uint64_t x) { return (x & 15u) == 0; }
 
 template <typename T>
-void launch(const Args &a, const QueryArgs<true> &qa, bool vec, int row_steps, hipStream_t stream) {
+void launch(const Args &a, QueryArgs<true> qa, bool vec, int row_steps, int rotate_steps, hipStream_t stream) {
     // 256-thread box: x = steps along a row, y = heads, z = tokens
     int bx = ceilPow2(row_steps);
     bx = bx > 64 ? 64 : bx;
     int by = ceilPow2(a.num_kv_heads + qa.num_q_heads);
     by = by > 256 / bx ? 256 / bx : by;
     const int bz = 256 / (bx * by);
+    const int rotate_threads = ceilPow2(rotate_steps > 0 ? rotate_steps : 1);
+    qa.threads_per_row = rotate_threads < bx * by ? rotate_threads : bx * by;
     const dim3 block(bx, by, bz);
     const dim3 grid(static_cast<unsigned>((a.num_tokens + bz - 1) / bz));
     if (qa.num_q_heads > 0) {
@@ -373,9 +379,9 @@ infiniStatus_t Descriptor::calculate(void *workspace, size_t workspace_size, voi
     const int row_steps = rotate_steps > copy_steps ? rotate_steps : copy_steps;
     auto stream = static_cast<hipStream_t>(stream_);
     switch (in.dtype) {
-    case INFINI_DTYPE_F16: launch<F16>(a, qa, vec, row_steps > 0 ? row_steps : 1, stream); break;
-    case INFINI_DTYPE_BF16: launch<BF16>(a, qa, vec, row_steps > 0 ? row_steps : 1, stream); break;
-    case INFINI_DTYPE_F32: launch<F32>(a, qa, vec, row_steps > 0 ? row_steps : 1, stream); break;
+    case INFINI_DTYPE_F16: launch<F16>(a, qa, vec, row_steps > 0 ? row_steps : 1, rotate_steps, stream); break;
+    case INFINI_DTYPE_BF16: launch<BF16>(a, qa, vec, row_steps > 0 ? row_steps : 1, rotate_steps, stream); break;
+    case INFINI_DTYPE_F32: launch<F32>(a, qa, vec, row_steps > 0 ? row_steps : 1, rotate_steps, stream); break;
     default: return INFINI_STATUS_BAD_TENSOR_DTYPE;
     }
     return hipGetLastError() == hipSuccess ? INFINI_STATUS_SUCCESS : INFINI_STATUS_INTERNAL_ERROR;
