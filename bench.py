@@ -48,7 +48,8 @@ MEASURED_TRAFFIC = {
     "m2_mla_128_heads_b32": (216_200_000, "decode_mla_m1_m2_kernel_stats_and_traffic.md", "0ad1a65"),
     "c5_prefill_scatter": (32_100_000, "paged_caching_c5_prefill_scatter_kernel_stats_and_traffic.md", "a636ea0"),
     "k2_append_prefill_chunk": (33_600_000, "kv_caching_k2_append_prefill_chunk_kernel_stats_and_traffic.md", "f6351eb"),
-    "r2_rope_scatter_prefill_chunk": (33_550_000, "rope_paged_caching_r1_r2_kernel_stats_and_traffic.md", "fa02f8a"),
+    "r2_rope_scatter_prefill_chunk": (33_550_000, "rope_paged_caching_r1_r2_kernel_stats_and_traffic.md", "1b3c6fa"),
+    "r4_rope_qk_scatter_prefill_chunk": (100_530_000, "rope_paged_caching_r1_r2_kernel_stats_and_traffic.md", "1b3c6fa"),
     "p3_llama3_8b_chunked": (451_500_000, "prefill_tiled_p3_llama3_8b_chunked_counters.md", "a4c5528"),  # fetched only
 }
 
