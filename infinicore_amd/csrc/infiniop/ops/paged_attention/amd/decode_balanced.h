@@ -364,7 +364,7 @@ decodeBalancedKernel(const void *early_seq_lens, int early_num_seqs, int early_m
             const int out_head = kv_head * a.group + hg;
             if (whole) {
                 S *o_ptr = static_cast<S *>(a.out) + seq * a.o_stride + out_head * a.o_head_stride;
-                storeOutputRow<T, HEAD>(o_ptr + G::kCols * c, state, rr, 1.0f / (l_h + 1e-6f));
+                storeOutputRow<T, HEAD>(o_ptr, c, state, rr, 1.0f / (l_h + 1e-6f));
             } else {
                 const int64_t slot = static_cast<int64_t>(piece + seq) * a.num_heads + out_head;
                 storePartialRow<HEAD>(a.part_acc + slot * HEAD + G::kCols * c, state, rr);
@@ -637,7 +637,7 @@ decodeBalancedKernel(const void *early_seq_lens, int early_num_seqs, int early_m
             for (int rr = 0; rr < 4; ++rr) {
                 if (4 * g + rr < heads_here) {
                     S *o_ptr = static_cast<S *>(a.out) + s * a.o_stride + (first_head + 4 * g + rr) * a.o_head_stride;
-                    storeOutputRow<T, HEAD>(o_ptr + G::kCols * c, own, rr, 1.0f / (l_run[rr] + 1e-6f));
+                    storeOutputRow<T, HEAD>(o_ptr, c, own, rr, 1.0f / (l_run[rr] + 1e-6f));
                 }
             }
         }
@@ -736,7 +736,7 @@ decodeBalancedMergeKernel(const void *early_seq_lens, const int2 *early_seq_piec
             w[i] = T::pack2(acc[2 * i] * inv_l, acc[2 * i + 1] * inv_l);
         }
         S *o_ptr = static_cast<S *>(a.out) + seq * a.o_stride + head * a.o_head_stride;
-        storeStrip<HEAD>(o_ptr + kCols * c, w);
+        storeStrip<HEAD>(o_ptr, c, w);
     }
 }
 

@@ -99,8 +99,18 @@ struct TileGeometry {
     static constexpr int kSwizzle = (HEAD == 64 || HEAD == 192) ? 8 : 16;
     static constexpr int kCols = HEAD / 16;           // V / output columns per lane
     static constexpr int kWords = kCols / 2;          // dwords of one V row strip
-    // register sets: about 16 KiB of requests in flight per wavefront (12 KiB at head 192, where a third set
-    // pushed the kernel out of the vector register file: 91.5 -> 90.9 us at the c2 shape with two)
+    // Which columns a lane's strip is made of: one contiguous piece (columns kCols c ..), except at head 192,
+    // where the 24 bytes of a lane are two pieces - the 16-byte chunk c of columns 0 .. 127 and the four columns
+    // from 128 + 4 c - so that the 16 lanes c = 0..15 of one load or store instruction cover one contiguous run
+    // of a row. (As one 24-byte piece fetched 8 bytes at a time, every instruction touched every cache line of
+    // the row three times over: 90.9 us at the Llama-3-8B batch-32 shape against 79.2 us with the two pieces.
+    // Head 256, two adjacent 16-byte loads per lane, gains nothing from the same split: 105.0 vs 103.1 us.)
+    static constexpr int kFirstCols = HEAD == 192 ? 8 : kCols;
+    static constexpr int kRestCols = kCols - kFirstCols; // 4 at head 192, else 0
+    static __host__ __device__ constexpr int firstColumn(int c) { return kFirstCols * c; }
+    static __host__ __device__ constexpr int restColumn(int c) { return 128 + kRestCols * c; }
+    // register sets: about 16 KiB of requests in flight per wavefront (12 KiB at head 192; a third set there
+    // changes nothing: 92.0 vs 90.9 us before the strips were split)
     static constexpr int kBuffers = HEAD == 64 ? 5 : (HEAD >= 192 ? 2 : 3);
     static __device__ __forceinline__ int kRow(int j, int lane) { return (64 * j + lane) / kChunksPerRow; }
     static __device__ __forceinline__ int kChunk(int j, int lane) { return (64 * j + lane) % kChunksPerRow; }
@@ -155,45 +165,50 @@ __device__ __forceinline__ uint2 loadLane8(const char *uniform_base, uint32_t la
     return make_uint2(v[0], v[1]);
 }
 
-// This lane's strip of one V row: 2 * kCols bytes at uniform_base + lane_offset
+// This lane's strip of one V row: the first piece at uniform_base + first_offset, the rest piece (heads above
+// 128) at uniform_base + rest_offset; 16-byte loads, 8-byte ones for pieces of four columns
 template <int HEAD>
-__device__ __forceinline__ void loadStrip(const char *uniform_base, uint32_t lane_offset,
+__device__ __forceinline__ void loadStrip(const char *uniform_base, uint32_t first_offset, uint32_t rest_offset,
                                           uint32_t (&w)[TileGeometry<HEAD>::kWords]) {
-    constexpr int kWords = TileGeometry<HEAD>::kWords;
-    if constexpr (kWords % 4 == 0) {
+    using G = TileGeometry<HEAD>;
+    static_assert(G::kFirstCols % 8 == 0 || G::kFirstCols == 4, "16-byte loads, or one 8-byte load");
+    static_assert(G::kRestCols == 0 || G::kRestCols == 4, "the rest piece is one 8-byte load");
+    if constexpr (G::kFirstCols % 8 == 0) {
 #pragma unroll
-        for (int i = 0; i < kWords / 4; ++i) {
-            const uint4 x = loadLane16(uniform_base, lane_offset + 16 * i);
+        for (int i = 0; i < G::kFirstCols / 8; ++i) {
+            const uint4 x = loadLane16(uniform_base, first_offset + 16 * i);
             w[4 * i] = x.x, w[4 * i + 1] = x.y, w[4 * i + 2] = x.z, w[4 * i + 3] = x.w;
         }
     } else {
-#pragma unroll
-        for (int i = 0; i < kWords / 2; ++i) {
-            const uint2 x = loadLane8(uniform_base, lane_offset + 8 * i);
-            w[2 * i] = x.x, w[2 * i + 1] = x.y;
-        }
+        const uint2 x = loadLane8(uniform_base, first_offset);
+        w[0] = x.x, w[1] = x.y;
+    }
+    if constexpr (G::kRestCols == 4) {
+        const uint2 x = loadLane8(uniform_base, rest_offset);
+        w[G::kFirstCols / 2] = x.x, w[G::kFirstCols / 2 + 1] = x.y;
     }
 }
 
-// kCols consecutive output values of one row, packed two per dword, to dst (2 * kCols bytes; 16-byte
-// stores when the strip is a multiple of 16 bytes, else 8-byte stores)
-template <int HEAD>
-__device__ __forceinline__ void storeStrip(void *dst, const uint32_t (&w)[TileGeometry<HEAD>::kWords]) {
-    constexpr int kWords = TileGeometry<HEAD>::kWords;
-    if constexpr (kWords % 4 == 0) {
+// The kCols output values of strip c of one row, packed two per dword, into the row that starts at `row`
+// (the pieces of TileGeometry: 16-byte stores, 8-byte ones for pieces of four columns)
+template <int HEAD, typename S>
+__device__ __forceinline__ void storeStrip(S *row, int c, const uint32_t (&w)[TileGeometry<HEAD>::kWords]) {
+    using G = TileGeometry<HEAD>;
+    static_assert(sizeof(S) == 2, "two values per dword");
+    if constexpr (G::kFirstCols % 8 == 0) {
 #pragma unroll
-        for (int i = 0; i < kWords / 4; ++i) {
-            reinterpret_cast<uint4 *>(dst)[i] = make_uint4(w[4 * i], w[4 * i + 1], w[4 * i + 2], w[4 * i + 3]);
+        for (int i = 0; i < G::kFirstCols / 8; ++i) {
+            reinterpret_cast<uint4 *>(row + G::firstColumn(c))[i] = make_uint4(w[4 * i], w[4 * i + 1], w[4 * i + 2], w[4 * i + 3]);
         }
     } else {
-#pragma unroll
-        for (int i = 0; i < kWords / 2; ++i) {
-            reinterpret_cast<uint2 *>(dst)[i] = make_uint2(w[2 * i], w[2 * i + 1]);
-        }
+        *reinterpret_cast<uint2 *>(row + G::firstColumn(c)) = make_uint2(w[0], w[1]);
+    }
+    if constexpr (G::kRestCols == 4) {
+        *reinterpret_cast<uint2 *>(row + G::restColumn(c)) = make_uint2(w[G::kFirstCols / 2], w[G::kFirstCols / 2 + 1]);
     }
 }
 
-// Softmax state of one wavefront. o[e][r] = O[head 4g+r of the chunk][column c*kCols + e].
+// Softmax state of one wavefront. o[e][r] = O[head 4g+r of the chunk][column e of strip c (TileGeometry)].
 template <int HEAD>
 struct TileState {
     f32x4 o[TileGeometry<HEAD>::kCols];
@@ -201,18 +216,35 @@ struct TileState {
     float l; // sum of rounded probabilities of head c over this lane's tokens only
 };
 
-// Row rr of the accumulators, scaled, rounded to the storage dtype and written to dst
+// Row rr of the accumulators, scaled, rounded to the storage dtype and written into the output row at `row`
 template <typename T, int HEAD>
-__device__ __forceinline__ void storeOutputRow(void *dst, const TileState<HEAD> &st, int rr, float factor) {
+__device__ __forceinline__ void storeOutputRow(typename T::storage *row, int c, const TileState<HEAD> &st, int rr, float factor) {
     uint32_t w[TileGeometry<HEAD>::kWords];
 #pragma unroll
     for (int i = 0; i < TileGeometry<HEAD>::kWords; ++i) {
         w[i] = T::pack2(st.o[2 * i][rr] * factor, st.o[2 * i + 1][rr] * factor);
     }
-    storeStrip<HEAD>(dst, w);
+    storeStrip<HEAD>(row, c, w);
 }
 
-// Row rr of the accumulators as fp32 partial result (kCols floats, 16-byte aligned)
+// Row rr of the accumulators as fp32 partial result in column order, into the partial row at `row` (what the
+// merge kernels of the fixed partitions read: value_size floats per row)
+template <int HEAD>
+__device__ __forceinline__ void storePartialRowInColumnOrder(float *row, int c, const TileState<HEAD> &st, int rr) {
+    using G = TileGeometry<HEAD>;
+#pragma unroll
+    for (int i = 0; i < G::kFirstCols / 4; ++i) {
+        reinterpret_cast<float4 *>(row + G::firstColumn(c))[i] = make_float4(st.o[4 * i][rr], st.o[4 * i + 1][rr], st.o[4 * i + 2][rr], st.o[4 * i + 3][rr]);
+    }
+#pragma unroll
+    for (int i = 0; i < G::kRestCols / 4; ++i) {
+        const int e = G::kFirstCols + 4 * i;
+        reinterpret_cast<float4 *>(row + G::restColumn(c))[i] = make_float4(st.o[e][rr], st.o[e + 1][rr], st.o[e + 2][rr], st.o[e + 3][rr]);
+    }
+}
+
+// Row rr of the accumulators as fp32 partial result, the lane's kCols floats side by side at dst (16-byte
+// aligned; the layout of the work-equalising schedule, whose merge reads the rows the same way)
 template <int HEAD>
 __device__ __forceinline__ void storePartialRow(float *dst, const TileState<HEAD> &st, int rr) {
 #pragma unroll
@@ -324,7 +356,7 @@ __device__ __forceinline__ void computeTile(TileState<HEAD> &st, const TileRegs<
     uint2 p_op, p_lo = make_uint2(0, 0);
     softmaxStep<T, G::kCols>(st.o, st.m, st.l, s, g, scale_log2, slope, rel_pos0, valid, p_op, p_lo);
 
-    // one 16-column output tile per e: column c*kCols + e of rows 4g..4g+3
+    // one 16-column output tile per e: column e of strip c, rows 4g..4g+3
 #pragma unroll
     for (int w = 0; w < G::kWords; ++w) {
         accumulatePair<T>(st.o[2 * w], st.o[2 * w + 1], r.v[0][w], r.v[1][w], r.v[2][w], r.v[3][w], p_op, p_lo, g, valid);
@@ -359,7 +391,8 @@ __device__ __forceinline__ void streamTiles(int n_tiles, Load loadTile, Compute 
 template <int HEAD>
 struct LaneOffsets {
     uint32_t k[TileGeometry<HEAD>::kLoads];
-    uint32_t v[4];
+    uint32_t v[4];       // first piece of the strip of token row 4g + j
+    uint32_t v_rest;     // from there to the rest piece of the same row (heads above 128)
     __device__ __forceinline__ LaneOffsets(int lane, uint32_t k_row_bytes, uint32_t v_row_bytes) {
         using G = TileGeometry<HEAD>;
 #pragma unroll
@@ -368,8 +401,9 @@ struct LaneOffsets {
         }
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            v[j] = (4 * (lane >> 4) + j) * v_row_bytes + 2 * G::kCols * (lane & 15);
+            v[j] = (4 * (lane >> 4) + j) * v_row_bytes + 2 * G::firstColumn(lane & 15);
         }
+        v_rest = 2 * (G::restColumn(lane & 15) - G::firstColumn(lane & 15));
     }
 };
 
@@ -385,7 +419,7 @@ __device__ __forceinline__ TileRegs<HEAD> loadTileRegs(const char *k_tile, const
     }
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-        loadStrip<HEAD>(v_tile, off.v[j] & lane_mask, r.v[j]);
+        loadStrip<HEAD>(v_tile, off.v[j] & lane_mask, (off.v[j] + off.v_rest) & lane_mask, r.v[j]);
     }
     return r;
 }
@@ -497,10 +531,10 @@ __global__ void __launch_bounds__(64) decodeTiledKernel(DecodeArgs a) {
         const int out_head = kv_head * a.group + hg;
         if (single) {
             S *o_ptr = static_cast<S *>(a.out) + seq * a.o_stride + out_head * a.o_head_stride;
-            storeOutputRow<T, HEAD>(o_ptr + G::kCols * c, st, rr, 1.0f / (l_h + 1e-6f));
+            storeOutputRow<T, HEAD>(o_ptr, c, st, rr, 1.0f / (l_h + 1e-6f));
         } else {
             const int64_t slot = (static_cast<int64_t>(seq) * a.num_heads + out_head) * a.max_partitions + part;
-            storePartialRow<HEAD>(a.part_acc + slot * HEAD + G::kCols * c, st, rr);
+            storePartialRowInColumnOrder<HEAD>(a.part_acc + slot * HEAD, c, st, rr);
             if (c == 0) {
                 a.part_m[slot] = m_h;
                 a.part_l[slot] = l_h;

@@ -103,22 +103,24 @@ __device__ __forceinline__ bool findRowBlock(const PrefillArgs &a, int lane, int
     return false;
 }
 
-// This lane's strip of one V row (2 * kCols bytes), through the caches
+// This lane's strip of one V row, through the caches: the first piece at `first`, the rest piece (heads above
+// 128; see TileGeometry) `rest_bytes` further on
 template <int HEAD>
-__device__ __forceinline__ void loadStripCached(const char *src, uint32_t (&w)[TileGeometry<HEAD>::kWords]) {
-    constexpr int kWords = TileGeometry<HEAD>::kWords;
-    if constexpr (kWords % 4 == 0) {
+__device__ __forceinline__ void loadStripCached(const char *first, uint32_t rest_bytes, uint32_t (&w)[TileGeometry<HEAD>::kWords]) {
+    using G = TileGeometry<HEAD>;
+    if constexpr (G::kFirstCols % 8 == 0) {
 #pragma unroll
-        for (int i = 0; i < kWords / 4; ++i) {
-            const uint4 x = reinterpret_cast<const uint4 *>(src)[i];
+        for (int i = 0; i < G::kFirstCols / 8; ++i) {
+            const uint4 x = reinterpret_cast<const uint4 *>(first)[i];
             w[4 * i] = x.x, w[4 * i + 1] = x.y, w[4 * i + 2] = x.z, w[4 * i + 3] = x.w;
         }
     } else {
-#pragma unroll
-        for (int i = 0; i < kWords / 2; ++i) {
-            const uint2 x = reinterpret_cast<const uint2 *>(src)[i];
-            w[2 * i] = x.x, w[2 * i + 1] = x.y;
-        }
+        const uint2 x = *reinterpret_cast<const uint2 *>(first);
+        w[0] = x.x, w[1] = x.y;
+    }
+    if constexpr (G::kRestCols == 4) {
+        const uint2 x = *reinterpret_cast<const uint2 *>(first + rest_bytes);
+        w[G::kFirstCols / 2] = x.x, w[G::kFirstCols / 2 + 1] = x.y;
     }
 }
 
@@ -262,7 +264,7 @@ __global__ void __launch_bounds__(kPrefillThreads, HEAD <= 192 ? 2 : 1) prefillT
                 for (int j = 0; j < 4; ++j) {
                     uint32_t lane_off = off.v[j];
                     asm volatile("" : "+v"(lane_off));
-                    loadStripCached<HEAD>(v_tile + lane_off, v_stage[j]);
+                    loadStripCached<HEAD>(v_tile + lane_off, off.v_rest, v_stage[j]);
                 }
             }
             return;
@@ -289,9 +291,9 @@ __global__ void __launch_bounds__(kPrefillThreads, HEAD <= 192 ? 2 : 1) prefillT
                 const int page = (small_pages && g >= 2) ? id1 : id0;
                 const int page_row = small_pages ? (o & 7) : row0 + o;
                 const char *src = v_head + (page * a.v_batch_stride + page_row * a.v_row_stride) * static_cast<int64_t>(sizeof(S))
-                                + 2 * G::kCols * c;
+                                + 2 * G::firstColumn(c);
                 if (t + o < kv_len) {
-                    loadStripCached<HEAD>(src, v_stage[i]);
+                    loadStripCached<HEAD>(src, off.v_rest, v_stage[i]);
                 } else {
 #pragma unroll
                     for (int wd = 0; wd < G::kWords; ++wd) {
@@ -323,7 +325,7 @@ __global__ void __launch_bounds__(kPrefillThreads, HEAD <= 192 ? 2 : 1) prefillT
     };
 
     // ---- softmax state ----
-    // o[r][e][rr] = O[row 4g+rr of group r][column c*kCols+e]; ol[r][rr] = sum of that row's probabilities
+    // o[r][e][rr] = O[row 4g+rr of group r][column e of strip c]; ol[r][rr] = sum of that row's probabilities
     // (computed by the matrix unit as P . 1, so it sums exactly the rounded probabilities the numerator
     // used and already sits in the accumulators' row layout); m[r] = running maximum of row c, in units
     // of the raw dot product when there is no ALiBi (scale > 0 keeps the order), else of the scaled score.
@@ -474,7 +476,7 @@ __global__ void __launch_bounds__(kPrefillThreads, HEAD <= 192 ? 2 : 1) prefillT
         }
     }
 
-    // ---- normalise and store: lane writes columns c*kCols .. of rows 4g..4g+3 of each group ----
+    // ---- normalise and store: lane writes strip c of rows 4g..4g+3 of each group ----
 #pragma unroll
     for (int r = 0; r < R; ++r) {
 #pragma unroll
@@ -494,7 +496,7 @@ __global__ void __launch_bounds__(kPrefillThreads, HEAD <= 192 ? 2 : 1) prefillT
                 packed[i] = T::pack2(o[r][2 * i][rr] * inv_l, o[r][2 * i + 1][rr] * inv_l);
             }
             S *o_ptr = static_cast<S *>(a.out) + (span.q_start + token) * a.o_stride + head * a.o_head_stride;
-            storeStrip<HEAD>(o_ptr + G::kCols * c, packed);
+            storeStrip<HEAD>(o_ptr, c, packed);
         }
     }
 }
