@@ -555,7 +555,8 @@ __global__ void __launch_bounds__(kMlaWideThreads, 2) decodeMlaWideKernel(Decode
 
     // Register sets for tiles on their way: one (tile t + 1 while tile t is computed). A second set fits
     // the single-chunk variant (185 registers, no spills) and was measured: 38.7 vs 37.6 us at 32 sequences,
-    // 139 vs 136 at 128 - one more tile in flight is not what holds that variant back.
+    // 139 vs 136 at 128 - one more tile in flight is not what holds that variant back. The four-chunk variant
+    // (211 registers with one set) does not take a second one: 256 registers and 100 spilled, inside the loop.
     constexpr int kSets = 1;
     uint4 stage_sets[kSets][kLoads];
 #pragma unroll
@@ -696,20 +697,26 @@ __global__ void __launch_bounds__(kMlaWideThreads, 2) decodeMlaWideKernel(Decode
         const int valid = min(kMlaWideTileTokens, end - tok0);
         uint4 p_op, p_lo;
         softmaxStepPair<T, kOwnBlocks>(o, m, l, s0, s1, g, a.scale_log2, slope, tok0 - (len - 1), valid, p_op, p_lo);
-        // all column blocks with the high parts first, then with the low parts (independent chains)
-        uint4 vf[kOwnBlocks];
+        // column blocks four at a time: their V operands from LDS, the high parts of the probabilities, then
+        // the low parts (four independent chains - a matrix instruction that accumulates into the result of the
+        // one before waits for it); all blocks at once kept 64 registers of operands alive
+        constexpr int kGroup = 4;
 #pragma unroll
-        for (int e = 0; e < kOwnBlocks; ++e) {
-            vf[e] = v_lds[buf][((first_block + e) * 4 + g) * 16 + c];
-        }
+        for (int e0 = 0; e0 < kOwnBlocks; e0 += kGroup) {
+            uint4 vf[kGroup];
 #pragma unroll
-        for (int e = 0; e < kOwnBlocks; ++e) {
-            o[e] = T::mfmaK32(p_op, vf[e], o[e]);
-        }
-        if constexpr (T::kSplitProbabilities) {
+            for (int e = 0; e < kGroup; ++e) {
+                vf[e] = v_lds[buf][((first_block + e0 + e) * 4 + g) * 16 + c];
+            }
 #pragma unroll
-            for (int e = 0; e < kOwnBlocks; ++e) {
-                o[e] = T::mfmaK32(p_lo, vf[e], o[e]);
+            for (int e = 0; e < kGroup; ++e) {
+                o[e0 + e] = T::mfmaK32(p_op, vf[e], o[e0 + e]);
+            }
+            if constexpr (T::kSplitProbabilities) {
+#pragma unroll
+                for (int e = 0; e < kGroup; ++e) {
+                    o[e0 + e] = T::mfmaK32(p_lo, vf[e], o[e0 + e]);
+                }
             }
         }
     }
