@@ -75,9 +75,10 @@ __global__ void __launch_bounds__(256) kvCachingAppendKernel(AppendArgs a) {
     }
 }
 
+// Smallest power of two >= x, at most 2^30.
 int ceilPow2(int x) {
     int p = 1;
-    while (p < x) {
+    while (p < x && p < (1 << 30)) {
         p <<= 1;
     }
     return p;

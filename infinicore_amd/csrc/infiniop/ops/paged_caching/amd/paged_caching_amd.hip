@@ -110,9 +110,10 @@ pagedCachingScatterKernel(const int64_t *early_slot_mapping, int64_t early_num_t
     }
 }
 
+// Smallest power of two >= x, at most 2^30.
 int ceilPow2(int x) {
     int p = 1;
-    while (p < x) {
+    while (p < x && p < (1 << 30)) {
         p <<= 1;
     }
     return p;
@@ -154,6 +155,11 @@ infiniStatus_t Descriptor::calculate(void *workspace, size_t workspace_size, voi
     }
     if (k_cache == nullptr || v_cache == nullptr || k == nullptr || v == nullptr || slot_mapping == nullptr) {
         return INFINI_STATUS_NULL_POINTER;
+    }
+    // the kernel counts heads, row units and workgroups in 32 bits
+    if (in.num_kv_heads > 0x7fffffff || in.head_size > 0x7fffffff || in.v_head_size > 0x7fffffff
+        || in.block_size > 0x7fffffff || in.num_tokens > 0x7fffffff) {
+        return INFINI_STATUS_BAD_TENSOR_SHAPE;
     }
 
     const uint64_t es = infiniSizeOf(in.dtype);

@@ -226,9 +226,10 @@ __global__ void __launch_bounds__(256) ropeScatterQueryKernel(Args a, QueryArgs<
     ropeScatter<T, VEC, true>(a, qa);
 }
 
+// Smallest power of two >= x, at most 2^30.
 int ceilPow2(int x) {
     int p = 1;
-    while (p < x) {
+    while (p < x && p < (1 << 30)) {
         p <<= 1;
     }
     return p;
@@ -294,7 +295,9 @@ infiniStatus_t Descriptor::calculate(void *workspace, size_t workspace_size, voi
     if (rotates_query && (q_out == nullptr || q == nullptr)) {
         return INFINI_STATUS_NULL_POINTER;
     }
-    if (in.num_kv_heads + (rotates_query ? _info.num_q_heads : 0) > 0x7fffffff) {
+    // the kernel counts heads, row steps and workgroups in 32 bits
+    if (in.num_kv_heads + (rotates_query ? _info.num_q_heads : 0) > 0x7fffffff || in.head_size > 0x7fffffff
+        || in.v_head_size > 0x7fffffff || in.block_size > 0x7fffffff || in.num_tokens > 0x7fffffff) {
         return INFINI_STATUS_BAD_TENSOR_SHAPE;
     }
     if (k_cache == nullptr || v_cache == nullptr || k == nullptr || v == nullptr || slot_mapping == nullptr

@@ -161,6 +161,17 @@ def test_query_operands_must_be_given_and_each_descriptor_runs_with_its_own_entr
         lib.check_error(lib.LIBINFINIOP.infiniopDestroyRoPEPagedCachingDescriptor(op))
 
 
+def test_extents_the_kernel_cannot_count_are_refused_before_any_gpu_call(lib, host_amd_handle):
+    """Heads, row steps and workgroups are counted in 32 bits: a descriptor beyond that (metadata only, nothing of
+    that size exists) is answered BAD_TENSOR_SHAPE at run time, before any device call."""
+    sp = qk_specs(Hq=(1 << 31) - 2, ntok=1, H=4, D=2, Dv=2, bs=1, NB=1)
+    status, op = create_qk(lib, host_amd_handle, sp)
+    assert status == OK
+    somewhere = ctypes.c_void_p(4096)  # never dereferenced
+    assert lib.LIBINFINIOP.infiniopRoPEQKPagedCaching(op, None, 0, *([somewhere] * 10), None) == BAD_SHAPE
+    lib.check_error(lib.LIBINFINIOP.infiniopDestroyRoPEPagedCachingDescriptor(op))
+
+
 # ---- the oracle function ------------------------------------------------------------------------------------
 
 def tables(table_len, D, dtype, theta=10000.0):

@@ -230,3 +230,16 @@ def test_tensor_descriptor_default_strides_are_packed(lib, host_amd_handle):
     assert status == OK
     lib.LIBINFINIOP.infiniopDestroyPagedCachingDescriptor(op)
     assert lib.LIBINFINIOP.infiniopCreateTensorDescriptor(None, 1, None, None, F16) == NULLP
+
+
+def test_paged_caching_refuses_extents_its_kernel_cannot_count_before_any_gpu_call(lib, host_amd_handle):
+    """The scatter kernel counts heads, row units and workgroups in 32 bits: a descriptor beyond that (descriptors are
+    metadata, nothing of that size exists) is answered BAD_TENSOR_SHAPE at run time, before any device call."""
+    big = 1 << 31
+    s = {"k_cache": Spec((1, big, 1, 2), BF16), "v_cache": Spec((1, big, 1, 2), BF16),
+         "k": Spec((1, big, 2), BF16), "v": Spec((1, big, 2), BF16), "slots": Spec((1,), I64)}
+    status, op = create_caching(lib, host_amd_handle, s)
+    assert status == OK
+    somewhere = ctypes.c_void_p(4096)  # never dereferenced
+    assert lib.LIBINFINIOP.infiniopPagedCaching(op, None, 0, *([somewhere] * 5), None) == BAD_SHAPE
+    assert lib.LIBINFINIOP.infiniopDestroyPagedCachingDescriptor(op) == OK
