@@ -26,7 +26,7 @@ using op::paged_attention::amd::IndexU32;
 // device memory and are never read on the host).
 struct Plan {
     bool tiled;          // matrix-core kernel (head 64 / 128 / 192 / 256, power-of-two pages >= 8, 16-byte aligned strides)
-    int groups_per_wave; // tiled: R = 1 or 2 column groups per wavefront -> 64 R rows per workgroup (heads above 128: always 1)
+    int groups_per_wave; // tiled: R = 1 or 2 column groups per wavefront -> 64 R rows per workgroup
     int dims_per_lane;   // element-wise kernel: ceil(max(head_size, value_size) / 64)
 };
 
@@ -53,13 +53,15 @@ Plan makePlan(const PagedAttentionPrefillInfo &in, const device::amd::DeviceInfo
             plan.tiled = false;
         }
     }
-    // Rows per workgroup: 128 (two column groups per wavefront; both sizes keep two workgroups per
-    // compute unit) unless the average sequence fills no more than 64, or the batch is too small to
-    // give every compute unit two workgroups of 128.
+    // Rows per workgroup: 128 (two column groups per wavefront: every K / V operand read from LDS then feeds two
+    // matrix instructions) unless the average sequence fills no more than 64, or the batch is too small to give
+    // every compute unit as many workgroups of 128 as it holds at a time: two up to head 128, one above (there the
+    // accumulators of 128 rows need more than half the register file).
     const long long seqs = in.num_seqs > 0 ? static_cast<long long>(in.num_seqs) : 1;
     const long long rows_per_seq = rows / seqs;
+    const long long resident = in.head_size <= 128 ? 2 : 1;
     int r = 2;
-    if (rows_per_seq <= 64 || rows / 128 * static_cast<long long>(in.num_kv_heads) < 2LL * dev.compute_units) {
+    if (rows_per_seq <= 64 || rows / 128 * static_cast<long long>(in.num_kv_heads) < resident * dev.compute_units) {
         r = 1;
     }
     if (const char *env = std::getenv("INFINIOP_AMD_PREFILL_GROUPS")) {
@@ -90,14 +92,12 @@ template <typename T, typename Tindex, int HEAD, bool PLAIN>
 void launchTiledHead(const PrefillArgs &a, const Plan &plan, hipStream_t stream) {
     // sum over sequences of ceil(rows / block_rows) is at most floor(total rows / block_rows) + num_seqs
     const long long rows = static_cast<long long>(a.total_q_tokens) * a.group;
-    const int groups = HEAD <= 128 ? plan.groups_per_wave : 1;
+    const int groups = plan.groups_per_wave;
     const int block_rows = prefillBlockRows(groups);
     const dim3 grid(static_cast<unsigned>((rows / block_rows + a.num_seqs) * a.num_kv_heads));
-    if constexpr (HEAD <= 128) {
-        if (groups == 2) {
-            prefillTiledKernel<T, Tindex, HEAD, 2, PLAIN><<<grid, kPrefillThreads, 0, stream>>>(a);
-            return;
-        }
+    if (groups == 2) {
+        prefillTiledKernel<T, Tindex, HEAD, 2, PLAIN><<<grid, kPrefillThreads, 0, stream>>>(a);
+        return;
     }
     prefillTiledKernel<T, Tindex, HEAD, 1, PLAIN><<<grid, kPrefillThreads, 0, stream>>>(a);
 }

@@ -124,19 +124,25 @@ __device__ __forceinline__ void loadStripCached(const char *first, uint32_t rest
     }
 }
 
-// Tokens per step: 64 for heads up to 128, 32 above (the two LDS buffers of K and V then stay within
-// 64 KiB and two workgroups share a compute unit).
-template <int HEAD>
-constexpr int prefillStepTokens() { return HEAD <= 128 ? 64 : 32; }
+// Tokens per step, and workgroups that share a compute unit. Up to head 128: 64 tokens, two workgroups. Head 256
+// needs more than half the register file even for 64 rows, so one workgroup has the unit to itself and takes 64-token
+// steps (its two K and two V buffers are 128 KiB of the 160). Head 192 fits two workgroups of 64 rows with 32-token
+// steps (48 KiB each); with 128 rows it is alone on the unit and takes 64-token steps (96 KiB).
+// At the Llama-3-8B chunked-prefill shape, 128 rows against 64 rows with 32-token steps: head 192 1 864 -> 1 692 us,
+// head 256 4 040 -> 2 046 us (2 787 us with 64 rows and 64-token steps).
+template <int HEAD, int R>
+constexpr int prefillStepTokens() { return (HEAD <= 128 || HEAD == 256 || R == 2) ? 64 : 32; }
+template <int HEAD, int R>
+constexpr int prefillWorkgroupsPerUnit() { return (HEAD <= 128 || (HEAD == 192 && R == 1)) ? 2 : 1; }
 
 // PLAIN: no ALiBi and scale > 0. The running maximum is then kept in units of the raw dot product
 // (a positive scale keeps the order) and each probability costs one fused multiply-add and one exp2.
 template <typename T, typename Tindex, int HEAD, int R, bool PLAIN>
-__global__ void __launch_bounds__(kPrefillThreads, HEAD <= 192 ? 2 : 1) prefillTiledKernel(PrefillArgs a) {
+__global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<HEAD, R>())) prefillTiledKernel(PrefillArgs a) {
     using S = typename T::storage;
     using G = TileGeometry<HEAD>;
     constexpr int BM = prefillBlockRows(R);
-    constexpr int BN = prefillStepTokens<HEAD>();
+    constexpr int BN = prefillStepTokens<HEAD, R>();
     constexpr int TT = BN / kTileTokens;             // 16-token tiles per step: 4 or 2
     constexpr int kTileChunks = kTileTokens * G::kChunksPerRow;
     __shared__ uint4 k_lds[2][TT * kTileChunks];       // [tile][token][16-byte chunk, XOR-swizzled by the token]

@@ -147,20 +147,23 @@ def test_element_wise_kernel_on_a_tiled_shape(gpu_handle, oracle, monkeypatch, d
     run_case(gpu_handle, oracle, workloads.make_prefill_inputs(cfg))
 
 
-@pytest.mark.parametrize("kernel", ["tiled", "generic"])
+@pytest.mark.parametrize("kernel", ["tiled-1", "tiled-2", "generic"])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("D", [64, 192, 256])
 def test_other_head_sizes(gpu_handle, oracle, monkeypatch, D, dtype, kernel):
-    """Head sizes 64 / 192 / 256 on the matrix-core kernel (steps of 32 tokens above 128) and on the element-wise one."""
+    """Head sizes 64 / 192 / 256 on the matrix-core kernel, 64 and 128 rows per workgroup (head 192 takes steps of 32
+    tokens with 64 rows and of 64 tokens with 128), and on the element-wise one."""
     if kernel == "generic":
         monkeypatch.setenv("INFINIOP_AMD_PREFILL_KERNEL", "generic")
+    else:
+        monkeypatch.setenv("INFINIOP_AMD_PREFILL_GROUPS", kernel[-1])
     small = kernel == "generic"
     cfg = prefill_config(f"head{D}_{kernel}", dtype, 4, 8, 4, D, 16, (1, 40 if small else 260), (0, 100 if small else 400),
                          seed=41 + D)
     run_case(gpu_handle, oracle, workloads.make_prefill_inputs(cfg))
 
 
-@pytest.mark.parametrize("D,groups", [(64, "1"), (64, "2"), (192, "1"), (256, "1")])
+@pytest.mark.parametrize("D,groups", [(64, "1"), (64, "2"), (192, "1"), (192, "2"), (256, "1"), (256, "2")])
 def test_other_head_sizes_pages_of_8_alibi_and_int32(gpu_handle, oracle, monkeypatch, D, groups):
     monkeypatch.setenv("INFINIOP_AMD_PREFILL_GROUPS", groups)
     cfg = prefill_config(f"mix{D}", torch.bfloat16, 3, 12, 2, D, 8, (1, 150), (0, 300), seed=91 + D)
@@ -168,10 +171,12 @@ def test_other_head_sizes_pages_of_8_alibi_and_int32(gpu_handle, oracle, monkeyp
     run_case(gpu_handle, oracle, workloads.make_prefill_inputs(cfg), alibi=slopes, index_dtype=torch.int32)
 
 
+@pytest.mark.parametrize("groups", ["1", "2"])
 @pytest.mark.parametrize("D", [64, 192, 256])
-def test_other_head_sizes_column_layout_and_garbage(gpu_handle, oracle, D):
+def test_other_head_sizes_column_layout_and_garbage(gpu_handle, oracle, monkeypatch, D, groups):
     """V with a distinct constant per column makes the expected output that constant (every output column
     lands where it belongs); NaN beyond the sequences must not leak in."""
+    monkeypatch.setenv("INFINIOP_AMD_PREFILL_GROUPS", groups)
     cfg = prefill_config(f"cols{D}", torch.float16, 3, 8, 2, D, 16, (5, 90), (3, 200), seed=97 + D)
     inp = workloads.make_prefill_inputs(cfg)
     ramp = ((torch.arange(D, dtype=torch.float32) - D / 2) / 8).to(torch.float16)
