@@ -298,9 +298,9 @@ __device__ __forceinline__ void softmaxStepPair(f32x4 (&o)[COLS], float &m, floa
             sc[i] = (16 * (i >> 2) + 4 * g + (i & 3) >= valid) ? -INFINITY : sc[i];
         }
     }
-    const float mx = maxAcrossTokenGroups(fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])),
-                                                fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7]))));
-    const float m_new = fmaxf(m, mx);
+    const float mx = maxAcrossTokenGroups(maxOf(maxOf(maxOf(sc[0], sc[1]), maxOf(sc[2], sc[3])),
+                                                maxOf(maxOf(sc[4], sc[5]), maxOf(sc[6], sc[7]))));
+    const float m_new = maxOf(m, mx);
     if (__builtin_amdgcn_ballot_w64(mx > m + kLazyRescaleLog2) != 0) {
         // rescale (see softmaxStep). Lane holds accumulators of heads 4g..4g+3, whose factors live in
         // lanes 4g..4g+3.

@@ -43,6 +43,7 @@ namespace op::paged_attention_prefill::amd {
 
 using op::paged_attention::amd::f32x4;
 using op::paged_attention::amd::maxAcrossTokenGroups;
+using op::paged_attention::amd::maxOf;
 using op::paged_attention::amd::sumAcrossTokenGroups;
 using op::paged_attention::amd::TileBF16;
 using op::paged_attention::amd::TileF16;
@@ -53,6 +54,10 @@ using op::paged_attention::amd::storeStrip;
 using op::paged_attention::amd::TileGeometry;
 
 constexpr int kPrefillThreads = 256;
+// K / V operands are requested from LDS this many uses before the matrix instructions that take them (an LDS read
+// takes longer than the R instructions one operand feeds; left alone the compiler requests one or two ahead and
+// the matrix unit waits). Eight ahead is no better where the registers allow it (heads above 128).
+constexpr int kOperandsAhead = 4;
 constexpr float kLazyLog2 = 8.0f; // how far (in powers of two) a row maximum may outgrow its reference point
 
 // 16-byte load from (wave-uniform base) + (32-bit per-lane byte offset), through the caches: K/V tiles
@@ -361,19 +366,34 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<HEA
                 s[r][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
             }
         }
+        // K.Q^T: operand idx = (tile tt, 32 dimensions kk). The scheduler groups pin the order "one LDS read, then the
+        // R matrix instructions of the operand read kAheadK earlier"; the first kAheadK reads are a group of their own.
+        {
+            constexpr int kAheadK = kOperandsAhead;
+            constexpr int kOperandsK = TT * G::kLoads;
+            auto readK = [&](int idx) {
+                const int tt = idx / G::kLoads, kk = idx % G::kLoads;
+                return k_lds[buf][tt * kTileChunks + G::ldsIndex(c, 4 * kk + g)];
+            };
+            uint4 kf[kAheadK];
 #pragma unroll
-        for (int tt = 0; tt < TT; ++tt) {
-            uint4 kf[G::kLoads];
-#pragma unroll
-            for (int kk = 0; kk < G::kLoads; ++kk) {
-                kf[kk] = k_lds[buf][tt * kTileChunks + G::ldsIndex(c, 4 * kk + g)];
+            for (int i = 0; i < kAheadK; ++i) {
+                kf[i] = readK(i);
             }
+            __builtin_amdgcn_sched_group_barrier(0x100, kAheadK, 0);
 #pragma unroll
-            for (int kk = 0; kk < G::kLoads; ++kk) {
+            for (int idx = 0; idx < kOperandsK; ++idx) {
+                const int tt = idx / G::kLoads, kk = idx % G::kLoads;
+                const uint4 cur = kf[idx % kAheadK];
+                if (idx + kAheadK < kOperandsK) {
+                    kf[idx % kAheadK] = readK(idx + kAheadK);
+                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                }
 #pragma unroll
                 for (int r = 0; r < R; ++r) {
-                    s[r][tt] = T::mfmaK32(kf[kk], q_reg[r][kk], s[r][tt]);
+                    s[r][tt] = T::mfmaK32(cur, q_reg[r][kk], s[r][tt]);
                 }
+                __builtin_amdgcn_sched_group_barrier(0x008, R, 0);
             }
         }
 
@@ -401,13 +421,13 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<HEA
                     }
                 }
             }
-            float mx = fmaxf(fmaxf(s[r][0][0], s[r][0][1]), fmaxf(s[r][0][2], s[r][0][3]));
+            float mx = maxOf(maxOf(s[r][0][0], s[r][0][1]), maxOf(s[r][0][2], s[r][0][3]));
 #pragma unroll
             for (int tt = 1; tt < TT; ++tt) {
-                mx = fmaxf(mx, fmaxf(fmaxf(s[r][tt][0], s[r][tt][1]), fmaxf(s[r][tt][2], s[r][tt][3])));
+                mx = maxOf(mx, maxOf(maxOf(s[r][tt][0], s[r][tt][1]), maxOf(s[r][tt][2], s[r][tt][3])));
             }
             mx = maxAcrossTokenGroups(mx);
-            const float m_new = fmaxf(m[r], mx);
+            const float m_new = maxOf(m[r], mx);
             // The reference point m[r] only has to keep the exponentials in range, it need not be the
             // exact maximum: it is moved (and the accumulators rescaled, ~70 vector instructions) only
             // when some row's maximum has grown by more than 2^kLazyLog2 since, so probabilities reach at
@@ -442,22 +462,41 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<HEA
             }
         }
 
+        // P.V: the V operands run kAhead ahead as well
+        constexpr int kAhead = kOperandsAhead;
+        constexpr int kOperands = (TT / 2) * G::kCols;
+        auto readV = [&](int idx) {
+            const int u = idx / G::kCols, e = idx % G::kCols;
+            const uint2 lo = v_lds[buf][((e * TT + 2 * u) * 4 + g) * 16 + c];
+            const uint2 hi = v_lds[buf][((e * TT + 2 * u + 1) * 4 + g) * 16 + c];
+            return make_uint4(lo.x, lo.y, hi.x, hi.y);
+        };
+        uint4 vf[kAhead];
 #pragma unroll
-        for (int u = 0; u < TT / 2; ++u) {
+        for (int i = 0; i < kAhead; ++i) {
+            vf[i] = readV(i);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 0);
 #pragma unroll
-            for (int r = 0; r < R; ++r) {
-                ol[r] = T::mfmaK32(p_op[r][u], ones, ol[r]);
+        for (int idx = 0; idx < kOperands; ++idx) {
+            const int u = idx / G::kCols, e = idx % G::kCols;
+            const uint4 cur = vf[idx % kAhead];
+            if (idx + kAhead < kOperands) {
+                vf[idx % kAhead] = readV(idx + kAhead);
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
             }
-#pragma unroll
-            for (int e = 0; e < G::kCols; ++e) {
-                const uint2 lo = v_lds[buf][((e * TT + 2 * u) * 4 + g) * 16 + c];
-                const uint2 hi = v_lds[buf][((e * TT + 2 * u + 1) * 4 + g) * 16 + c];
-                const uint4 vf = make_uint4(lo.x, lo.y, hi.x, hi.y);
+            if (e == 0) {
 #pragma unroll
                 for (int r = 0; r < R; ++r) {
-                    o[r][e] = T::mfmaK32(p_op[r][u], vf, o[r][e]);
+                    ol[r] = T::mfmaK32(p_op[r][u], ones, ol[r]);
                 }
+                __builtin_amdgcn_sched_group_barrier(0x008, R, 0);
             }
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                o[r][e] = T::mfmaK32(p_op[r][u], cur, o[r][e]);
+            }
+            __builtin_amdgcn_sched_group_barrier(0x008, R, 0);
         }
     };
 
