@@ -271,6 +271,14 @@ __global__ void __launch_bounds__(kMlaThreads, 2) decodeMlaKernel(DecodeArgs a) 
 // Partial results and their merge are those of the kernel above.
 constexpr int kMlaWideThreads = 512;
 constexpr int kMlaWideTileTokens = 32; // two halves of 16
+// K / V operands of the wide kernel are requested from LDS this many matrix instructions before the one that takes
+// them: every operand feeds a single instruction (16 clocks) and an LDS read takes several times that.
+constexpr int kMlaOperandsAhead = 6;
+// The wide kernels feed the probabilities to P.V as one term in the storage dtype, as the prefill kernel does. They
+// are bound by instruction issue, not by memory, and the second term that the other decode kernels add for bf16
+// (decode_tiled.h: p = hi + lo) costs 16 more matrix and ~50 more vector instructions per wavefront and tile while the
+// largest error against the fp32 oracle at the 128-head shape moves from 0.96e-3 to 1.01e-3 (77 -> 73 us per call).
+constexpr bool kMlaWideSplitProbabilities = false;
 
 // Online-softmax step of one 32-token tile. s0 / s1 = raw scores of head c for tokens 4g..4g+3 of the
 // first / second half; the rest as softmaxStep (decode_tiled.h). The probabilities come back as the A
@@ -323,7 +331,7 @@ __device__ __forceinline__ void softmaxStepPair(f32x4 (&o)[COLS], float &m, floa
         const float pa = fastExp2(sc[2 * i] - m), pb = fastExp2(sc[2 * i + 1] - m);
         hi[i] = T::pack2(pa, pb);
         p_used += T::unpackLo(hi[i]) + T::unpackHi(hi[i]);
-        if constexpr (T::kSplitProbabilities) {
+        if constexpr (T::kSplitProbabilities && kMlaWideSplitProbabilities) {
             lo[i] = T::pack2(pa - T::unpackLo(hi[i]), pb - T::unpackHi(hi[i]));
             p_used += T::unpackLo(lo[i]) + T::unpackHi(lo[i]);
         }
@@ -667,11 +675,24 @@ __global__ void __launch_bounds__(kMlaWideThreads, 2) decodeMlaWideKernel(Decode
             // matrix instruction that accumulates into the result of the previous one waits ~44 cycles
             // for it, an independent one issues after 16)
             f32x4 sp[2][2] = {{{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}}, {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}}};
+            // operand idx = (K-step idx / 2, token half idx % 2), requested kMlaOperandsAhead uses ahead
+            constexpr int kOperands = 2 * kOwnSteps;
+            auto readK = [&](int idx) { return k_lds[buf][(16 * (idx & 1) + c) * kPitch + 4 * (first_step + (idx >> 1)) + g]; };
+            uint4 kf[kOperands];
 #pragma unroll
-            for (int i = 0; i < kOwnSteps; ++i) {
-                const int kk = first_step + i;
-                sp[0][i & 1] = T::mfmaK32(k_lds[buf][c * kPitch + 4 * kk + g], q_reg[i], sp[0][i & 1]);
-                sp[1][i & 1] = T::mfmaK32(k_lds[buf][(16 + c) * kPitch + 4 * kk + g], q_reg[i], sp[1][i & 1]);
+            for (int idx = 0; idx < kMlaOperandsAhead; ++idx) {
+                kf[idx] = readK(idx);
+            }
+            __builtin_amdgcn_sched_group_barrier(0x100, kMlaOperandsAhead, 0);
+#pragma unroll
+            for (int idx = 0; idx < kOperands; ++idx) {
+                if (idx + kMlaOperandsAhead < kOperands) {
+                    kf[idx + kMlaOperandsAhead] = readK(idx + kMlaOperandsAhead);
+                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                }
+                const int i = idx >> 1;
+                sp[idx & 1][i & 1] = T::mfmaK32(kf[idx], q_reg[i], sp[idx & 1][i & 1]);
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
             }
             s0 = sp[0][0] + sp[0][1], s1 = sp[1][0] + sp[1][1];
             s_lds[wave][0][lane] = s0;
@@ -682,10 +703,22 @@ __global__ void __launch_bounds__(kMlaWideThreads, 2) decodeMlaWideKernel(Decode
         } else {
             // partial scores of this wavefront's token half over its quarter of the K-steps
             f32x4 sp[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+            auto readK = [&](int i) { return k_lds[buf][(16 * th + c) * kPitch + 4 * min(first_step + i, kSteps - 1) + g]; };
+            constexpr int kAheadOne = kOwnSteps < kMlaOperandsAhead ? kOwnSteps : kMlaOperandsAhead;
+            uint4 kf[kOwnSteps];
+#pragma unroll
+            for (int i = 0; i < kAheadOne; ++i) {
+                kf[i] = readK(i);
+            }
+            __builtin_amdgcn_sched_group_barrier(0x100, kAheadOne, 0);
 #pragma unroll
             for (int i = 0; i < kOwnSteps; ++i) {
-                const int kk = min(first_step + i, kSteps - 1);
-                sp[i & 1] = T::mfmaK32(k_lds[buf][(16 * th + c) * kPitch + 4 * kk + g], q_reg[i], sp[i & 1]);
+                if (i + kAheadOne < kOwnSteps) {
+                    kf[i + kAheadOne] = readK(i + kAheadOne);
+                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                }
+                sp[i & 1] = T::mfmaK32(kf[i], q_reg[i], sp[i & 1]);
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
             }
             s_lds[wave][0][lane] = sp[0] + sp[1];
             __syncthreads(); // all eight partial tiles are there: wavefront 2 q + h holds quarter q of half h
@@ -697,25 +730,32 @@ __global__ void __launch_bounds__(kMlaWideThreads, 2) decodeMlaWideKernel(Decode
         const int valid = min(kMlaWideTileTokens, end - tok0);
         uint4 p_op, p_lo;
         softmaxStepPair<T, kOwnBlocks>(o, m, l, s0, s1, g, a.scale_log2, slope, tok0 - (len - 1), valid, p_op, p_lo);
-        // column blocks four at a time: their V operands from LDS, the high parts of the probabilities, then
-        // the low parts (four independent chains - a matrix instruction that accumulates into the result of the
-        // one before waits for it); all blocks at once kept 64 registers of operands alive
-        constexpr int kGroup = 4;
+        // P.V one column block after the other, its V operand requested from LDS kMlaOperandsAhead blocks ahead;
+        // the low parts of the probabilities follow two blocks behind the high parts (a matrix instruction that
+        // accumulates into the result of the one before waits for it)
+        constexpr int kAheadV = kOwnBlocks < kMlaOperandsAhead ? kOwnBlocks : kMlaOperandsAhead;
+        constexpr int kSkew = 2; // the low part of block e goes kSkew blocks behind its high part
+        auto readV = [&](int e) { return v_lds[buf][((first_block + e) * 4 + g) * 16 + c]; };
+        uint4 vf[kOwnBlocks];
 #pragma unroll
-        for (int e0 = 0; e0 < kOwnBlocks; e0 += kGroup) {
-            uint4 vf[kGroup];
+        for (int e = 0; e < kAheadV; ++e) {
+            vf[e] = readV(e);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x100, kAheadV, 0);
 #pragma unroll
-            for (int e = 0; e < kGroup; ++e) {
-                vf[e] = v_lds[buf][((first_block + e0 + e) * 4 + g) * 16 + c];
+        for (int e = 0; e < kOwnBlocks + kSkew; ++e) {
+            if (e + kAheadV < kOwnBlocks) {
+                vf[e + kAheadV] = readV(e + kAheadV);
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
             }
-#pragma unroll
-            for (int e = 0; e < kGroup; ++e) {
-                o[e0 + e] = T::mfmaK32(p_op, vf[e], o[e0 + e]);
+            if (e < kOwnBlocks) {
+                o[e] = T::mfmaK32(p_op, vf[e], o[e]);
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
             }
-            if constexpr (T::kSplitProbabilities) {
-#pragma unroll
-                for (int e = 0; e < kGroup; ++e) {
-                    o[e0 + e] = T::mfmaK32(p_lo, vf[e], o[e0 + e]);
+            if constexpr (T::kSplitProbabilities && kMlaWideSplitProbabilities) {
+                if (e >= kSkew) {
+                    o[e - kSkew] = T::mfmaK32(p_lo, vf[e - kSkew], o[e - kSkew]);
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
                 }
             }
         }
