@@ -56,8 +56,11 @@ using op::paged_attention::amd::TileGeometry;
 constexpr int kPrefillThreads = 256;
 // K / V operands are requested from LDS this many uses before the matrix instructions that take them (an LDS read
 // takes longer than the R instructions one operand feeds; left alone the compiler requests one or two ahead and
-// the matrix unit waits). Eight ahead is no better where the registers allow it (heads above 128).
-constexpr int kOperandsAhead = 4;
+// the matrix unit waits). At the Llama-3-8B chunked-prefill shape, head 128, two to six ahead are within 3 % of each
+// other (600 - 620 us, run-to-run spread 1.5 %) against 639 us left to the compiler; above head 128, where the
+// registers allow more, 8 is no better than 4.
+template <int HEAD>
+constexpr int prefillOperandsAhead() { return HEAD <= 128 ? 3 : 4; }
 constexpr float kLazyLog2 = 8.0f; // how far (in powers of two) a row maximum may outgrow its reference point
 
 // 16-byte load from (wave-uniform base) + (32-bit per-lane byte offset), through the caches: K/V tiles
@@ -369,7 +372,7 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<HEA
         // K.Q^T: operand idx = (tile tt, 32 dimensions kk). The scheduler groups pin the order "one LDS read, then the
         // R matrix instructions of the operand read kAheadK earlier"; the first kAheadK reads are a group of their own.
         {
-            constexpr int kAheadK = kOperandsAhead;
+            constexpr int kAheadK = prefillOperandsAhead<HEAD>();
             constexpr int kOperandsK = TT * G::kLoads;
             auto readK = [&](int idx) {
                 const int tt = idx / G::kLoads, kk = idx % G::kLoads;
@@ -463,7 +466,7 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<HEA
         }
 
         // P.V: the V operands run kAhead ahead as well
-        constexpr int kAhead = kOperandsAhead;
+        constexpr int kAhead = prefillOperandsAhead<HEAD>();
         constexpr int kOperands = (TT / 2) * G::kCols;
         auto readV = [&](int idx) {
             const int u = idx / G::kCols, e = idx % G::kCols;
