@@ -71,6 +71,14 @@ __device__ __forceinline__ uint4 loadLane16Cached(const char *uniform_base, uint
     return *reinterpret_cast<const uint4 *>(uniform_base + lane_offset);
 }
 
+// 16 bytes per lane from global memory straight into LDS, without a register in between: lane i of the wavefront
+// writes the 16 bytes at lds_base + 16 i (lds_base is the same for all lanes); lanes that are switched off write
+// nothing. The data is in LDS when the wavefront's vector-memory counter has counted the instruction off.
+__device__ __forceinline__ void loadLane16ToLds(const char *global_src, uint4 *lds_base) {
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)global_src,
+                                     (__attribute__((address_space(3))) void *)lds_base, 16, 0, 0);
+}
+
 // Rows of one workgroup for R column groups per wavefront.
 __host__ __device__ constexpr int prefillBlockRows(int r) { return 64 * r; }
 
@@ -251,10 +259,19 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<HEA
     // byte offsets of this lane's pieces inside a 16-token tile (pages >= 16 tokens)
     const LaneOffsets<HEAD> off(lane, static_cast<uint32_t>(a.k_row_stride) * sizeof(S),
                                 static_cast<uint32_t>(a.v_row_stride) * sizeof(S));
-    uint4 k_stage[G::kLoads];
+    // K goes from global memory straight into its place in LDS: slot 64 j + lane of the tile holds chunk
+    // (slot % chunks per row) ^ swizzle(row) of row slot / chunks per row (TileGeometry::ldsIndex read backwards), so
+    // that is the chunk this lane asks for with instruction j. V passes through registers (it is transposed on
+    // the way).
+    uint32_t k_src_off[G::kLoads];
+#pragma unroll
+    for (int j = 0; j < G::kLoads; ++j) {
+        const int row = G::kRow(j, lane), slot = G::kChunk(j, lane);
+        k_src_off[j] = row * static_cast<uint32_t>(a.k_row_stride) * sizeof(S) + 16 * (slot ^ (row & (G::kSwizzle - 1)));
+    }
     uint32_t v_stage[4][G::kWords];
     auto loadStage = [&](int step) {
-        // K: flat chunks 64 j + lane of the tile; V: rows 4 g + i. Tokens past kv_len are not fetched.
+        // K: slots 64 j + lane of the tile; V: rows 4 g + i, tokens past kv_len zeroed.
         const int t = step * BN + kTileTokens * copy_tile;
         const int e0 = t >> a.block_shift;
         if ((min(e0, last_entry) >> 6) > id_batch) {
@@ -262,24 +279,43 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<HEA
             ++id_batch;
             ids_next = loadIdBatch(id_batch + 1);
         }
-        if (t + kTileTokens <= kv_len && !small_pages) {
-            const int page = pageOfEntry(e0);
-            const int row0 = t & block_mask;
-            if (copies_k) {
-                const char *k_tile = k_head + (page * a.k_batch_stride + row0 * a.k_row_stride) * static_cast<int64_t>(sizeof(S));
+        if (copies_k) {
+            // Rows past the end of the sequence are fetched like the others: the page they lie in exists (its id
+            // is clamped to the sequence's last entry and to the pool), and whatever they hold only reaches scores
+            // that the causal mask replaces.
+            uint4 *k_dst = &k_lds[step & 1][copy_tile * kTileChunks];
+            if (!small_pages) {
+                const int page = pageOfEntry(e0);
+                const char *k_tile = k_head + (page * a.k_batch_stride + (t & block_mask) * a.k_row_stride) * static_cast<int64_t>(sizeof(S));
 #pragma unroll
                 for (int j = 0; j < G::kLoads; ++j) {
-                    k_stage[j] = loadLane16Cached(k_tile, off.k[j]);
+                    uint32_t lane_off = k_src_off[j];
+                    asm volatile("" : "+v"(lane_off));
+                    loadLane16ToLds(k_tile + lane_off, k_dst + 64 * j);
+                }
+            } else { // pages of 8 tokens: rows 8..15 of the tile lie in the next page
+                const int id0 = pageOfEntry(e0), id1 = pageOfEntry(e0 + 1);
+#pragma unroll
+                for (int j = 0; j < G::kLoads; ++j) {
+                    const int row = G::kRow(j, lane), slot = G::kChunk(j, lane);
+                    const int page = row >= 8 ? id1 : id0;
+                    const char *src = k_head + (page * a.k_batch_stride + (row & 7) * a.k_row_stride) * static_cast<int64_t>(sizeof(S))
+                                    + 16 * (slot ^ (row & (G::kSwizzle - 1)));
+                    loadLane16ToLds(src, k_dst + 64 * j);
                 }
             }
-            if (copies_v) {
-                const char *v_tile = v_head + (page * a.v_batch_stride + row0 * a.v_row_stride) * static_cast<int64_t>(sizeof(S));
+        }
+        if (!copies_v) {
+            return;
+        }
+        if (t + kTileTokens <= kv_len && !small_pages) {
+            const int page = pageOfEntry(e0);
+            const char *v_tile = v_head + (page * a.v_batch_stride + (t & block_mask) * a.v_row_stride) * static_cast<int64_t>(sizeof(S));
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    uint32_t lane_off = off.v[j];
-                    asm volatile("" : "+v"(lane_off));
-                    loadStripCached<HEAD>(v_tile + lane_off, off.v_rest, v_stage[j]);
-                }
+            for (int j = 0; j < 4; ++j) {
+                uint32_t lane_off = off.v[j];
+                asm volatile("" : "+v"(lane_off));
+                loadStripCached<HEAD>(v_tile + lane_off, off.v_rest, v_stage[j]);
             }
             return;
         }
@@ -287,43 +323,25 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<HEA
         const int id0 = t < kv_len ? pageOfEntry(e0) : 0;
         const int id1 = (small_pages && t < kv_len) ? pageOfEntry(e0 + 1) : id0;
         const int row0 = small_pages ? 0 : (t & block_mask);
-        if (copies_k) {
 #pragma unroll
-            for (int j = 0; j < G::kLoads; ++j) {
-                const int o = G::kRow(j, lane);
-                const int page = (small_pages && o >= 8) ? id1 : id0;
-                const int page_row = small_pages ? (o & 7) : row0 + o;
-                const char *src = k_head + (page * a.k_batch_stride + page_row * a.k_row_stride) * static_cast<int64_t>(sizeof(S))
-                                + 16 * G::kChunk(j, lane);
-                k_stage[j] = (t + o < kv_len) ? *reinterpret_cast<const uint4 *>(src) : make_uint4(0, 0, 0, 0);
-            }
-        }
-        if (copies_v) {
+        for (int i = 0; i < 4; ++i) {
+            const int o = 4 * g + i;
+            const int page = (small_pages && g >= 2) ? id1 : id0;
+            const int page_row = small_pages ? (o & 7) : row0 + o;
+            const char *src = v_head + (page * a.v_batch_stride + page_row * a.v_row_stride) * static_cast<int64_t>(sizeof(S))
+                            + 2 * G::firstColumn(c);
+            if (t + o < kv_len) {
+                loadStripCached<HEAD>(src, off.v_rest, v_stage[i]);
+            } else {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int o = 4 * g + i;
-                const int page = (small_pages && g >= 2) ? id1 : id0;
-                const int page_row = small_pages ? (o & 7) : row0 + o;
-                const char *src = v_head + (page * a.v_batch_stride + page_row * a.v_row_stride) * static_cast<int64_t>(sizeof(S))
-                                + 2 * G::firstColumn(c);
-                if (t + o < kv_len) {
-                    loadStripCached<HEAD>(src, off.v_rest, v_stage[i]);
-                } else {
-#pragma unroll
-                    for (int wd = 0; wd < G::kWords; ++wd) {
-                        v_stage[i][wd] = 0u;
-                    }
+                for (int wd = 0; wd < G::kWords; ++wd) {
+                    v_stage[i][wd] = 0u;
                 }
             }
         }
     };
+    // V of the stage loaded last: registers -> LDS; K of that stage: wait until it has arrived
     auto storeStage = [&](int buf) {
-        if (copies_k) {
-#pragma unroll
-            for (int j = 0; j < G::kLoads; ++j) {
-                k_lds[buf][copy_tile * kTileChunks + G::ldsIndex(G::kRow(j, lane), G::kChunk(j, lane))] = k_stage[j];
-            }
-        }
         if (copies_v) {
 #pragma unroll
             for (int wd = 0; wd < G::kWords; ++wd) {
@@ -335,6 +353,9 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<HEA
                 v_lds[buf][(((2 * wd) * TT + copy_tile) * 4 + g) * 16 + c] = even;
                 v_lds[buf][(((2 * wd + 1) * TT + copy_tile) * 4 + g) * 16 + c] = odd;
             }
+        }
+        if (copies_k) {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // the K tile asked for by loadStage is in LDS
         }
     };
 
