@@ -162,7 +162,11 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<HEA
     constexpr int TT = BN / kTileTokens;             // 16-token tiles per step: 4 or 2
     constexpr int kTileChunks = kTileTokens * G::kChunksPerRow;
     __shared__ uint4 k_lds[2][TT * kTileChunks];       // [tile][token][16-byte chunk, XOR-swizzled by the token]
-    __shared__ uint2 v_lds[2][G::kCols * TT * 64];     // [column e][tile][token group g][strip c]
+    // V tile in LDS: [row half (8 rows)][block of 16 columns (32 bytes)][row of the half][two 16-byte chunks], i.e.
+    // slot = half * 8 * chunks per row + block * 16 + (row % 8) * 2 + chunk % 2. A transposing read of one block then
+    // touches two runs of 256 bytes, and 64 consecutive slots (one load instruction) are four blocks of eight rows:
+    // 128 contiguous bytes of each row in global memory.
+    __shared__ uint4 v_lds[2][TT * kTileChunks];
 
     const int lane = threadIdx.x & 63;
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -269,9 +273,16 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<HEA
         const int row = G::kRow(j, lane), slot = G::kChunk(j, lane);
         k_src_off[j] = row * static_cast<uint32_t>(a.k_row_stride) * sizeof(S) + 16 * (slot ^ (row & (G::kSwizzle - 1)));
     }
-    uint32_t v_stage[4][G::kWords];
+    // V likewise, into the layout described at v_lds
+    auto vRowOfSlot = [](int slot) { return 8 * (slot / (8 * G::kChunksPerRow)) + (slot % 16) / 2; };
+    auto vChunkOfSlot = [](int slot) { return 2 * ((slot % (8 * G::kChunksPerRow)) / 16) + slot % 2; };
+    uint32_t v_src_off[G::kLoads];
+#pragma unroll
+    for (int j = 0; j < G::kLoads; ++j) {
+        v_src_off[j] = vRowOfSlot(64 * j + lane) * static_cast<uint32_t>(a.v_row_stride) * sizeof(S) + 16 * vChunkOfSlot(64 * j + lane);
+    }
     auto loadStage = [&](int step) {
-        // K: slots 64 j + lane of the tile; V: rows 4 g + i, tokens past kv_len zeroed.
+        // K and V: slots 64 j + lane of the tile; V rows past kv_len are zeroed.
         const int t = step * BN + kTileTokens * copy_tile;
         const int e0 = t >> a.block_shift;
         if ((min(e0, last_entry) >> 6) > id_batch) {
@@ -308,59 +319,41 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<HEA
         if (!copies_v) {
             return;
         }
+        uint4 *v_dst = &v_lds[step & 1][copy_tile * kTileChunks];
         if (t + kTileTokens <= kv_len && !small_pages) {
             const int page = pageOfEntry(e0);
             const char *v_tile = v_head + (page * a.v_batch_stride + (t & block_mask) * a.v_row_stride) * static_cast<int64_t>(sizeof(S));
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                uint32_t lane_off = off.v[j];
+            for (int j = 0; j < G::kLoads; ++j) {
+                uint32_t lane_off = v_src_off[j];
                 asm volatile("" : "+v"(lane_off));
-                loadStripCached<HEAD>(v_tile + lane_off, off.v_rest, v_stage[j]);
+                loadLane16ToLds(v_tile + lane_off, v_dst + 64 * j);
             }
             return;
         }
-        // last tile of the sequence, or two pages per tile
-        const int id0 = t < kv_len ? pageOfEntry(e0) : 0;
-        const int id1 = (small_pages && t < kv_len) ? pageOfEntry(e0 + 1) : id0;
+        // Last tile of the sequence, or two pages per tile. Rows past the sequence may hold anything (NaN included)
+        // and 0 * NaN is NaN: their lanes are switched off for the load and store zeros instead.
+        const int id0 = pageOfEntry(e0), id1 = small_pages ? pageOfEntry(e0 + 1) : id0;
         const int row0 = small_pages ? 0 : (t & block_mask);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int o = 4 * g + i;
-            const int page = (small_pages && g >= 2) ? id1 : id0;
-            const int page_row = small_pages ? (o & 7) : row0 + o;
+        for (int j = 0; j < G::kLoads; ++j) {
+            const int row = vRowOfSlot(64 * j + lane);
+            const int page = (small_pages && row >= 8) ? id1 : id0;
+            const int page_row = small_pages ? (row & 7) : row0 + row;
             const char *src = v_head + (page * a.v_batch_stride + page_row * a.v_row_stride) * static_cast<int64_t>(sizeof(S))
-                            + 2 * G::firstColumn(c);
-            if (t + o < kv_len) {
-                loadStripCached<HEAD>(src, off.v_rest, v_stage[i]);
+                            + 16 * vChunkOfSlot(64 * j + lane);
+            if (t + row < kv_len) {
+                loadLane16ToLds(src, v_dst + 64 * j);
             } else {
-#pragma unroll
-                for (int wd = 0; wd < G::kWords; ++wd) {
-                    v_stage[i][wd] = 0u;
-                }
+                v_dst[64 * j + lane] = make_uint4(0, 0, 0, 0);
             }
         }
     };
-    // V of the stage loaded last: registers -> LDS; K of that stage: wait until it has arrived
-    auto storeStage = [&](int buf) {
-        if (copies_v) {
-#pragma unroll
-            for (int wd = 0; wd < G::kWords; ++wd) {
-                uint2 even, odd;
-                even.x = __builtin_amdgcn_perm(v_stage[1][wd], v_stage[0][wd], 0x05040100u);
-                even.y = __builtin_amdgcn_perm(v_stage[3][wd], v_stage[2][wd], 0x05040100u);
-                odd.x = __builtin_amdgcn_perm(v_stage[1][wd], v_stage[0][wd], 0x07060302u);
-                odd.y = __builtin_amdgcn_perm(v_stage[3][wd], v_stage[2][wd], 0x07060302u);
-                v_lds[buf][(((2 * wd) * TT + copy_tile) * 4 + g) * 16 + c] = even;
-                v_lds[buf][(((2 * wd + 1) * TT + copy_tile) * 4 + g) * 16 + c] = odd;
-            }
-        }
-        if (copies_k) {
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // the K tile asked for by loadStage is in LDS
-        }
-    };
+    // the tiles asked for by the last loadStage are in LDS
+    auto awaitStage = [&]() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); };
 
     // ---- softmax state ----
-    // o[r][e][rr] = O[row 4g+rr of group r][column e of strip c]; ol[r][rr] = sum of that row's probabilities
+    // o[r][e][rr] = O[row 4g+rr of group r][column 16 e + c]; ol[r][rr] = sum of that row's probabilities
     // (computed by the matrix unit as P . 1, so it sums exactly the rounded probabilities the numerator
     // used and already sits in the accumulators' row layout); m[r] = running maximum of row c, in units
     // of the raw dot product when there is no ALiBi (scale > 0 keeps the order), else of the scaled score.
@@ -375,6 +368,11 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<HEA
         ol[r] = f32x4{0.f, 0.f, 0.f, 0.f};
         m[r] = -INFINITY;
     }
+    // this lane's piece of a transposing V read (see readV below), relative to block 0 of tile 0 of buffer 0
+    typedef short s16x4 __attribute__((ext_vector_type(4)));
+    typedef __attribute__((address_space(3))) s16x4 *LdsPiece;
+    const auto v_read_base = (__attribute__((address_space(3))) char *)v_lds
+                           + 16 * ((g >> 1) * 8 * G::kChunksPerRow + (4 * (g & 1) + (c >> 2)) * 2 + ((c & 3) >> 1)) + 8 * (c & 1);
     const uint32_t one2 = T::pack2(1.0f, 1.0f);
     const uint4 ones = make_uint4(one2, one2, one2, one2);
     const float unit = PLAIN ? a.scale_log2 : 1.0f; // log2-domain size of one unit of m
@@ -489,10 +487,15 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<HEA
         // P.V: the V operands run kAhead ahead as well
         constexpr int kAhead = prefillOperandsAhead<HEAD>();
         constexpr int kOperands = (TT / 2) * G::kCols;
+        // Operand (u, e) = V[32 tokens of tiles 2u, 2u + 1][columns 16 e .. 16 e + 15]: lane (g, c) needs tokens
+        // 4g..4g+3 of either tile at column 16 e + c. A transposing read hands lane c of a group of 16 the element
+        // c % 4 of the four 8-byte pieces that lanes c / 4, c / 4 + 4, + 8, + 12 of the group point at; so lane
+        // (g, c) points at token 4g + c / 4, columns 16 e + 4 (c % 4) .. + 3.
         auto readV = [&](int idx) {
             const int u = idx / G::kCols, e = idx % G::kCols;
-            const uint2 lo = v_lds[buf][((e * TT + 2 * u) * 4 + g) * 16 + c];
-            const uint2 hi = v_lds[buf][((e * TT + 2 * u + 1) * 4 + g) * 16 + c];
+            const auto base = v_read_base + (buf * TT + 2 * u) * (kTileChunks * 16) + 256 * e;
+            const uint2 lo = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<LdsPiece>(base)));
+            const uint2 hi = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<LdsPiece>(base + kTileChunks * 16)));
             return make_uint4(lo.x, lo.y, hi.x, hi.y);
         };
         uint4 vf[kAhead];
@@ -500,14 +503,14 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<HEA
         for (int i = 0; i < kAhead; ++i) {
             vf[i] = readV(i);
         }
-        __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 2 * kAhead, 0); // two reads per operand
 #pragma unroll
         for (int idx = 0; idx < kOperands; ++idx) {
             const int u = idx / G::kCols, e = idx % G::kCols;
             const uint4 cur = vf[idx % kAhead];
             if (idx + kAhead < kOperands) {
                 vf[idx % kAhead] = readV(idx + kAhead);
-                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
             }
             if (e == 0) {
 #pragma unroll
@@ -526,7 +529,7 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<HEA
 
     // ---- pipeline ----
     loadStage(0);
-    storeStage(0);
+    awaitStage();
     __syncthreads();
     if (n_steps > 1) {
         loadStage(1);
@@ -536,37 +539,50 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<HEA
         if (t0 < wave_max_visible) {
             computeStep(j & 1, t0, t0 + BN > wave_min_visible);
         }
-        if (j + 1 < n_steps) {
-            storeStage((j + 1) & 1);
-        }
+        awaitStage();
         __syncthreads();
         if (j + 2 < n_steps) {
             loadStage(j + 2);
         }
     }
 
-    // ---- normalise and store: lane writes strip c of rows 4g..4g+3 of each group ----
+    // ---- normalise and store. A lane holds single columns (16 e + c) of its rows; the wavefront's 16 R rows pass
+    // through LDS (the K buffers: every wavefront is past the last barrier of the loop, nothing is in flight) and go
+    // out as 16-byte pieces, 64 lanes on consecutive pieces ----
+    static_assert(TT >= 2 * R, "the K buffers hold the output rows of all four wavefronts");
+    unsigned short *stage = reinterpret_cast<unsigned short *>(&k_lds[0][0]) + w * (R * 16 * HEAD);
 #pragma unroll
     for (int r = 0; r < R; ++r) {
 #pragma unroll
         for (int rr = 0; rr < 4; ++rr) {
-            const int src_lane = 4 * g + rr;
-            const int visible_row = __shfl(visible[r], src_lane, 64);
-            const int row = block_row0 + (w * R + r) * 16 + src_lane;
-            if (row >= total_rows || visible_row <= 0) {
-                continue;
-            }
-            const int token = row / a.group;
-            const int head = kv_head * a.group + (row - token * a.group);
             const float inv_l = 1.0f / (ol[r][rr] + 1e-6f);
-            uint32_t packed[G::kWords];
+            unsigned short *row = stage + (r * 16 + 4 * g + rr) * HEAD + c;
 #pragma unroll
-            for (int i = 0; i < G::kWords; ++i) {
-                packed[i] = T::pack2(o[r][2 * i][rr] * inv_l, o[r][2 * i + 1][rr] * inv_l);
+            for (int e = 0; e < G::kCols; ++e) {
+                row[16 * e] = static_cast<unsigned short>(T::pack2(o[r][e][rr] * inv_l, 0.0f));
             }
-            S *o_ptr = static_cast<S *>(a.out) + (span.q_start + token) * a.o_stride + head * a.o_head_stride;
-            storeStrip<HEAD>(o_ptr, c, packed);
         }
+    }
+    // the wavefront's own stores have landed before its lanes read each other's columns (also keeps the compiler
+    // from moving the differently typed loads below across the stores above)
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    constexpr int kPieces = R * 16 * G::kChunksPerRow; // 16-byte pieces of the wavefront's rows
+#pragma unroll
+    for (int i = 0; i < kPieces / 64; ++i) {
+        const int piece = 64 * i + lane;
+        const int local_row = piece / G::kChunksPerRow, chunk = piece % G::kChunksPerRow;
+        const int row = block_row0 + w * R * 16 + local_row;
+        if (row >= total_rows) {
+            continue;
+        }
+        const int token = row / a.group;
+        if (visibleTokens(span, token) <= 0) {
+            continue;
+        }
+        const int head = kv_head * a.group + (row - token * a.group);
+        const uint4 x = *reinterpret_cast<const uint4 *>(stage + local_row * HEAD + 8 * chunk);
+        S *o_ptr = static_cast<S *>(a.out) + (span.q_start + token) * a.o_stride + head * a.o_head_stride;
+        *reinterpret_cast<uint4 *>(o_ptr + 8 * chunk) = x;
     }
 }
 
