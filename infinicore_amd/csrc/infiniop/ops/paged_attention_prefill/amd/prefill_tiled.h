@@ -56,11 +56,10 @@ using op::paged_attention::amd::TileGeometry;
 constexpr int kPrefillThreads = 256;
 // K / V operands are requested from LDS this many uses before the matrix instructions that take them (an LDS read
 // takes longer than the R instructions one operand feeds; left alone the compiler requests one or two ahead and
-// the matrix unit waits). At the Llama-3-8B chunked-prefill shape, head 128, two to six ahead are within 3 % of each
-// other (600 - 620 us, run-to-run spread 1.5 %) against 639 us left to the compiler; above head 128, where the
-// registers allow more, 8 is no better than 4.
-template <int HEAD>
-constexpr int prefillOperandsAhead() { return HEAD <= 128 ? 3 : 4; }
+// the matrix unit waits). At the Llama-3-8B chunked-prefill shape, head 128, three to six ahead are within 1.5 % of
+// each other, the run-to-run spread (571 - 578 us; with V staged through registers 600 - 620 us against 639 us left
+// to the compiler); above head 128, where the registers allow more, 8 is no better than 4.
+constexpr int kOperandsAhead = 4;
 constexpr float kLazyLog2 = 8.0f; // how far (in powers of two) a row maximum may outgrow its reference point
 
 // 16-byte load from (wave-uniform base) + (32-bit per-lane byte offset), through the caches: K/V tiles
@@ -391,7 +390,7 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<HEA
         // K.Q^T: operand idx = (tile tt, 32 dimensions kk). The scheduler groups pin the order "one LDS read, then the
         // R matrix instructions of the operand read kAheadK earlier"; the first kAheadK reads are a group of their own.
         {
-            constexpr int kAheadK = prefillOperandsAhead<HEAD>();
+            constexpr int kAheadK = kOperandsAhead;
             constexpr int kOperandsK = TT * G::kLoads;
             auto readK = [&](int idx) {
                 const int tt = idx / G::kLoads, kk = idx % G::kLoads;
@@ -485,7 +484,7 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<HEA
         }
 
         // P.V: the V operands run kAhead ahead as well
-        constexpr int kAhead = prefillOperandsAhead<HEAD>();
+        constexpr int kAhead = kOperandsAhead;
         constexpr int kOperands = (TT / 2) * G::kCols;
         // Operand (u, e) = V[32 tokens of tiles 2u, 2u + 1][columns 16 e .. 16 e + 15]: lane (g, c) needs tokens
         // 4g..4g+3 of either tile at column 16 e + c. A transposing read hands lane c of a group of 16 the element
