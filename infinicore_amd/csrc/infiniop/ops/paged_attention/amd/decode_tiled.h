@@ -145,6 +145,16 @@ __device__ __forceinline__ uint4 loadLane16(const char *uniform_base, uint32_t l
 // keeps three-operand forms from fusing: the maximum of 16 scores is 10 instructions this way and 27 with fmaxf.
 __device__ __forceinline__ float maxOf(float a, float b) { return __builtin_elementwise_maximum(a, b); }
 
+// 16 bytes per lane from global memory straight into LDS, without a register in between: lane i of the wavefront
+// writes the 16 bytes at lds_base + 16 i (lds_base is the same for all lanes); lanes that are switched off write
+// nothing. The data is in LDS when the wavefront's vector-memory counter has counted the instruction off.
+// NONTEMPORAL: for data read once per call (see loadLane16).
+template <bool NONTEMPORAL = false>
+__device__ __forceinline__ void loadLane16ToLds(const char *global_src, uint4 *lds_base) {
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)global_src,
+                                     (__attribute__((address_space(3))) void *)lds_base, 16, 0, NONTEMPORAL ? 2 : 0);
+}
+
 // max over the four lanes {c, c+16, c+32, c+48}; every one of them gets the result (two lane swaps,
 // no LDS traffic)
 __device__ __forceinline__ float maxAcrossTokenGroups(float x) {

@@ -50,6 +50,7 @@ using op::paged_attention::amd::TileF16;
 
 using op::paged_attention::amd::kTileTokens;
 using op::paged_attention::amd::LaneOffsets;
+using op::paged_attention::amd::loadLane16ToLds;
 using op::paged_attention::amd::storeStrip;
 using op::paged_attention::amd::TileGeometry;
 
@@ -68,14 +69,6 @@ constexpr float kLazyLog2 = 8.0f; // how far (in powers of two) a row maximum ma
 __device__ __forceinline__ uint4 loadLane16Cached(const char *uniform_base, uint32_t lane_offset) {
     asm volatile("" : "+v"(lane_offset));
     return *reinterpret_cast<const uint4 *>(uniform_base + lane_offset);
-}
-
-// 16 bytes per lane from global memory straight into LDS, without a register in between: lane i of the wavefront
-// writes the 16 bytes at lds_base + 16 i (lds_base is the same for all lanes); lanes that are switched off write
-// nothing. The data is in LDS when the wavefront's vector-memory counter has counted the instruction off.
-__device__ __forceinline__ void loadLane16ToLds(const char *global_src, uint4 *lds_base) {
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)global_src,
-                                     (__attribute__((address_space(3))) void *)lds_base, 16, 0, 0);
 }
 
 // Rows of one workgroup for R column groups per wavefront.
