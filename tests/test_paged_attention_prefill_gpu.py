@@ -223,7 +223,7 @@ def test_alibi(gpu_handle, oracle, monkeypatch, dtype, kernel):
     run_case(gpu_handle, oracle, workloads.make_prefill_inputs(cfg), alibi=slopes)
 
 
-@pytest.mark.parametrize("seed", range(16))
+@pytest.mark.parametrize("seed", range(40))
 def test_random_shapes_row_blocks_and_dtypes(gpu_handle, oracle, monkeypatch, seed):
     """Every knob drawn at random from one seed: head size, group size, page size, batch, new-token and history
     ranges, dtype, index dtype, ALiBi and rows per workgroup."""
