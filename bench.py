@@ -108,7 +108,7 @@ def run_prefill(args, torch, L, workloads, dev):
     handle = L.create_handle()
     tensors = [t.to(dev) for t in (inp.q, inp.k_cache, inp.v_cache, inp.block_tables, inp.seq_lens, inp.cum_seq_lens_q)]
     q, k_cache, v_cache, bt, sl, cu = tensors
-    out = torch.zeros_like(q)
+    out = torch.zeros((*q.shape[:-1], v_cache.shape[-1]), dtype=q.dtype, device=dev)
     DTYPES = {torch.float16: L.InfiniDtype.F16, torch.bfloat16: L.InfiniDtype.BF16, torch.int64: L.InfiniDtype.I64}
     descs = [L.create_tensor_descriptor(tuple(t.shape), tuple(t.stride()), DTYPES[t.dtype]) for t in (out, *tensors)]
     op = L.infiniopOperatorDescriptor_t()
@@ -155,8 +155,8 @@ def run_prefill(args, torch, L, workloads, dev):
     tflops_dev = flops / (us_dev * 1e-6) / 1e12
 
     result = {
-        "metric": "PagedAttn prefill achieved TFLOP/s (4 * head_size * heads * visible query-key pairs / time per call), "
-                  "8B-GQA, 1 GPU",
+        "metric": "PagedAttn prefill achieved TFLOP/s (2 * (head_size + value_size) * heads * visible query-key pairs / "
+                  "time per call), 1 GPU",
         "value": round(tflops_wall, 1),
         "unit": "TFLOP/s",
         "n_gpus": 1,
@@ -172,7 +172,7 @@ def run_prefill(args, torch, L, workloads, dev):
         "config": {
             "workload": cfg.name,
             "num_seqs": cfg.num_seqs, "num_heads": cfg.num_heads, "num_kv_heads": cfg.num_kv_heads,
-            "head_size": cfg.head_size, "block_size": cfg.block_size,
+            "head_size": cfg.head_size, "value_size": cfg.v_size, "block_size": cfg.block_size,
             "new_tokens": f"uniform[{cfg.min_new},{cfg.max_new}] sum={int(new.sum())}",
             "history_tokens": f"uniform[{cfg.min_history},{cfg.max_history}] sum={int(history.sum())}",
             "flops_per_call": flops,
@@ -221,7 +221,7 @@ def run_prefill(args, torch, L, workloads, dev):
         for r in rows:
             s = int(np.searchsorted(np.asarray(cum), r, side="right") - 1)
             sample_pairs += int(history[s]) + (r - cum[s]) + 1
-        sample_flops = sample_pairs * cfg.num_heads * 4 * cfg.head_size
+        sample_flops = sample_pairs * cfg.num_heads * 2 * (cfg.head_size + cfg.v_size)
         reps, t0 = 0, time.perf_counter()
         while reps < 50 and time.perf_counter() - t0 < 12.0:
             paged_oracle.paged_attention_prefill(inp.q, inp.k_cache, inp.v_cache, inp.block_tables, inp.seq_lens,

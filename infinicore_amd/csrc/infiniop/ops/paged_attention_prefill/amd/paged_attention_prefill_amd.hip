@@ -25,7 +25,7 @@ using op::paged_attention::amd::IndexU32;
 // Decided once, at descriptor creation, from shapes and the device alone (sequence lengths live in
 // device memory and are never read on the host).
 struct Plan {
-    bool tiled;          // matrix-core kernel (head 64 / 128 / 192 / 256, power-of-two pages >= 8, 16-byte aligned strides)
+    bool tiled;          // matrix-core kernel (head 64 / 128 / 192 / 256 or keys 576 with values 512, power-of-two pages >= 8, 16-byte aligned strides)
     int groups_per_wave; // tiled: R = 1 or 2 column groups per wavefront -> 64 R rows per workgroup
     int dims_per_lane;   // element-wise kernel: ceil(max(head_size, value_size) / 64)
 };
@@ -38,8 +38,10 @@ Plan makePlan(const PagedAttentionPrefillInfo &in, const device::amd::DeviceInfo
     const bool pow2_page = bs >= 8 && (bs & (bs - 1)) == 0;
     const long long group = static_cast<long long>(in.num_heads / in.num_kv_heads);
     const long long rows = static_cast<long long>(in.total_q_tokens) * group; // per KV head
-    const bool tiled_head = in.head_size == 64 || in.head_size == 128 || in.head_size == 192 || in.head_size == 256;
-    plan.tiled = tiled_head && in.value_size == in.head_size && pow2_page
+    const bool equal_sizes = in.value_size == in.head_size
+                          && (in.head_size == 64 || in.head_size == 128 || in.head_size == 192 || in.head_size == 256);
+    const bool latent = in.head_size == 576 && in.value_size == 512; // keys 576, values 512
+    plan.tiled = (equal_sizes || latent) && pow2_page
               && multipleOf8(in.q_stride) && multipleOf8(in.q_head_stride) && multipleOf8(in.o_stride)
               && multipleOf8(in.o_head_stride) && multipleOf8(in.k_batch_stride) && multipleOf8(in.k_head_stride)
               && multipleOf8(in.k_row_stride) && multipleOf8(in.v_batch_stride) && multipleOf8(in.v_head_stride)
@@ -63,6 +65,9 @@ Plan makePlan(const PagedAttentionPrefillInfo &in, const device::amd::DeviceInfo
     int r = 2;
     if (rows_per_seq <= 64 || rows / 128 * static_cast<long long>(in.num_kv_heads) < resident * dev.compute_units) {
         r = 1;
+    }
+    if (latent) {
+        r = 1; // the accumulators of 64 rows x 512 columns are half the register file
     }
     if (const char *env = std::getenv("INFINIOP_AMD_PREFILL_GROUPS")) {
         const int forced = std::atoi(env);
@@ -88,27 +93,30 @@ void launchGeneric(const PrefillArgs &a, const Plan &plan, hipStream_t stream) {
     }
 }
 
-template <typename T, typename Tindex, int HEAD, bool PLAIN>
+template <typename T, typename Tindex, int KHEAD, int VHEAD, bool PLAIN>
 void launchTiledHead(const PrefillArgs &a, const Plan &plan, hipStream_t stream) {
     // sum over sequences of ceil(rows / block_rows) is at most floor(total rows / block_rows) + num_seqs
     const long long rows = static_cast<long long>(a.total_q_tokens) * a.group;
     const int groups = plan.groups_per_wave;
     const int block_rows = prefillBlockRows(groups);
     const dim3 grid(static_cast<unsigned>((rows / block_rows + a.num_seqs) * a.num_kv_heads));
-    if (groups == 2) {
-        prefillTiledKernel<T, Tindex, HEAD, 2, PLAIN><<<grid, kPrefillThreads, 0, stream>>>(a);
-        return;
+    if constexpr (KHEAD == VHEAD) {
+        if (groups == 2) {
+            prefillTiledKernel<T, Tindex, KHEAD, VHEAD, 2, PLAIN><<<grid, kPrefillThreads, 0, stream>>>(a);
+            return;
+        }
     }
-    prefillTiledKernel<T, Tindex, HEAD, 1, PLAIN><<<grid, kPrefillThreads, 0, stream>>>(a);
+    prefillTiledKernel<T, Tindex, KHEAD, VHEAD, 1, PLAIN><<<grid, kPrefillThreads, 0, stream>>>(a);
 }
 
 template <typename T, typename Tindex, bool PLAIN>
 void launchTiledPlain(const PrefillArgs &a, const Plan &plan, hipStream_t stream) {
     switch (a.head_size) {
-    case 64: launchTiledHead<T, Tindex, 64, PLAIN>(a, plan, stream); break;
-    case 128: launchTiledHead<T, Tindex, 128, PLAIN>(a, plan, stream); break;
-    case 192: launchTiledHead<T, Tindex, 192, PLAIN>(a, plan, stream); break;
-    default: launchTiledHead<T, Tindex, 256, PLAIN>(a, plan, stream); break;
+    case 64: launchTiledHead<T, Tindex, 64, 64, PLAIN>(a, plan, stream); break;
+    case 128: launchTiledHead<T, Tindex, 128, 128, PLAIN>(a, plan, stream); break;
+    case 192: launchTiledHead<T, Tindex, 192, 192, PLAIN>(a, plan, stream); break;
+    case 256: launchTiledHead<T, Tindex, 256, 256, PLAIN>(a, plan, stream); break;
+    default: launchTiledHead<T, Tindex, 576, 512, PLAIN>(a, plan, stream); break;
     }
 }
 

@@ -1,31 +1,32 @@
-// Tiled prefill kernel for head_size = value_size = 64, 128, 192 or 256 on gfx950 (CDNA4, 64-lane
-// wavefronts). Figures below are for head 128; tile geometry per head size is TileGeometry<HEAD> of
-// the decode kernels.
+// Tiled prefill kernel on gfx950 (CDNA4, 64-lane wavefronts) for head_size = value_size = 64, 128, 192 or 256 and
+// for latent attention (keys of 576, values of 512 elements). Figures below are for head 128; the geometry per
+// size is PrefillGeometry below.
 //
 // Work unit: one 256-thread workgroup = 64*R "rows" of one (sequence, KV head). A row is a (new
 // token, query head of the KV head's group) pair, token-major: row = token * group + head_in_group.
 // Packing the heads of a group into the row dimension means a K/V tile fetched once serves all of
 // them, and short prompts still fill the matrix instructions. Each of the four wavefronts owns 16*R
-// consecutive rows (R = 1 or 2 column groups of 16; 1 only for heads above 128).
+// consecutive rows (R = 1 or 2 column groups of 16).
 //
-// The K/V tokens the rows may see are consumed in steps of 64 (32 for heads above 128). Per step the
-// workgroup copies that many K rows and V rows (16 KiB each) from the paged pool into LDS, a wavefront
-// 16 tokens at a time, double-buffered: the global loads of step j+1 are in flight while step j is
-// computed, and one barrier per step separates writers and readers.
-//   * K is stored as it comes (16-byte chunks, XOR-swizzled so the later row-wise reads are
-//     conflict-free): the matrix instruction wants lane i to hold token i.
-//   * V is stored already transposed into matrix-operand order: the lane that loaded rows 4g..4g+3
-//     of a column strip interleaves them per column with byte permutes and writes, for each of its
-//     columns, the four tokens as one 8-byte word. A reader fetches two such words (tokens
-//     4g..4g+3 of two 16-token tiles) and has the 8-deep operand of one 16x16x32 instruction.
+// The K/V tokens the rows may see are consumed in steps of 64 (32 where LDS or registers ask for it: see
+// prefillStepTokens). Per step the workgroup brings that many K rows and V rows (16 KiB each) from the paged pool
+// straight into LDS (16 bytes per lane, no register in between), a wavefront 16 tokens at a time, double-buffered:
+// the loads of step j+2 are issued after the barrier that ends step j and awaited before the barrier that ends
+// step j+1; one barrier per step separates writers and readers. Which global chunk a lane asks for decides the
+// layout in LDS:
+//   * K row-major, 16-byte chunks XOR-swizzled by the row so that the later row-wise reads are conflict-free: the
+//     matrix instruction wants lane i to hold token i.
+//   * V row-major in blocks of 16 columns (see v_lds): the operand of P.V wants 8 tokens of one column per lane,
+//     which the transposing LDS read of gfx950 (ds_read_b64_tr_b16) delivers from row-major data, four tokens per
+//     read.
 //
 // Arithmetic per step and column group, lane = 16*g + c:
 //   S[token][row] = K . Q^T   16 x v_mfma_f32_16x16x32 (A = K tile from LDS, B = Q held in registers
 //                             for the whole kernel; lane holds S[16T + 4g + 0..3][row c], T = 0..3)
 //   causal mask (only in steps that touch the diagonal), online softmax in fp32 / log2 domain
 //   O[row][dim] += P . V      16 x v_mfma_f32_16x16x32 (A = P rounded to the storage dtype, straight
-//                             from the registers S came out in; B = V words from LDS; lane holds
-//                             O[row 4g + 0..3][8c + e], e = 0..7)
+//                             from the registers S came out in; B = V from LDS; lane holds
+//                             O[row 4g + 0..3][16 e + c], e = 0..7)
 //   l[row]      += P . 1       2 x v_mfma_f32_16x16x32: the denominator sums the rounded probabilities
 // K/V fragments read from LDS are shared by the R column groups of a wavefront. A step whose tokens
 // lie beyond everything a wavefront's rows may see is skipped by that wavefront (it still takes part
@@ -49,10 +50,7 @@ using op::paged_attention::amd::TileBF16;
 using op::paged_attention::amd::TileF16;
 
 using op::paged_attention::amd::kTileTokens;
-using op::paged_attention::amd::LaneOffsets;
 using op::paged_attention::amd::loadLane16ToLds;
-using op::paged_attention::amd::storeStrip;
-using op::paged_attention::amd::TileGeometry;
 
 constexpr int kPrefillThreads = 256;
 // K / V operands are requested from LDS this many uses before the matrix instructions that take them (an LDS read
@@ -111,26 +109,25 @@ __device__ __forceinline__ bool findRowBlock(const PrefillArgs &a, int lane, int
     return false;
 }
 
-// This lane's strip of one V row, through the caches: the first piece at `first`, the rest piece (heads above
-// 128; see TileGeometry) `rest_bytes` further on
-template <int HEAD>
-__device__ __forceinline__ void loadStripCached(const char *first, uint32_t rest_bytes, uint32_t (&w)[TileGeometry<HEAD>::kWords]) {
-    using G = TileGeometry<HEAD>;
-    if constexpr (G::kFirstCols % 8 == 0) {
-#pragma unroll
-        for (int i = 0; i < G::kFirstCols / 8; ++i) {
-            const uint4 x = reinterpret_cast<const uint4 *>(first)[i];
-            w[4 * i] = x.x, w[4 * i + 1] = x.y, w[4 * i + 2] = x.z, w[4 * i + 3] = x.w;
-        }
-    } else {
-        const uint2 x = *reinterpret_cast<const uint2 *>(first);
-        w[0] = x.x, w[1] = x.y;
+// Geometry of the 16-token tiles for keys of KHEAD and values of VHEAD elements (equal except for latent attention,
+// 576 / 512). K: kLoadsK instructions of 64 16-byte chunks per tile, row r keeps its chunks XOR-swizzled by
+// r mod kSwizzle (TileGeometry of the decode kernels for equal sizes). V: kLoadsV instructions, kColsV blocks of 16
+// columns.
+template <int KHEAD, int VHEAD>
+struct PrefillGeometry {
+    static_assert(KHEAD % 64 == 0 && VHEAD % 64 == 0, "whole load instructions per tile, whole blocks of four V blocks");
+    static constexpr int kLoadsK = KHEAD / 32; // K load instructions per tile = K-steps of K.Q^T
+    static constexpr int kChunksPerRowK = KHEAD / 8;
+    static constexpr int kSwizzle = KHEAD % 128 == 0 ? 16 : 8; // stays inside a row: its chunk count is a multiple
+    static constexpr int kLoadsV = VHEAD / 32;
+    static constexpr int kChunksPerRowV = VHEAD / 8;
+    static constexpr int kColsV = VHEAD / 16; // blocks of 16 value columns
+    static __device__ __forceinline__ int kRow(int j, int lane) { return (64 * j + lane) / kChunksPerRowK; }
+    static __device__ __forceinline__ int kChunk(int j, int lane) { return (64 * j + lane) % kChunksPerRowK; }
+    static __device__ __forceinline__ int ldsIndex(int row, int chunk) {
+        return row * kChunksPerRowK + (chunk ^ (row & (kSwizzle - 1)));
     }
-    if constexpr (G::kRestCols == 4) {
-        const uint2 x = *reinterpret_cast<const uint2 *>(first + rest_bytes);
-        w[G::kFirstCols / 2] = x.x, w[G::kFirstCols / 2 + 1] = x.y;
-    }
-}
+};
 
 // Tokens per step, and workgroups that share a compute unit. Up to head 128: 64 tokens, two workgroups. Head 256
 // needs more than half the register file even for 64 rows, so one workgroup has the unit to itself and takes 64-token
@@ -138,27 +135,29 @@ __device__ __forceinline__ void loadStripCached(const char *first, uint32_t rest
 // steps (48 KiB each); with 128 rows it is alone on the unit and takes 64-token steps (96 KiB).
 // At the Llama-3-8B chunked-prefill shape, 128 rows against 64 rows with 32-token steps: head 192 1 864 -> 1 692 us,
 // head 256 4 040 -> 2 046 us (2 787 us with 64 rows and 64-token steps).
-template <int HEAD, int R>
-constexpr int prefillStepTokens() { return (HEAD <= 128 || HEAD == 256 || R == 2) ? 64 : 32; }
-template <int HEAD, int R>
-constexpr int prefillWorkgroupsPerUnit() { return (HEAD <= 128 || (HEAD == 192 && R == 1)) ? 2 : 1; }
+// Latent attention (keys 576): 64 rows need 200 accumulator and query registers, so one workgroup per unit, and
+// 32-token steps (two K and two V buffers: 136 KiB).
+template <int KHEAD, int R>
+constexpr int prefillStepTokens() { return (KHEAD <= 128 || KHEAD == 256 || (KHEAD == 192 && R == 2)) ? 64 : 32; }
+template <int KHEAD, int R>
+constexpr int prefillWorkgroupsPerUnit() { return (KHEAD <= 128 || (KHEAD == 192 && R == 1)) ? 2 : 1; }
 
 // PLAIN: no ALiBi and scale > 0. The running maximum is then kept in units of the raw dot product
 // (a positive scale keeps the order) and each probability costs one fused multiply-add and one exp2.
-template <typename T, typename Tindex, int HEAD, int R, bool PLAIN>
-__global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<HEAD, R>())) prefillTiledKernel(PrefillArgs a) {
+template <typename T, typename Tindex, int KHEAD, int VHEAD, int R, bool PLAIN>
+__global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<KHEAD, R>())) prefillTiledKernel(PrefillArgs a) {
     using S = typename T::storage;
-    using G = TileGeometry<HEAD>;
+    using G = PrefillGeometry<KHEAD, VHEAD>;
     constexpr int BM = prefillBlockRows(R);
-    constexpr int BN = prefillStepTokens<HEAD, R>();
+    constexpr int BN = prefillStepTokens<KHEAD, R>();
     constexpr int TT = BN / kTileTokens;             // 16-token tiles per step: 4 or 2
-    constexpr int kTileChunks = kTileTokens * G::kChunksPerRow;
-    __shared__ uint4 k_lds[2][TT * kTileChunks];       // [tile][token][16-byte chunk, XOR-swizzled by the token]
+    constexpr int kTileChunksK = kTileTokens * G::kChunksPerRowK, kTileChunksV = kTileTokens * G::kChunksPerRowV;
+    __shared__ uint4 k_lds[2][TT * kTileChunksK];       // [tile][token][16-byte chunk, XOR-swizzled by the token]
     // V tile in LDS: [row half (8 rows)][block of 16 columns (32 bytes)][row of the half][two 16-byte chunks], i.e.
     // slot = half * 8 * chunks per row + block * 16 + (row % 8) * 2 + chunk % 2. A transposing read of one block then
     // touches two runs of 256 bytes, and 64 consecutive slots (one load instruction) are four blocks of eight rows:
     // 128 contiguous bytes of each row in global memory.
-    __shared__ uint4 v_lds[2][TT * kTileChunks];
+    __shared__ uint4 v_lds[2][TT * kTileChunksV];
 
     const int lane = threadIdx.x & 63;
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -190,7 +189,7 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<HEA
     const int n_steps = (block_visible + BN - 1) / BN;
 
     // ---- this lane's columns: row c of each of the wavefront's R column groups ----
-    uint4 q_reg[R][G::kLoads];
+    uint4 q_reg[R][G::kLoadsK];
     int visible[R];
     float slope[R];
     int wave_max_visible = 0, wave_min_visible = 0x7fffffff;
@@ -204,7 +203,7 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<HEA
         slope[r] = (a.alibi_slopes != nullptr && valid) ? a.alibi_slopes[head] * kLog2e : 0.0f;
         const S *q_ptr = static_cast<const S *>(a.q) + (span.q_start + token) * a.q_stride + head * a.q_head_stride;
 #pragma unroll
-        for (int kk = 0; kk < G::kLoads; ++kk) {
+        for (int kk = 0; kk < G::kLoadsK; ++kk) {
             q_reg[r][kk] = valid ? *reinterpret_cast<const uint4 *>(q_ptr + 32 * kk + 8 * g) : make_uint4(0, 0, 0, 0);
         }
         wave_max_visible = max(wave_max_visible, visible[r]);
@@ -252,25 +251,22 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<HEA
         return clampPage(raw, a.num_blocks);
     };
 
-    // byte offsets of this lane's pieces inside a 16-token tile (pages >= 16 tokens)
-    const LaneOffsets<HEAD> off(lane, static_cast<uint32_t>(a.k_row_stride) * sizeof(S),
-                                static_cast<uint32_t>(a.v_row_stride) * sizeof(S));
     // K goes from global memory straight into its place in LDS: slot 64 j + lane of the tile holds chunk
-    // (slot % chunks per row) ^ swizzle(row) of row slot / chunks per row (TileGeometry::ldsIndex read backwards), so
+    // (slot % chunks per row) ^ swizzle(row) of row slot / chunks per row (PrefillGeometry::ldsIndex read backwards), so
     // that is the chunk this lane asks for with instruction j. V passes through registers (it is transposed on
     // the way).
-    uint32_t k_src_off[G::kLoads];
+    uint32_t k_src_off[G::kLoadsK];
 #pragma unroll
-    for (int j = 0; j < G::kLoads; ++j) {
+    for (int j = 0; j < G::kLoadsK; ++j) {
         const int row = G::kRow(j, lane), slot = G::kChunk(j, lane);
         k_src_off[j] = row * static_cast<uint32_t>(a.k_row_stride) * sizeof(S) + 16 * (slot ^ (row & (G::kSwizzle - 1)));
     }
     // V likewise, into the layout described at v_lds
-    auto vRowOfSlot = [](int slot) { return 8 * (slot / (8 * G::kChunksPerRow)) + (slot % 16) / 2; };
-    auto vChunkOfSlot = [](int slot) { return 2 * ((slot % (8 * G::kChunksPerRow)) / 16) + slot % 2; };
-    uint32_t v_src_off[G::kLoads];
+    auto vRowOfSlot = [](int slot) { return 8 * (slot / (8 * G::kChunksPerRowV)) + (slot % 16) / 2; };
+    auto vChunkOfSlot = [](int slot) { return 2 * ((slot % (8 * G::kChunksPerRowV)) / 16) + slot % 2; };
+    uint32_t v_src_off[G::kLoadsV];
 #pragma unroll
-    for (int j = 0; j < G::kLoads; ++j) {
+    for (int j = 0; j < G::kLoadsV; ++j) {
         v_src_off[j] = vRowOfSlot(64 * j + lane) * static_cast<uint32_t>(a.v_row_stride) * sizeof(S) + 16 * vChunkOfSlot(64 * j + lane);
     }
     auto loadStage = [&](int step) {
@@ -286,12 +282,12 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<HEA
             // Rows past the end of the sequence are fetched like the others: the page they lie in exists (its id
             // is clamped to the sequence's last entry and to the pool), and whatever they hold only reaches scores
             // that the causal mask replaces.
-            uint4 *k_dst = &k_lds[step & 1][copy_tile * kTileChunks];
+            uint4 *k_dst = &k_lds[step & 1][copy_tile * kTileChunksK];
             if (!small_pages) {
                 const int page = pageOfEntry(e0);
                 const char *k_tile = k_head + (page * a.k_batch_stride + (t & block_mask) * a.k_row_stride) * static_cast<int64_t>(sizeof(S));
 #pragma unroll
-                for (int j = 0; j < G::kLoads; ++j) {
+                for (int j = 0; j < G::kLoadsK; ++j) {
                     uint32_t lane_off = k_src_off[j];
                     asm volatile("" : "+v"(lane_off));
                     loadLane16ToLds(k_tile + lane_off, k_dst + 64 * j);
@@ -299,7 +295,7 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<HEA
             } else { // pages of 8 tokens: rows 8..15 of the tile lie in the next page
                 const int id0 = pageOfEntry(e0), id1 = pageOfEntry(e0 + 1);
 #pragma unroll
-                for (int j = 0; j < G::kLoads; ++j) {
+                for (int j = 0; j < G::kLoadsK; ++j) {
                     const int row = G::kRow(j, lane), slot = G::kChunk(j, lane);
                     const int page = row >= 8 ? id1 : id0;
                     const char *src = k_head + (page * a.k_batch_stride + (row & 7) * a.k_row_stride) * static_cast<int64_t>(sizeof(S))
@@ -311,12 +307,12 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<HEA
         if (!copies_v) {
             return;
         }
-        uint4 *v_dst = &v_lds[step & 1][copy_tile * kTileChunks];
+        uint4 *v_dst = &v_lds[step & 1][copy_tile * kTileChunksV];
         if (t + kTileTokens <= kv_len && !small_pages) {
             const int page = pageOfEntry(e0);
             const char *v_tile = v_head + (page * a.v_batch_stride + (t & block_mask) * a.v_row_stride) * static_cast<int64_t>(sizeof(S));
 #pragma unroll
-            for (int j = 0; j < G::kLoads; ++j) {
+            for (int j = 0; j < G::kLoadsV; ++j) {
                 uint32_t lane_off = v_src_off[j];
                 asm volatile("" : "+v"(lane_off));
                 loadLane16ToLds(v_tile + lane_off, v_dst + 64 * j);
@@ -328,7 +324,7 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<HEA
         const int id0 = pageOfEntry(e0), id1 = small_pages ? pageOfEntry(e0 + 1) : id0;
         const int row0 = small_pages ? 0 : (t & block_mask);
 #pragma unroll
-        for (int j = 0; j < G::kLoads; ++j) {
+        for (int j = 0; j < G::kLoadsV; ++j) {
             const int row = vRowOfSlot(64 * j + lane);
             const int page = (small_pages && row >= 8) ? id1 : id0;
             const int page_row = small_pages ? (row & 7) : row0 + row;
@@ -349,12 +345,12 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<HEA
     // (computed by the matrix unit as P . 1, so it sums exactly the rounded probabilities the numerator
     // used and already sits in the accumulators' row layout); m[r] = running maximum of row c, in units
     // of the raw dot product when there is no ALiBi (scale > 0 keeps the order), else of the scaled score.
-    f32x4 o[R][G::kCols], ol[R];
+    f32x4 o[R][G::kColsV], ol[R];
     float m[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
 #pragma unroll
-        for (int e = 0; e < G::kCols; ++e) {
+        for (int e = 0; e < G::kColsV; ++e) {
             o[r][e] = f32x4{0.f, 0.f, 0.f, 0.f};
         }
         ol[r] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -364,7 +360,7 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<HEA
     typedef short s16x4 __attribute__((ext_vector_type(4)));
     typedef __attribute__((address_space(3))) s16x4 *LdsPiece;
     const auto v_read_base = (__attribute__((address_space(3))) char *)v_lds
-                           + 16 * ((g >> 1) * 8 * G::kChunksPerRow + (4 * (g & 1) + (c >> 2)) * 2 + ((c & 3) >> 1)) + 8 * (c & 1);
+                           + 16 * ((g >> 1) * 8 * G::kChunksPerRowV + (4 * (g & 1) + (c >> 2)) * 2 + ((c & 3) >> 1)) + 8 * (c & 1);
     const uint32_t one2 = T::pack2(1.0f, 1.0f);
     const uint4 ones = make_uint4(one2, one2, one2, one2);
     const float unit = PLAIN ? a.scale_log2 : 1.0f; // log2-domain size of one unit of m
@@ -384,10 +380,10 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<HEA
         // R matrix instructions of the operand read kAheadK earlier"; the first kAheadK reads are a group of their own.
         {
             constexpr int kAheadK = kOperandsAhead;
-            constexpr int kOperandsK = TT * G::kLoads;
+            constexpr int kOperandsK = TT * G::kLoadsK;
             auto readK = [&](int idx) {
-                const int tt = idx / G::kLoads, kk = idx % G::kLoads;
-                return k_lds[buf][tt * kTileChunks + G::ldsIndex(c, 4 * kk + g)];
+                const int tt = idx / G::kLoadsK, kk = idx % G::kLoadsK;
+                return k_lds[buf][tt * kTileChunksK + G::ldsIndex(c, 4 * kk + g)];
             };
             uint4 kf[kAheadK];
 #pragma unroll
@@ -397,7 +393,7 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<HEA
             __builtin_amdgcn_sched_group_barrier(0x100, kAheadK, 0);
 #pragma unroll
             for (int idx = 0; idx < kOperandsK; ++idx) {
-                const int tt = idx / G::kLoads, kk = idx % G::kLoads;
+                const int tt = idx / G::kLoadsK, kk = idx % G::kLoadsK;
                 const uint4 cur = kf[idx % kAheadK];
                 if (idx + kAheadK < kOperandsK) {
                     kf[idx % kAheadK] = readK(idx + kAheadK);
@@ -456,7 +452,7 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<HEA
                     const float alpha_r = __shfl(alpha, 4 * g + rr, 64);
                     ol[r][rr] *= alpha_r;
 #pragma unroll
-                    for (int e = 0; e < G::kCols; ++e) {
+                    for (int e = 0; e < G::kColsV; ++e) {
                         o[r][e][rr] *= alpha_r;
                     }
                 }
@@ -478,16 +474,16 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<HEA
 
         // P.V: the V operands run kAhead ahead as well
         constexpr int kAhead = kOperandsAhead;
-        constexpr int kOperands = (TT / 2) * G::kCols;
+        constexpr int kOperands = (TT / 2) * G::kColsV;
         // Operand (u, e) = V[32 tokens of tiles 2u, 2u + 1][columns 16 e .. 16 e + 15]: lane (g, c) needs tokens
         // 4g..4g+3 of either tile at column 16 e + c. A transposing read hands lane c of a group of 16 the element
         // c % 4 of the four 8-byte pieces that lanes c / 4, c / 4 + 4, + 8, + 12 of the group point at; so lane
         // (g, c) points at token 4g + c / 4, columns 16 e + 4 (c % 4) .. + 3.
         auto readV = [&](int idx) {
-            const int u = idx / G::kCols, e = idx % G::kCols;
-            const auto base = v_read_base + (buf * TT + 2 * u) * (kTileChunks * 16) + 256 * e;
+            const int u = idx / G::kColsV, e = idx % G::kColsV;
+            const auto base = v_read_base + (buf * TT + 2 * u) * (kTileChunksV * 16) + 256 * e;
             const uint2 lo = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<LdsPiece>(base)));
-            const uint2 hi = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<LdsPiece>(base + kTileChunks * 16)));
+            const uint2 hi = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<LdsPiece>(base + kTileChunksV * 16)));
             return make_uint4(lo.x, lo.y, hi.x, hi.y);
         };
         uint4 vf[kAhead];
@@ -498,7 +494,7 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<HEA
         __builtin_amdgcn_sched_group_barrier(0x100, 2 * kAhead, 0); // two reads per operand
 #pragma unroll
         for (int idx = 0; idx < kOperands; ++idx) {
-            const int u = idx / G::kCols, e = idx % G::kCols;
+            const int u = idx / G::kColsV, e = idx % G::kColsV;
             const uint4 cur = vf[idx % kAhead];
             if (idx + kAhead < kOperands) {
                 vf[idx % kAhead] = readV(idx + kAhead);
@@ -541,16 +537,16 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<HEA
     // ---- normalise and store. A lane holds single columns (16 e + c) of its rows; the wavefront's 16 R rows pass
     // through LDS (the K buffers: every wavefront is past the last barrier of the loop, nothing is in flight) and go
     // out as 16-byte pieces, 64 lanes on consecutive pieces ----
-    static_assert(TT >= 2 * R, "the K buffers hold the output rows of all four wavefronts");
-    unsigned short *stage = reinterpret_cast<unsigned short *>(&k_lds[0][0]) + w * (R * 16 * HEAD);
+    static_assert(2 * TT * kTileChunksK * 16 >= 4 * R * 16 * VHEAD * 2, "the K buffers hold the output rows of all four wavefronts");
+    unsigned short *stage = reinterpret_cast<unsigned short *>(&k_lds[0][0]) + w * (R * 16 * VHEAD);
 #pragma unroll
     for (int r = 0; r < R; ++r) {
 #pragma unroll
         for (int rr = 0; rr < 4; ++rr) {
             const float inv_l = 1.0f / (ol[r][rr] + 1e-6f);
-            unsigned short *row = stage + (r * 16 + 4 * g + rr) * HEAD + c;
+            unsigned short *row = stage + (r * 16 + 4 * g + rr) * VHEAD + c;
 #pragma unroll
-            for (int e = 0; e < G::kCols; ++e) {
+            for (int e = 0; e < G::kColsV; ++e) {
                 row[16 * e] = static_cast<unsigned short>(T::pack2(o[r][e][rr] * inv_l, 0.0f));
             }
         }
@@ -558,11 +554,11 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<HEA
     // the wavefront's own stores have landed before its lanes read each other's columns (also keeps the compiler
     // from moving the differently typed loads below across the stores above)
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    constexpr int kPieces = R * 16 * G::kChunksPerRow; // 16-byte pieces of the wavefront's rows
+    constexpr int kPieces = R * 16 * G::kChunksPerRowV; // 16-byte pieces of the wavefront's rows
 #pragma unroll
     for (int i = 0; i < kPieces / 64; ++i) {
         const int piece = 64 * i + lane;
-        const int local_row = piece / G::kChunksPerRow, chunk = piece % G::kChunksPerRow;
+        const int local_row = piece / G::kChunksPerRowV, chunk = piece % G::kChunksPerRowV;
         const int row = block_row0 + w * R * 16 + local_row;
         if (row >= total_rows) {
             continue;
@@ -572,7 +568,7 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<HEA
             continue;
         }
         const int head = kv_head * a.group + (row - token * a.group);
-        const uint4 x = *reinterpret_cast<const uint4 *>(stage + local_row * HEAD + 8 * chunk);
+        const uint4 x = *reinterpret_cast<const uint4 *>(stage + local_row * VHEAD + 8 * chunk);
         S *o_ptr = static_cast<S *>(a.out) + (span.q_start + token) * a.o_stride + head * a.o_head_stride;
         *reinterpret_cast<uint4 *>(o_ptr + 8 * chunk) = x;
     }

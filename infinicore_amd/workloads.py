@@ -68,6 +68,11 @@ class PrefillConfig:
     max_history: int
     spare_block_fraction: float = 0.0
     seed: int = 0
+    value_size: int = 0  # 0 = head_size
+
+    @property
+    def v_size(self) -> int:
+        return self.value_size or self.head_size
 
     @property
     def scale(self) -> float:
@@ -131,6 +136,9 @@ PREFILL_CONFIGS = {
                                          spare_block_fraction=0.10, seed=202),
     "p3_llama3_8b_chunked": PrefillConfig("p3_llama3_8b_chunked", torch.bfloat16, 16, 32, 8, 128, 16, 128, 512,
                                           1024, 8192, spare_block_fraction=0.10, seed=203),
+    # latent-attention cache (one KV head, keys 576, values 512), 16 query heads: chunked prefill like p3
+    "p4_mla_16_heads_chunked": PrefillConfig("p4_mla_16_heads_chunked", torch.bfloat16, 16, 16, 1, 576, 16, 128, 512,
+                                             1024, 8192, spare_block_fraction=0.10, seed=204, value_size=512),
 }
 
 
@@ -217,7 +225,7 @@ def prefill_flops(cfg: PrefillConfig, new, history) -> int:
     """Multiply-adds x 2 of Q.K^T and P.V over the (query token, visible K/V token) pairs."""
     new, history = np.asarray(new, dtype=np.int64), np.asarray(history, dtype=np.int64)
     pairs = int((new * history + new * (new + 1) // 2).sum())
-    return pairs * cfg.num_heads * 4 * cfg.head_size
+    return pairs * cfg.num_heads * 2 * (cfg.head_size + cfg.v_size)
 
 
 def prefill_algorithmic_bytes(cfg: PrefillConfig, new, history) -> int:
@@ -225,8 +233,8 @@ def prefill_algorithmic_bytes(cfg: PrefillConfig, new, history) -> int:
     e = 2
     new, history = np.asarray(new, dtype=np.int64), np.asarray(history, dtype=np.int64)
     total = new + history
-    qo = 2 * int(new.sum()) * cfg.num_heads * cfg.head_size * e
-    kv = int(total.sum()) * cfg.num_kv_heads * 2 * cfg.head_size * e
+    qo = int(new.sum()) * cfg.num_heads * (cfg.head_size + cfg.v_size) * e
+    kv = int(total.sum()) * cfg.num_kv_heads * (cfg.head_size + cfg.v_size) * e
     idx = int(((total + cfg.block_size - 1) // cfg.block_size).sum()) * 8 + (2 * cfg.num_seqs + 1) * 8
     return qo + kv + idx
 
@@ -252,6 +260,8 @@ def make_prefill_inputs(cfg: PrefillConfig) -> PrefillInputs:
     cache_shape = (num_blocks, cfg.num_kv_heads, cfg.block_size, cfg.head_size)
     k_cache = _normal(rng, cache_shape, cfg.dtype)
     v_cache = _normal(rng, cache_shape, cfg.dtype)
+    if cfg.v_size != cfg.head_size:
+        v_cache = v_cache[..., :cfg.v_size].contiguous()
     return PrefillInputs(cfg, q, k_cache, v_cache, torch.from_numpy(table), torch.from_numpy(total),
                          torch.from_numpy(cum), cfg.scale)
 

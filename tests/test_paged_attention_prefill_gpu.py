@@ -114,6 +114,52 @@ def test_reference_mla_shape(gpu_handle, oracle, dtype, idx):
     run_case(gpu_handle, oracle, inp, index_dtype=idx)
 
 
+def mla_inputs(name, dtype, B, H, bs, new, history, seed):
+    """Latent-attention caches: keys of 576 elements, values of 512, one KV head."""
+    inp = workloads.make_prefill_inputs(prefill_config(name, dtype, B, H, 1, 576, bs, new, history, seed=seed))
+    inp.v_cache = inp.v_cache[..., :512].contiguous()
+    return inp
+
+
+@pytest.mark.parametrize("kernel", ["tiled", "generic"])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("H", [16, 128, 5])
+def test_mla_ragged_batches(gpu_handle, oracle, monkeypatch, H, dtype, kernel):
+    """Keys 576 / values 512 on the matrix-core kernel (64 rows per workgroup, 32-token steps) and on the
+    element-wise one: 16 heads (a tensor-parallel shard), all 128, and a head count that fills no tile."""
+    if kernel == "generic":
+        monkeypatch.setenv("INFINIOP_AMD_PREFILL_KERNEL", "generic")
+    small = kernel == "generic" or H == 128
+    inp = mla_inputs(f"mla_h{H}_{kernel}", dtype, 3, H, 16, (1, 30 if small else 200), (0, 80 if small else 500), seed=500 + H)
+    run_case(gpu_handle, oracle, inp)
+
+
+@pytest.mark.parametrize("bs", [8, 64])
+def test_mla_page_sizes_alibi_and_int32(gpu_handle, oracle, bs):
+    inp = mla_inputs(f"mla_bs{bs}", torch.bfloat16, 3, 16, bs, (1, 120), (0, 300), seed=520 + bs)
+    slopes = torch.tensor([2.0 ** -(i % 5 + 1) for i in range(16)], dtype=torch.float32)
+    run_case(gpu_handle, oracle, inp, alibi=slopes, index_dtype=torch.int32)
+
+
+def test_mla_column_layout_and_garbage(gpu_handle, oracle):
+    """V with a distinct constant per column makes the expected output that constant (every one of the 512 output
+    columns lands where it belongs); NaN beyond the sequences must not leak in."""
+    inp = mla_inputs("mla_cols", torch.float16, 3, 16, 16, (5, 90), (3, 200), seed=540)
+    cfg = inp.config
+    ramp = ((torch.arange(512, dtype=torch.float32) - 256) / 16).to(torch.float16)
+    inp.v_cache[:] = ramp
+    for s in range(cfg.num_seqs):
+        L = int(inp.seq_lens[s])
+        if L % 16:
+            page = int(inp.block_tables[s, (L - 1) // 16])
+            inp.k_cache[page, :, L % 16:, :] = float("nan")
+            inp.v_cache[page, :, L % 16:, :] = float("nan")
+    dev = [t.to(DEV) for t in (inp.q, inp.k_cache, inp.v_cache, inp.block_tables, inp.seq_lens, inp.cum_seq_lens_q)]
+    got = run_paged_attention_prefill(gpu_handle, *dev, inp.scale).float().cpu()
+    want = ramp.float().expand_as(got)
+    assert torch.allclose(got, want, atol=2e-3 * float(ramp.float().abs().max()), rtol=0), (got - want).abs().max()
+
+
 # ---- kernel variants --------------------------------------------------------------------------------------
 
 @pytest.mark.parametrize("groups", ["1", "2"])
