@@ -9,9 +9,10 @@ together), so every call streams its K/V from HBM as a real model does when it m
 Inputs are resident in HBM before the timed region. ``us_per_call`` = step time / 32; ``value`` is the
 algorithmic bytes of the step over its time.
 
-With ``--workload p2_llama3_8b_prompt`` or ``p3_llama3_8b_chunked`` a step is one
-``infiniopPagedAttentionPrefill`` call instead, bounded by the bf16 matrix-core peak; the line then
-reports TFLOP/s (2 x multiply-adds of Q.K^T and P.V over the visible query/key pairs).
+With ``--workload p2_llama3_8b_prompt``, ``p3_llama3_8b_chunked`` or ``p4_mla_16_heads_chunked`` (latent
+attention: keys 576, values 512) a step is one ``infiniopPagedAttentionPrefill`` call instead, bounded by the
+bf16 matrix-core peak; the line then reports TFLOP/s (2 x multiply-adds of Q.K^T and P.V over the visible
+query/key pairs).
 
 Prints one JSON line: throughput in algorithmic GB/s (K and V once per KV head + Q + O + the
 needed table entries + lengths), the time per call, the HBM roofline of the step measured with
