@@ -141,6 +141,22 @@ def test_mla_page_sizes_alibi_and_int32(gpu_handle, oracle, bs):
     run_case(gpu_handle, oracle, inp, alibi=slopes, index_dtype=torch.int32)
 
 
+@pytest.mark.parametrize("kernel", ["tiled", "generic"])
+def test_mla_values_as_a_view_of_the_keys(gpu_handle, oracle, monkeypatch, kernel):
+    """The latent layout of DeepSeek-style caches: one tensor of 576 columns per token, the values being its first
+    512 columns (a V row stride of 576 elements)."""
+    if kernel == "generic":
+        monkeypatch.setenv("INFINIOP_AMD_PREFILL_KERNEL", "generic")
+    inp = mla_inputs(f"mla_view_{kernel}", torch.bfloat16, 3, 16, 16, (1, 40), (0, 150), seed=560)
+    k_dev = inp.k_cache.to(DEV)
+    v_dev = k_dev[..., :512]
+    idx = [t.to(DEV) for t in (inp.block_tables, inp.seq_lens, inp.cum_seq_lens_q)]
+    got = run_paged_attention_prefill(gpu_handle, inp.q.to(DEV), k_dev, v_dev, *idx, inp.scale).cpu()
+    want, want_f32 = oracle.paged_attention_prefill(inp.q, inp.k_cache, inp.k_cache[..., :512], inp.block_tables, inp.seq_lens,
+                                                    inp.cum_seq_lens_q, inp.scale, num_threads=ORACLE_THREADS, return_fp32=True)
+    assert_close(got, want, f"mla_view_{kernel}", want_f32)
+
+
 def test_mla_column_layout_and_garbage(gpu_handle, oracle):
     """V with a distinct constant per column makes the expected output that constant (every one of the 512 output
     columns lands where it belongs); NaN beyond the sequences must not leak in."""
