@@ -152,12 +152,17 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<KHE
     constexpr int BN = prefillStepTokens<KHEAD, R>();
     constexpr int TT = BN / kTileTokens;             // 16-token tiles per step: 4 or 2
     constexpr int kTileChunksK = kTileTokens * G::kChunksPerRowK, kTileChunksV = kTileTokens * G::kChunksPerRowV;
-    __shared__ uint4 k_lds[2][TT * kTileChunksK];       // [tile][token][16-byte chunk, XOR-swizzled by the token]
+    struct Tiles {
+        uint4 k[2][TT * kTileChunksK]; // [tile][token][16-byte chunk, XOR-swizzled by the token]
+        uint4 v[2][TT * kTileChunksV]; // see below
+    };
+    __shared__ Tiles tiles;
+    auto &k_lds = tiles.k;
     // V tile in LDS: [row half (8 rows)][block of 16 columns (32 bytes)][row of the half][two 16-byte chunks], i.e.
     // slot = half * 8 * chunks per row + block * 16 + (row % 8) * 2 + chunk % 2. A transposing read of one block then
     // touches two runs of 256 bytes, and 64 consecutive slots (one load instruction) are four blocks of eight rows:
     // 128 contiguous bytes of each row in global memory.
-    __shared__ uint4 v_lds[2][TT * kTileChunksV];
+    auto &v_lds = tiles.v;
 
     const int lane = threadIdx.x & 63;
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -535,10 +540,10 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<KHE
     }
 
     // ---- normalise and store. A lane holds single columns (16 e + c) of its rows; the wavefront's 16 R rows pass
-    // through LDS (the K buffers: every wavefront is past the last barrier of the loop, nothing is in flight) and go
+    // through LDS (the tile buffers: every wavefront is past the last barrier of the loop, nothing is in flight) and go
     // out as 16-byte pieces, 64 lanes on consecutive pieces ----
-    static_assert(2 * TT * kTileChunksK * 16 >= 4 * R * 16 * VHEAD * 2, "the K buffers hold the output rows of all four wavefronts");
-    unsigned short *stage = reinterpret_cast<unsigned short *>(&k_lds[0][0]) + w * (R * 16 * VHEAD);
+    static_assert(sizeof(Tiles) >= 4 * R * 16 * VHEAD * 2, "the tile buffers hold the output rows of all four wavefronts");
+    unsigned short *stage = reinterpret_cast<unsigned short *>(&tiles) + w * (R * 16 * VHEAD);
 #pragma unroll
     for (int r = 0; r < R; ++r) {
 #pragma unroll
