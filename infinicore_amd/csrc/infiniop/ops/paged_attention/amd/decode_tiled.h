@@ -145,14 +145,32 @@ __device__ __forceinline__ uint4 loadLane16(const char *uniform_base, uint32_t l
 // keeps three-operand forms from fusing: the maximum of 16 scores is 10 instructions this way and 27 with fmaxf.
 __device__ __forceinline__ float maxOf(float a, float b) { return __builtin_elementwise_maximum(a, b); }
 
-// 16 bytes per lane from global memory straight into LDS, without a register in between: lane i of the wavefront
-// writes the 16 bytes at lds_base + 16 i (lds_base is the same for all lanes); lanes that are switched off write
-// nothing. The data is in LDS when the wavefront's vector-memory counter has counted the instruction off.
-// NONTEMPORAL: for data read once per call (see loadLane16).
-template <bool NONTEMPORAL = false>
-__device__ __forceinline__ void loadLane16ToLds(const char *global_src, uint4 *lds_base) {
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)global_src,
-                                     (__attribute__((address_space(3))) void *)lds_base, 16, 0, NONTEMPORAL ? 2 : 0);
+// 16 bytes per lane from global memory straight into LDS, without a register in between (global_load_lds_dwordx4):
+// lane i of the wavefront writes the 16 bytes at lds_base + 16 i (lds_base is the same for all lanes, it travels in
+// M0); lanes that are switched off write nothing. The data is in LDS when the wavefront's vector-memory counter has
+// counted the instruction off: the caller waits for that (s_waitcnt vmcnt) before anybody reads the bytes.
+// Written as assembly on purpose. Through the compiler's builtin the instruction is known to write LDS, and every
+// LDS read that follows - of any LDS address: the pass that places the waits cannot tell the buffers of a
+// double-buffered tile apart - is preceded by a wait for all of these loads, which serialises the loads of the
+// next tile with the arithmetic on the current one.
+// Source as (wave-uniform base, 32-bit lane offset) or as a pointer per lane.
+__device__ __forceinline__ void loadLane16ToLds(const char *uniform_base, uint32_t lane_offset, uint4 *lds_base) {
+    const uint32_t lds_address = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) void *)lds_base));
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :: "v"(lane_offset), "s"(uniform_base), "s"(lds_address) : "memory");
+}
+// the same with the lanes of `lanes` only (an EXEC mask: all ones, or zero for an instruction that does nothing)
+__device__ __forceinline__ void loadLane16ToLdsMasked(const char *uniform_base, uint32_t lane_offset, uint4 *lds_base,
+                                                      unsigned long long lanes) {
+    const uint32_t lds_address = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) void *)lds_base));
+    unsigned long long saved;
+    asm volatile("s_mov_b32 m0, %3\n\ts_and_saveexec_b64 %0, %4\n\tglobal_load_lds_dwordx4 %1, %2\n\ts_mov_b64 exec, %0"
+                 : "=&s"(saved) : "v"(lane_offset), "s"(uniform_base), "s"(lds_address), "s"(lanes) : "memory", "scc");
+}
+__device__ __forceinline__ void loadLane16ToLds(const char *lane_pointer, uint4 *lds_base) {
+    const uint32_t lds_address = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) void *)lds_base));
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                 :: "v"(lane_pointer), "s"(lds_address) : "memory");
 }
 
 // max over the four lanes {c, c+16, c+32, c+48}; every one of them gets the result (two lane swaps,

@@ -51,6 +51,7 @@ using op::paged_attention::amd::TileF16;
 
 using op::paged_attention::amd::kTileTokens;
 using op::paged_attention::amd::loadLane16ToLds;
+using op::paged_attention::amd::loadLane16ToLdsMasked;
 
 constexpr int kPrefillThreads = 256;
 // K / V operands are requested from LDS this many uses before the matrix instructions that take them (an LDS read
@@ -274,8 +275,39 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<KHE
     for (int j = 0; j < G::kLoadsV; ++j) {
         v_src_off[j] = vRowOfSlot(64 * j + lane) * static_cast<uint32_t>(a.v_row_stride) * sizeof(S) + 16 * vChunkOfSlot(64 * j + lane);
     }
-    auto loadStage = [&](int step) {
+    // A stage's load instructions are not issued in one burst after the barrier but one at a time between the matrix
+    // instructions of the step that follows (computeStep): a wavefront cannot issue its next direct load before the
+    // memory pipeline has taken the one before (each carries its LDS address in M0), and with every wavefront of the
+    // compute unit issuing eight at once that cost each of them ~1 us per step. loadStage(step, true) only records
+    // where the instructions of the stage read and write; issueSlot(i) issues the i-th of them (slots [0, kLoadsK)
+    // are K, the rest V; a wavefront that copies one kind only has its instructions in the first slots). A slot with
+    // nothing to do (no further stage, or a stage that took the lane-by-lane path) runs with no lane switched on.
+    constexpr int kSlots = TT == 4 ? G::kLoadsK + G::kLoadsV : (G::kLoadsK > G::kLoadsV ? G::kLoadsK : G::kLoadsV);
+    constexpr int kPendV = TT == 4 ? 1 : 0; // a wavefront that copies one kind keeps that kind's record at index 0
+    uint32_t slot_off[kSlots];              // the lane's source offset for slot i
+#pragma unroll
+    for (int i = 0; i < kSlots; ++i) {
+        if constexpr (TT == 4) {
+            slot_off[i] = i < G::kLoadsK ? k_src_off[i < G::kLoadsK ? i : 0] : v_src_off[i < G::kLoadsK ? 0 : i - G::kLoadsK];
+        } else {
+            slot_off[i] = copies_k ? k_src_off[i < G::kLoadsK ? i : 0] : v_src_off[i < G::kLoadsV ? i : 0];
+        }
+    }
+    const char *pend_src[2] = {k_head, v_head};
+    uint4 *pend_dst[2] = {&k_lds[0][0], &v_lds[0][0]};
+    unsigned long long pend_live[2] = {0ull, 0ull}; // EXEC mask of the slot's instruction: all lanes or none
+    auto issueSlot = [&](int i) {
+        if constexpr (TT == 4) {
+            const int kind = i < G::kLoadsK ? 0 : 1, inst = kind ? i - G::kLoadsK : i;
+            loadLane16ToLdsMasked(pend_src[kind], slot_off[i], pend_dst[kind] + 64 * inst, pend_live[kind]);
+        } else {
+            const bool exists = i < (copies_k ? G::kLoadsK : G::kLoadsV);
+            loadLane16ToLdsMasked(pend_src[0], slot_off[i], pend_dst[0] + 64 * i, exists ? pend_live[0] : 0ull);
+        }
+    };
+    auto loadStage = [&](int step, bool deferred) {
         // K and V: slots 64 j + lane of the tile; V rows past kv_len are zeroed.
+        pend_live[0] = pend_live[1] = 0ull;
         const int t = step * BN + kTileTokens * copy_tile;
         const int e0 = t >> a.block_shift;
         if ((min(e0, last_entry) >> 6) > id_batch) {
@@ -283,22 +315,25 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<KHE
             ++id_batch;
             ids_next = loadIdBatch(id_batch + 1);
         }
+        // Page ids first, loads after: reading an id out of its register waits for every vector-memory operation
+        // in flight (the id batch may have been loaded in an earlier trip), the tile loads just issued included.
+        const int id0 = pageOfEntry(e0), id1 = small_pages ? pageOfEntry(e0 + 1) : id0;
         if (copies_k) {
             // Rows past the end of the sequence are fetched like the others: the page they lie in exists (its id
             // is clamped to the sequence's last entry and to the pool), and whatever they hold only reaches scores
             // that the causal mask replaces.
             uint4 *k_dst = &k_lds[step & 1][copy_tile * kTileChunksK];
             if (!small_pages) {
-                const int page = pageOfEntry(e0);
-                const char *k_tile = k_head + (page * a.k_batch_stride + (t & block_mask) * a.k_row_stride) * static_cast<int64_t>(sizeof(S));
+                const char *k_tile = k_head + (id0 * a.k_batch_stride + (t & block_mask) * a.k_row_stride) * static_cast<int64_t>(sizeof(S));
+                if (deferred) {
+                    pend_src[0] = k_tile, pend_dst[0] = k_dst, pend_live[0] = ~0ull;
+                } else {
 #pragma unroll
-                for (int j = 0; j < G::kLoadsK; ++j) {
-                    uint32_t lane_off = k_src_off[j];
-                    asm volatile("" : "+v"(lane_off));
-                    loadLane16ToLds(k_tile + lane_off, k_dst + 64 * j);
+                    for (int j = 0; j < G::kLoadsK; ++j) {
+                        loadLane16ToLds(k_tile, k_src_off[j], k_dst + 64 * j);
+                    }
                 }
             } else { // pages of 8 tokens: rows 8..15 of the tile lie in the next page
-                const int id0 = pageOfEntry(e0), id1 = pageOfEntry(e0 + 1);
 #pragma unroll
                 for (int j = 0; j < G::kLoadsK; ++j) {
                     const int row = G::kRow(j, lane), slot = G::kChunk(j, lane);
@@ -314,19 +349,19 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<KHE
         }
         uint4 *v_dst = &v_lds[step & 1][copy_tile * kTileChunksV];
         if (t + kTileTokens <= kv_len && !small_pages) {
-            const int page = pageOfEntry(e0);
-            const char *v_tile = v_head + (page * a.v_batch_stride + (t & block_mask) * a.v_row_stride) * static_cast<int64_t>(sizeof(S));
+            const char *v_tile = v_head + (id0 * a.v_batch_stride + (t & block_mask) * a.v_row_stride) * static_cast<int64_t>(sizeof(S));
+            if (deferred) {
+                pend_src[kPendV] = v_tile, pend_dst[kPendV] = v_dst, pend_live[kPendV] = ~0ull;
+            } else {
 #pragma unroll
-            for (int j = 0; j < G::kLoadsV; ++j) {
-                uint32_t lane_off = v_src_off[j];
-                asm volatile("" : "+v"(lane_off));
-                loadLane16ToLds(v_tile + lane_off, v_dst + 64 * j);
+                for (int j = 0; j < G::kLoadsV; ++j) {
+                    loadLane16ToLds(v_tile, v_src_off[j], v_dst + 64 * j);
+                }
             }
             return;
         }
         // Last tile of the sequence, or two pages per tile. Rows past the sequence may hold anything (NaN included)
         // and 0 * NaN is NaN: their lanes are switched off for the load and store zeros instead.
-        const int id0 = pageOfEntry(e0), id1 = small_pages ? pageOfEntry(e0 + 1) : id0;
         const int row0 = small_pages ? 0 : (t & block_mask);
 #pragma unroll
         for (int j = 0; j < G::kLoadsV; ++j) {
@@ -409,7 +444,11 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<KHE
                     s[r][tt] = T::mfmaK32(cur, q_reg[r][kk], s[r][tt]);
                 }
                 __builtin_amdgcn_sched_group_barrier(0x008, R, 0);
+                if (idx % 2 == 1 && idx / 2 < kSlots) {
+                    issueSlot(idx / 2); // one load instruction of the next stage after every second operand
+                }
             }
+            static_assert(kOperandsK / 2 >= kSlots, "a place in the step for every load instruction of a stage");
         }
 
         uint4 p_op[R][TT / 2];
@@ -521,22 +560,27 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<KHE
     };
 
     // ---- pipeline ----
-    loadStage(0);
+    loadStage(0, false);
     awaitStage();
     __syncthreads();
-    if (n_steps > 1) {
-        loadStage(1);
-    }
     for (int j = 0; j < n_steps; ++j) {
         const int t0 = j * BN;
+        // stage j + 1 goes into the other buffer while this step computes (everybody is past step j - 1)
+        if (j + 1 < n_steps) {
+            loadStage(j + 1, true);
+        } else {
+            pend_live[0] = pend_live[1] = 0ull;
+        }
         if (t0 < wave_max_visible) {
             computeStep(j & 1, t0, t0 + BN > wave_min_visible);
+        } else {
+#pragma unroll
+            for (int i = 0; i < kSlots; ++i) {
+                issueSlot(i);
+            }
         }
         awaitStage();
         __syncthreads();
-        if (j + 2 < n_steps) {
-            loadStage(j + 2);
-        }
     }
 
     // ---- normalise and store. A lane holds single columns (16 e + c) of its rows; the wavefront's 16 R rows pass
