@@ -380,6 +380,27 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<KHE
     // the tiles asked for by the last loadStage are in LDS
     auto awaitStage = [&]() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); };
 
+    // Wavefront priorities. On a SIMD that holds wavefronts of two workgroups (heads up to 128) nothing keeps the two in
+    // different phases of their steps, and a wavefront in its softmax can hold up the matrix instructions of the other
+    // for as long as it has vector instructions ready. The two blocks of matrix instructions of a step therefore run at
+    // a higher priority than the softmax between them (a softmax then fills the issue slots that the other wavefront's
+    // matrix instructions leave free), and of two wavefronts in the same kind of phase the one in the odd hardware
+    // slot goes first, which pushes the pair apart. Bit 0 of the wavefront's slot number: HW_ID bits [3:0].
+    const bool odd_slot = (__builtin_amdgcn_s_getreg((3 << 11) | 4) & 1) != 0;
+    auto matrixPhase = [&]() {
+        if (odd_slot) {
+            __builtin_amdgcn_s_setprio(3);
+        } else {
+            __builtin_amdgcn_s_setprio(2);
+        }
+    };
+    auto vectorPhase = [&]() {
+        if (odd_slot) {
+            __builtin_amdgcn_s_setprio(1);
+        } else {
+            __builtin_amdgcn_s_setprio(0);
+        }
+    };
     // ---- softmax state ----
     // o[r][e][rr] = O[row 4g+rr of group r][column 16 e + c]; ol[r][rr] = sum of that row's probabilities
     // (computed by the matrix unit as P . 1, so it sums exactly the rounded probabilities the numerator
@@ -416,6 +437,7 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<KHE
                 s[r][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
             }
         }
+        matrixPhase();
         // K.Q^T: operand idx = (tile tt, 32 dimensions kk). The scheduler groups pin the order "one LDS read, then the
         // R matrix instructions of the operand read kAheadK earlier"; the first kAheadK reads are a group of their own.
         {
@@ -451,6 +473,7 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<KHE
             static_assert(kOperandsK / 2 >= kSlots, "a place in the step for every load instruction of a stage");
         }
 
+        vectorPhase();
         uint4 p_op[R][TT / 2];
 #pragma unroll
         for (int r = 0; r < R; ++r) {
@@ -516,6 +539,7 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<KHE
             }
         }
 
+        matrixPhase();
         // P.V: the V operands run kAhead ahead as well
         constexpr int kAhead = kOperandsAhead;
         constexpr int kOperands = (TT / 2) * G::kColsV;
@@ -557,6 +581,7 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<KHE
             }
             __builtin_amdgcn_sched_group_barrier(0x008, R, 0);
         }
+        vectorPhase();
     };
 
     // ---- pipeline ----
