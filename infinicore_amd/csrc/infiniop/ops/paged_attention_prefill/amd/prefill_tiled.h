@@ -425,6 +425,7 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<KHE
     const uint32_t one2 = T::pack2(1.0f, 1.0f);
     const uint4 ones = make_uint4(one2, one2, one2, one2);
     const float unit = PLAIN ? a.scale_log2 : 1.0f; // log2-domain size of one unit of m
+    const float lazy = kLazyLog2 / unit;             // kLazyLog2 powers of two, in units of m
 
     // One step over the BN tokens in LDS buffer `buf`. masked: some score of the step lies beyond
     // what its row may see (steps on the causal diagonal); the other steps skip the comparison.
@@ -510,7 +511,8 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<KHE
             // when some row's maximum has grown by more than 2^kLazyLog2 since, so probabilities reach at
             // most that factor above 1. Numerator and denominator carry the same reference, the quotient
             // is unchanged.
-            if (__builtin_amdgcn_ballot_w64(mx * unit > m[r] * unit + kLazyLog2 || (m[r] == -INFINITY && mx > -INFINITY)) != 0) {
+            // (a row that has seen nothing yet has m = -inf: any finite maximum is above -inf + lazy)
+            if (__builtin_amdgcn_ballot_w64(mx > m[r] + lazy) != 0) {
                 // rescale. Lane holds accumulators of rows 4g..4g+3, whose factors live in lanes 4g..4g+3.
                 const float alpha = m_new > m[r] ? fastExp2((m[r] - m_new) * unit) : 1.0f;
                 m[r] = m_new;
