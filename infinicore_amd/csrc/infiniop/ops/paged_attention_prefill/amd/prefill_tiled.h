@@ -504,15 +504,17 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<KHE
             for (int tt = 1; tt < TT; ++tt) {
                 mx = maxOf(mx, maxOf(maxOf(s[r][tt][0], s[r][tt][1]), maxOf(s[r][tt][2], s[r][tt][3])));
             }
-            mx = maxAcrossTokenGroups(mx);
-            const float m_new = maxOf(m[r], mx);
+            // mx: maximum over this lane's 4 x TT tokens; the row's maximum is the largest of its four lanes' (c, c + 16,
+            // c + 32, c + 48) and is only formed when it is needed.
             // The reference point m[r] only has to keep the exponentials in range, it need not be the
             // exact maximum: it is moved (and the accumulators rescaled, ~70 vector instructions) only
             // when some row's maximum has grown by more than 2^kLazyLog2 since, so probabilities reach at
             // most that factor above 1. Numerator and denominator carry the same reference, the quotient
             // is unchanged.
             // (a row that has seen nothing yet has m = -inf: any finite maximum is above -inf + lazy)
-            if (__builtin_amdgcn_ballot_w64(mx > m[r] + lazy) != 0) {
+            if (__builtin_amdgcn_ballot_w64(mx > m[r] + lazy) != 0) { // some lane's maximum, hence some row's
+                mx = maxAcrossTokenGroups(mx);
+                const float m_new = maxOf(m[r], mx);
                 // rescale. Lane holds accumulators of rows 4g..4g+3, whose factors live in lanes 4g..4g+3.
                 const float alpha = m_new > m[r] ? fastExp2((m[r] - m_new) * unit) : 1.0f;
                 m[r] = m_new;
