@@ -422,6 +422,12 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<KHE
     typedef __attribute__((address_space(3))) s16x4 *LdsPiece;
     const auto v_read_base = (__attribute__((address_space(3))) char *)v_lds
                            + 16 * ((g >> 1) * 8 * G::kChunksPerRowV + (4 * (g & 1) + (c >> 2)) * 2 + ((c & 3) >> 1)) + 8 * (c & 1);
+    // this lane's chunk of row c in K-step kk, within a tile (the swizzle makes it a different one per kk)
+    int k_read_index[G::kLoadsK];
+#pragma unroll
+    for (int kk = 0; kk < G::kLoadsK; ++kk) {
+        k_read_index[kk] = G::ldsIndex(c, 4 * kk + g);
+    }
     const uint32_t one2 = T::pack2(1.0f, 1.0f);
     const uint4 ones = make_uint4(one2, one2, one2, one2);
     const float unit = PLAIN ? a.scale_log2 : 1.0f; // log2-domain size of one unit of m
@@ -446,7 +452,7 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<KHE
             constexpr int kOperandsK = TT * G::kLoadsK;
             auto readK = [&](int idx) {
                 const int tt = idx / G::kLoadsK, kk = idx % G::kLoadsK;
-                return k_lds[buf][tt * kTileChunksK + G::ldsIndex(c, 4 * kk + g)];
+                return k_lds[buf][tt * kTileChunksK + k_read_index[kk]];
             };
             uint4 kf[kAheadK];
 #pragma unroll
@@ -499,11 +505,18 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<KHE
                     }
                 }
             }
-            float mx = maxOf(maxOf(s[r][0][0], s[r][0][1]), maxOf(s[r][0][2], s[r][0][3]));
+            // three-operand maxima: 4 TT values in 2 TT instructions
+            float mx = maxOf(maxOf(s[r][0][0], s[r][0][1]), s[r][0][2]);
+            mx = maxOf(maxOf(mx, s[r][0][3]), s[r][1][0]);
+            mx = maxOf(maxOf(mx, s[r][1][1]), s[r][1][2]);
 #pragma unroll
-            for (int tt = 1; tt < TT; ++tt) {
-                mx = maxOf(mx, maxOf(maxOf(s[r][tt][0], s[r][tt][1]), maxOf(s[r][tt][2], s[r][tt][3])));
+            for (int tt = 2; tt < TT; tt += 2) {
+                mx = maxOf(maxOf(mx, s[r][tt - 1][3]), s[r][tt][0]);
+                mx = maxOf(maxOf(mx, s[r][tt][1]), s[r][tt][2]);
+                mx = maxOf(maxOf(mx, s[r][tt][3]), s[r][tt + 1][0]);
+                mx = maxOf(maxOf(mx, s[r][tt + 1][1]), s[r][tt + 1][2]);
             }
+            mx = maxOf(mx, s[r][TT - 1][3]);
             // mx: maximum over this lane's 4 x TT tokens; the row's maximum is the largest of its four lanes' (c, c + 16,
             // c + 32, c + 48) and is only formed when it is needed.
             // The reference point m[r] only has to keep the exponentials in range, it need not be the
