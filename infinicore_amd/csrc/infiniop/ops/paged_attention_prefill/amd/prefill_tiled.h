@@ -408,8 +408,10 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<KHE
     // of the raw dot product when there is no ALiBi (scale > 0 keeps the order), else of the scaled score.
     f32x4 o[R][G::kColsV], ol[R];
     float m[R];
+    float shift[R]; // -m[r] in log2 units (0 while m[r] = -inf): what the exponent of a probability adds to its score
 #pragma unroll
     for (int r = 0; r < R; ++r) {
+        shift[r] = 0.0f;
 #pragma unroll
         for (int e = 0; e < G::kColsV; ++e) {
             o[r][e] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -531,6 +533,8 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<KHE
                 // rescale. Lane holds accumulators of rows 4g..4g+3, whose factors live in lanes 4g..4g+3.
                 const float alpha = m_new > m[r] ? fastExp2((m[r] - m_new) * unit) : 1.0f;
                 m[r] = m_new;
+                // a row that has seen nothing yet keeps m = -inf: subtract 0, p = 2^-inf = 0
+                shift[r] = m_new == -INFINITY ? 0.0f : -m_new * unit;
 #pragma unroll
                 for (int rr = 0; rr < 4; ++rr) {
                     const float alpha_r = __shfl(alpha, 4 * g + rr, 64);
@@ -541,16 +545,14 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<KHE
                     }
                 }
             }
-            // a row that has seen nothing yet keeps m = -inf: subtract 0, p = 2^-inf = 0
-            const float shift = m[r] == -INFINITY ? 0.0f : -m[r] * unit;
 #pragma unroll
             for (int u = 0; u < TT / 2; ++u) {
                 uint32_t wds[4];
 #pragma unroll
                 for (int h = 0; h < 2; ++h) {
                     const f32x4 x = s[r][2 * u + h];
-                    wds[2 * h] = T::pack2(fastExp2(__builtin_fmaf(x[0], unit, shift)), fastExp2(__builtin_fmaf(x[1], unit, shift)));
-                    wds[2 * h + 1] = T::pack2(fastExp2(__builtin_fmaf(x[2], unit, shift)), fastExp2(__builtin_fmaf(x[3], unit, shift)));
+                    wds[2 * h] = T::pack2(fastExp2(__builtin_fmaf(x[0], unit, shift[r])), fastExp2(__builtin_fmaf(x[1], unit, shift[r])));
+                    wds[2 * h + 1] = T::pack2(fastExp2(__builtin_fmaf(x[2], unit, shift[r])), fastExp2(__builtin_fmaf(x[3], unit, shift[r])));
                 }
                 p_op[r][u] = make_uint4(wds[0], wds[1], wds[2], wds[3]);
             }
