@@ -51,7 +51,7 @@ MEASURED_TRAFFIC = {
     "k2_append_prefill_chunk": (33_600_000, "kv_caching_k2_append_prefill_chunk_kernel_stats_and_traffic.md", "f6351eb"),
     "r2_rope_scatter_prefill_chunk": (33_550_000, "rope_paged_caching_r1_r2_kernel_stats_and_traffic.md", "1b3c6fa"),
     "r4_rope_qk_scatter_prefill_chunk": (100_530_000, "rope_paged_caching_r1_r2_kernel_stats_and_traffic.md", "1b3c6fa"),
-    "p3_llama3_8b_chunked": (511_000_000, "prefill_tiled_p3_llama3_8b_chunked_counters.md", "0dae317"),  # fetched 466.7 MB + written 44.35 MB
+    "p3_llama3_8b_chunked": (552_500_000, "prefill_tiled_p3_llama3_8b_chunked_counters.md", "60c46ff"),  # fetched 508.1 MB + written 44.35 MB
 }
 
 
