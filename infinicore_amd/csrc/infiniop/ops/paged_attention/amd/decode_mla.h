@@ -306,10 +306,11 @@ __device__ __forceinline__ void softmaxStepPair(f32x4 (&o)[COLS], float &m, floa
             sc[i] = (16 * (i >> 2) + 4 * g + (i & 3) >= valid) ? -INFINITY : sc[i];
         }
     }
-    const float mx = maxAcrossTokenGroups(maxOf(maxOf(maxOf(sc[0], sc[1]), maxOf(sc[2], sc[3])),
-                                                maxOf(maxOf(sc[4], sc[5]), maxOf(sc[6], sc[7]))));
-    const float m_new = maxOf(m, mx);
-    if (__builtin_amdgcn_ballot_w64(mx > m + kLazyRescaleLog2) != 0) {
+    // this lane's eight tokens; the head's maximum (four lanes) is only formed when it is needed (see softmaxStep)
+    const float mx_lane = maxOf(maxOf(maxOf(sc[0], sc[1]), maxOf(sc[2], sc[3])),
+                                maxOf(maxOf(sc[4], sc[5]), maxOf(sc[6], sc[7])));
+    if (__builtin_amdgcn_ballot_w64(mx_lane > m + kLazyRescaleLog2) != 0) {
+        const float m_new = maxOf(m, maxAcrossTokenGroups(mx_lane));
         // rescale (see softmaxStep). Lane holds accumulators of heads 4g..4g+3, whose factors live in
         // lanes 4g..4g+3.
         const float alpha = fastExp2(m - m_new);

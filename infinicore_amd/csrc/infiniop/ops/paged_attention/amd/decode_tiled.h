@@ -307,14 +307,16 @@ __device__ __forceinline__ void softmaxStep(f32x4 (&o)[COLS], float &m, float &l
         sc[rr] = s[rr] * scale_log2 + slope * static_cast<float>(rel_pos0 + 4 * g + rr);
         sc[rr] = (tail && 4 * g + rr >= valid) ? -INFINITY : sc[rr];
     }
-    const float mx = maxAcrossTokenGroups(maxOf(maxOf(sc[0], sc[1]), maxOf(sc[2], sc[3])));
-    const float m_new = maxOf(m, mx);
+    // this lane's four tokens; a head's maximum is the largest of its four lanes' (c, c + 16, c + 32, c + 48) and
+    // is only formed when it is needed
+    const float mx_lane = maxOf(maxOf(sc[0], sc[1]), maxOf(sc[2], sc[3]));
 
     // m only has to keep the exponentials in range, it need not be the exact maximum: it is moved (and the
     // accumulators rescaled) only when some head's maximum has outgrown it by more than 2^kLazyRescaleLog2,
     // so a probability reaches at most that factor above 1. Numerator and denominator carry the same
     // reference point, the quotient is unchanged, and the partial results stay mergeable as they are.
-    if (__builtin_amdgcn_ballot_w64(mx > m + kLazyRescaleLog2) != 0) {
+    if (__builtin_amdgcn_ballot_w64(mx_lane > m + kLazyRescaleLog2) != 0) { // some lane's maximum, hence some head's
+        const float m_new = maxOf(m, maxAcrossTokenGroups(mx_lane));
         // rescale. Lane holds accumulators of heads 4g..4g+3, whose factors live in lanes 4g..4g+3.
         const float alpha = fastExp2(m - m_new);
         l *= alpha;
