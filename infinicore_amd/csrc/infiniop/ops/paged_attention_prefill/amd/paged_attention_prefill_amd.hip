@@ -66,14 +66,16 @@ Plan makePlan(const PagedAttentionPrefillInfo &in, const device::amd::DeviceInfo
     if (rows_per_seq <= 64 || rows / 128 * static_cast<long long>(in.num_kv_heads) < resident * dev.compute_units) {
         r = 1;
     }
-    if (latent) {
-        r = 1; // the accumulators of 64 rows x 512 columns are half the register file
-    }
     if (const char *env = std::getenv("INFINIOP_AMD_PREFILL_GROUPS")) {
         const int forced = std::atoi(env);
         if (forced == 1 || forced == 2) {
             r = forced;
         }
+    }
+    if (latent) {
+        // the accumulators of 64 rows x 512 columns are half the register file: there is no kernel with two
+        // groups, whatever the knob says (grid and kernel must agree on the rows per workgroup)
+        r = 1;
     }
     plan.groups_per_wave = r;
     const size_t widest = in.head_size > in.value_size ? in.head_size : in.value_size;

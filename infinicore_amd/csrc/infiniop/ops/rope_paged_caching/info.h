@@ -78,6 +78,15 @@ struct RoPEPagedCachingInfo {
         if (!sin_desc->isContiguous() || !cos_desc->isContiguous()) {
             return INFINI_STATUS_BAD_TENSOR_STRIDES;
         }
+        // The kernel finds head h of a token at h * head_size (as the scatter it is built on does,
+        // paged_caching/cuda/kernel.cuh:70-78); the reference's RoPE would honour any head stride
+        // (rope/cuda/kernel.cuh:29-31), so heads that are padded or interleaved inside a token are refused
+        // here rather than read from the wrong place.
+        if (info.scatter.num_kv_heads > 1
+            && (k_desc->stride(1) != static_cast<ptrdiff_t>(info.scatter.head_size)
+                || v_desc->stride(1) != static_cast<ptrdiff_t>(info.scatter.v_head_size))) {
+            return INFINI_STATUS_BAD_TENSOR_STRIDES;
+        }
         info.has_query = with_query;
         if (with_query) {
             // the checks of the reference's RoPE for its x / y pair (rope.h:79-160): both given, dtype of the

@@ -65,6 +65,15 @@ CASES = [
     ("k last stride 2 (rope.h:152)", BAD_STRIDES, lambda s: mutate(s, "k", strides=(512, 128, 2))),
     ("sin padded rows (rope.h:159)", BAD_STRIDES, lambda s: mutate(s, "sin", strides=(40, 1))),
     ("positions strided", BAD_STRIDES, lambda s: mutate(s, "pos", strides=(2,))),
+    # heads of a token must follow one another (the kernel finds head h at h * head_size; rope/cuda/kernel.cuh:29-31
+    # would honour a head stride, the scatter of paged_caching/cuda/kernel.cuh:70-78 does not)
+    ("k heads padded inside a token", BAD_STRIDES, lambda s: mutate(s, "k", strides=(4 * 80, 80, 1))),
+    ("v heads interleaved with another tensor", BAD_STRIDES, lambda s: mutate(s, "v", strides=(4 * 128, 128, 1))),
+    ("valid: k and v as column slices of one projection output (token stride only)", OK,
+     lambda s: mutate(mutate(s, "k", strides=(3 * 256, 64, 1)), "v", strides=(3 * 256, 64, 1))),
+    ("valid: one KV head, any head stride", OK,
+     lambda s: mutate(mutate(mutate(mutate(s, "k", shape=(6, 1, 64), strides=(640, 80, 1)), "v", shape=(6, 1, 64)),
+                             "k_cache", shape=(8, 1, 16, 64)), "v_cache", shape=(8, 1, 16, 64))),
 ]
 
 

@@ -1,6 +1,7 @@
 """infiniopPagedAttentionNoAlloc (the call without a workspace argument: partial results in the library's own
 per-device scratch array) against infiniopPagedAttention, through the C ABI: bit-identical outputs, on two
-calls in a row of which the second is the smaller, and a clear refusal above the array's size."""
+calls in a row of which the second is the smaller, each also within atol 1e-2 / rtol 2e-3 of the CPU oracle's
+unrounded result, and a clear refusal above the array's size."""
 import ctypes
 from ctypes import c_void_p
 
@@ -14,7 +15,7 @@ from tests import capi
 pytestmark = pytest.mark.gpu
 
 
-def _both_ways(handle, cfg):
+def _both_ways(handle, cfg, oracle):
     dev = torch.device("cuda:0")
     inp = workloads.make_decode_inputs(cfg)
     q, kc, vc, bt, sl = (t.to(dev) for t in (inp.q, inp.k_cache, inp.v_cache, inp.block_tables, inp.seq_lens))
@@ -29,22 +30,27 @@ def _both_ways(handle, cfg):
                   "infiniopPagedAttentionNoAlloc")
     torch.cuda.synchronize()
     L.check_error(L.LIBINFINIOP.infiniopDestroyPagedAttentionDescriptor(op))
+    # the entry point against the oracle itself, not only against its sibling
+    _, exact = oracle.paged_attention(inp.q, inp.k_cache, inp.v_cache, inp.block_tables, inp.seq_lens, inp.scale,
+                                      num_threads=8, return_fp32=True)
+    err = (got.float().cpu() - exact).abs()
+    assert torch.all(err <= 1e-2 + 2e-3 * exact.abs()), f"{cfg.name}: max abs err {err.max().item():.4g} against the oracle"
     return want, got, size
 
 
-def test_two_calls_in_a_row_the_second_smaller(gpu_handle):
+def test_two_calls_in_a_row_the_second_smaller(gpu_handle, oracle):
     # both use partial results (sequences cut across wavefronts), so both go through the scratch array
     big = workloads.DecodeConfig("noalloc_big", torch.bfloat16, 24, 32, 8, 128, 16, 300, 3000, seed=501)
     small = workloads.DecodeConfig("noalloc_small", torch.float16, 3, 16, 4, 128, 16, 100, 900, seed=502)
     for cfg in (big, small):
-        want, got, size = _both_ways(gpu_handle, cfg)
+        want, got, size = _both_ways(gpu_handle, cfg, oracle)
         assert size > 0, "the case must need scratch to test anything"
         assert torch.equal(want.view(torch.int16), got.view(torch.int16)), cfg.name
 
 
-def test_latent_attention_goes_through_the_array_too(gpu_handle):
+def test_latent_attention_goes_through_the_array_too(gpu_handle, oracle):
     cfg = workloads.DecodeConfig("noalloc_mla", torch.bfloat16, 4, 16, 1, 576, 16, 200, 1200, seed=503, value_size=512)
-    want, got, size = _both_ways(gpu_handle, cfg)
+    want, got, size = _both_ways(gpu_handle, cfg, oracle)
     assert size > 0
     assert torch.equal(want.view(torch.int16), got.view(torch.int16))
 
