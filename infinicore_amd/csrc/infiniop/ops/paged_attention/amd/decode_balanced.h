@@ -138,14 +138,27 @@ decodeBalancedKernel(const void *early_seq_lens, int early_num_seqs, int early_m
     // FUSED: the state of the segment this wavefront is the reader of, until the end of the piece
     __shared__ float reader_stash[FUSED ? (4 * G::kCols + 2) * 64 : 1];
 
-    const int piece = blockIdx.x;
     const int head_chunks = (a.group + kHeadsPerWave - 1) / kHeadsPerWave;
-    const int kv_head = blockIdx.y / head_chunks;
-    const int chunk = blockIdx.y - kv_head * head_chunks;
+    const int streams = static_cast<int>(gridDim.y);
+    const int piece = static_cast<int>(blockIdx.x);
+    const int stream = static_cast<int>(blockIdx.y);
+    const int kv_head = stream / head_chunks;
+    const int chunk = stream - kv_head * head_chunks;
     const int lane = threadIdx.x;
     const int c = lane & 15;
     const int g = lane >> 4;
 
+    // Where this wavefront's first kLead tiles were in the previous call on this workspace, as (page, first
+    // row) pairs: requested beside the lengths, used further down to ask for those tiles one memory round trip
+    // early (see "speculative first tiles").
+    constexpr int kLead = NBUF - 1;
+    static_assert(2 * kLead <= kFirstTileInts, "an entry holds the pairs of kLead tiles");
+    int *const my_first_tiles = a.first_tiles + (static_cast<int64_t>(piece) * streams + stream) * kFirstTileInts;
+    int guess[2 * kLead];
+#pragma unroll
+    for (int i = 0; i < 2 * kLead; ++i) {
+        guess[i] = my_first_tiles[i];
+    }
     const int total_tiles = tilePrefixSums<Tindex>(early_seq_lens, early_num_seqs, early_max_blocks_per_seq,
                                                    early_block_shift, lane, pre_incl);
     // The flat range is not cut into equal tile counts but into equal COST: a sequence that begins inside
@@ -157,10 +170,15 @@ decodeBalancedKernel(const void *early_seq_lens, int early_num_seqs, int early_m
     constexpr int kStartCost = HEAD <= 128 ? 384 / HEAD : 2;
     static_assert(kStartCost <= kBalancedMaxStartCost, "the launch plan bounds the flat axis with this");
     const int q = tilesPerPiece(total_tiles + kStartCost * a.num_seqs, waves_per_stream);
-    auto pieceOf = [&](int x) { return x / q; }; // the piece that holds virtual slot x
-    // Real tiles below virtual positions x0 = piece * q and x1 = x0 + q: count the sequences that lie
+    // Pieces come in pairs (even, odd) that share 2 q slots; the even one takes q + relief of them.
+    const int relief = (q * a.odd_piece_relief) >> 8;
+    auto pieceOf = [&](int x) { // the piece that holds virtual slot x
+        const int pair = x / (2 * q);
+        return 2 * pair + (x - 2 * pair * q >= q + relief ? 1 : 0);
+    };
+    // Real tiles below virtual positions x0 and x1, the ends of this piece: count the sequences that lie
     // entirely below each (one pass over the prefix sums for both), then add the part of the next one.
-    const int x0 = piece * q, x1 = x0 + q;
+    const int x0 = piece * q + ((piece & 1) ? relief : 0), x1 = (piece + 1) * q + ((piece & 1) ? 0 : relief);
     int s0 = 0, s1 = 0;
     int first_64 = 0; // prefix sum of sequence `lane`: the first 64 are kept in a register as well
     for (int base = 0; base < a.num_seqs; base += 64) {
@@ -404,7 +422,7 @@ decodeBalancedKernel(const void *early_seq_lens, int early_num_seqs, int early_m
         }
         waitVectorMemory(); // the rows are in memory before the flag says so
         if (lane == 0) {
-            storeAgent(a.seg_flags + static_cast<int64_t>(piece + seq) * gridDim.y + blockIdx.y, a.token);
+            storeAgent(a.seg_flags + static_cast<int64_t>(piece + seq) * streams + stream, a.token);
         }
     };
 
@@ -494,7 +512,7 @@ decodeBalancedKernel(const void *early_seq_lens, int early_num_seqs, int early_m
     // Tell the merge kernel which pieces hold each sequence that starts in this piece (one writer per
     // sequence: the wavefront of the first stream whose piece contains the sequence's first tile).
     // Done before the first tile is requested, for the reason given at parkSegment.
-    if (!FUSED && blockIdx.y == 0) {
+    if (!FUSED && stream == 0) {
         for (int base = seq0; base < a.num_seqs; base += 64) {
             const int s = base + lane;
             bool more = false;
@@ -511,25 +529,58 @@ decodeBalancedKernel(const void *early_seq_lens, int early_num_seqs, int early_m
             }
         }
     }
-    // The first tiles are requested before the first query: the query's round trip then overlaps
-    // with theirs.
     const int n_flat = f1 - f0;
     TileRegs<HEAD> buf[NBUF];
+    // The first query and length go out in front of the first tiles (results come back in the order of the
+    // requests: behind the tiles they would be held up until the last tile is in).
+    const int64_t first_len64 = loadIndex<Tindex>(a.seq_lens, seq0);
+    requestQuery(seq0, q_reg);
+    // Speculative first tiles. The page ids of this piece are one more dependent round trip away (lengths ->
+    // prefix sums -> table entries -> tiles), during which the memory system would idle. The calls of one
+    // decoding step (one per layer) see the same lengths and block table, so the kLead tiles the pipeline
+    // starts with are most likely where they were in the previous call: they are requested now, from the
+    // (page, row) pairs that call left in the workspace, next to the table entries. When the entries arrive
+    // the guess is checked against them; tiles guessed right are used as they are, a wrong guess (another
+    // batch, a workspace never used before: any bit pattern, forced into the pool before it is used as an
+    // address) costs the bandwidth of the tiles and nothing else: their slots of the pipeline are skipped.
+    int guess_page[kLead], guess_row[kLead];
 #pragma unroll
-    for (int i = 0; i < NBUF - 1; ++i) {
-        buf[i] = loadNextTile();
+    for (int i = 0; i < kLead; ++i) {
+        guess_page[i] = __builtin_amdgcn_readfirstlane(guess[2 * i]);
+        guess_row[i] = __builtin_amdgcn_readfirstlane(guess[2 * i + 1]);
+        const int page = clampPage(guess_page[i], a.num_blocks);
+        const int row0 = guess_row[i] & block_mask & ~(kTileTokens - 1);
+        const char *k_tile = k_head + (page * a.k_batch_stride + row0 * a.k_row_stride) * static_cast<int64_t>(sizeof(S));
+        const char *v_tile = v_head + (page * a.v_batch_stride + row0 * a.v_row_stride) * static_cast<int64_t>(sizeof(S));
+        buf[i] = loadTileRegs<HEAD>(k_tile, v_tile, off, 0xffffffffu);
     }
-    {
-        const int64_t len64 = loadIndex<Tindex>(a.seq_lens, seq0);
-        requestQuery(seq0, q_reg);
-        pinQuery();
-        beginSegment(seq0, f0, clampLength(len64));
+    // (all of them go out before anything below waits for the table entries: left alone, the scheduler moves the
+    // first use of the entries, and with it the wait, up between the guessed tiles)
+    __builtin_amdgcn_sched_barrier(0);
+    // what the table says: only pieces whose first run is longer than kLead tiles take part (no run switch
+    // inside the guessed tiles); the others leave an entry that matches nothing
+    int true_page[kLead], true_row[kLead];
+    bool guessed = ld_run.t1 - ld_run.t0 > kLead;
+#pragma unroll
+    for (int i = 0; i < kLead; ++i) {
+        const int t = ld_run.t0 + (guessed ? i : 0);
+        true_page[i] = clampPage(__builtin_amdgcn_readlane(ld_ids, (t >> tiles_per_entry_shift) - ld_run.first_entry), a.num_blocks);
+        true_row[i] = guessed ? (t * kTileTokens) & block_mask : -1;
+        guessed = guessed && true_page[i] == guess_page[i] && true_row[i] == guess_row[i];
     }
-    for (int t = 0; t < n_flat; t += NBUF) {
+    if (guessed) {
+        ld_t += kLead; // those tiles are on their way
+    }
+    const int dead_slots = guessed ? 0 : kLead;
+    pinQuery();
+    beginSegment(seq0, f0, clampLength(first_len64));
+    // (slot s of the pipeline holds tile s - dead_slots of the piece; the slots of a wrong guess hold nothing)
+    const int n_slots = n_flat + dead_slots;
+    for (int t = 0; t < n_slots; t += NBUF) {
 #pragma unroll
         for (int i = 0; i < NBUF; ++i) {
             buf[(i + NBUF - 1) % NBUF] = loadNextTile();
-            if (t + i < n_flat) {
+            if (t + i < n_slots && t + i >= dead_slots) {
                 computeNextTile(buf[i]);
             }
         }
@@ -548,6 +599,15 @@ decodeBalancedKernel(const void *early_seq_lens, int early_num_seqs, int early_m
     if (stash_seq >= 0) {
         flushStash();
     }
+    // where this piece's first tiles were, for the next call on this workspace
+    if (lane < 2 * kLead) {
+        int word = 0;
+#pragma unroll
+        for (int i = 0; i < kLead; ++i) {
+            word = lane == 2 * i ? true_page[i] : (lane == 2 * i + 1 ? true_row[i] : word);
+        }
+        my_first_tiles[lane] = word;
+    }
     if constexpr (FUSED) {
         if (reader_seq < 0) {
             return;
@@ -556,8 +616,8 @@ decodeBalancedKernel(const void *early_seq_lens, int early_num_seqs, int early_m
         const int s = reader_seq;
         const int first_piece = pieceOf(seqFirstTile(s) + kStartCost * (s + 1)); // piece of the sequence's first tile
         const int count = piece - first_piece;                                // earlier segments, >= 1
-        const int64_t flag_stride = gridDim.y;
-        unsigned long long *flags = a.seg_flags + static_cast<int64_t>(first_piece + s) * flag_stride + blockIdx.y;
+        const int64_t flag_stride = streams;
+        unsigned long long *flags = a.seg_flags + static_cast<int64_t>(first_piece + s) * flag_stride + stream;
         bool arrived = true;
         for (int base = 0; base < count && arrived; base += 64) {
             const int idx = base + lane;
@@ -569,15 +629,16 @@ decodeBalancedKernel(const void *early_seq_lens, int early_num_seqs, int early_m
                 }
                 __builtin_amdgcn_s_sleep(1);
                 if (++spins > kReaderSpinLimit) {
-                    arrived = false; // cannot happen with in-order dispatch; never spin for ever
+                    arrived = false; // not with in-order dispatch; never spin for ever
                     break;
                 }
             }
         }
         compilerMemoryBarrier(); // the row loads below stay below the flag loads above
-        if (!arrived) {
-            return;
-        }
+        // A wait that ran out must not pass for a result: the rows of this sequence are then stored as NaN
+        // (and the flags cleared like any others, so that the next call starts clean).
+        const int merged = arrived ? count : 0;
+        const float poison = arrived ? 1.0f : __builtin_nanf("");
         TileState<HEAD> own;
 #pragma unroll
         for (int e = 0; e < G::kCols; ++e) {
@@ -596,7 +657,7 @@ decodeBalancedKernel(const void *early_seq_lens, int early_num_seqs, int early_m
         }
         if (4 * g < heads_here) { // lanes that hold at least one real head
             constexpr int kBatch = 4; // segments per round trip
-            for (int i0 = 0; i0 < count; i0 += kBatch) {
+            for (int i0 = 0; i0 < merged; i0 += kBatch) {
                 float2 ml[kBatch][4];
                 float4 v[kBatch][4][G::kCols / 4];
 #pragma unroll
@@ -637,7 +698,7 @@ decodeBalancedKernel(const void *early_seq_lens, int early_num_seqs, int early_m
             for (int rr = 0; rr < 4; ++rr) {
                 if (4 * g + rr < heads_here) {
                     S *o_ptr = static_cast<S *>(a.out) + s * a.o_stride + (first_head + 4 * g + rr) * a.o_head_stride;
-                    storeOutputRow<T, HEAD>(o_ptr, c, own, rr, 1.0f / (l_run[rr] + 1e-6f));
+                    storeOutputRow<T, HEAD>(o_ptr, c, own, rr, poison / (l_run[rr] + 1e-6f));
                 }
             }
         }

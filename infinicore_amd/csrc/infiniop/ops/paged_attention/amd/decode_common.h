@@ -37,6 +37,9 @@ struct DecodeArgs {
     // [(piece + sequence) x streams]; it holds `token` once the rows of that segment are complete in memory
     unsigned long long *seg_flags;
     unsigned long long token; // differs from call to call (a replayed graph repeats it: flags are cleared by their reader)
+    // work-equalising schedule: per wavefront [piece x stream] kFirstTileInts words, the (page, first row) pairs of
+    // the tiles its pipeline started with in the last call; any content is legal (a guess, checked before use)
+    int32_t *first_tiles;
     // 64-head latent-attention kernel only: the partition size the decode kernel settled on for this
     // call (>= partition_tokens), written by its first workgroup for the merge kernel; else nullptr
     int32_t *chosen_partition;
@@ -55,6 +58,7 @@ struct DecodeArgs {
     int32_t partition_tokens;
     int32_t max_partitions;
     int32_t compute_units; // of the device the call runs on
+    int32_t odd_piece_relief; // work-equalising schedule: odd pieces hand this many 256ths of a piece to their even neighbour
 
     // element strides
     int64_t q_stride, q_head_stride;

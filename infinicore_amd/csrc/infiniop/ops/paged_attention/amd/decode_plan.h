@@ -21,6 +21,7 @@ constexpr int kHeadsPerWave = 16;      // query heads of one KV head packed into
 constexpr int kPageIdsPerWave = 64;    // block-table entries a wavefront holds at a time, one per lane
 constexpr int kBalancedMaxSeqs = 1024; // work-equalising schedule: prefix sums of the batch live in LDS
 constexpr int kBalancedMaxStartCost = 6; // largest per-sequence start cost (in tiles) that schedule adds to its flat axis
+constexpr int kFirstTileInts = 8;      // that schedule: words per wavefront that remember where its first tiles were (32 bytes)
 constexpr int kMlaKeySize = 576;       // latent attention: key / query vector
 constexpr int kMlaValueSize = 512;     // latent attention: value / output vector
 constexpr int kMlaWideChunks = 4;      // latent attention: head chunks of 16 per workgroup of the 64-head kernel
@@ -41,10 +42,11 @@ struct Plan {
     int fallback_max_partitions;
     int dims_per_lane;     // element-wise kernel: ceil(max(head_size, value_size) / 64)
     int waves_per_stream;  // balanced: wavefronts that share the tiles of one (KV head, 16-head chunk)
-    // Workspace regions, each 256-byte aligned: [acc][m][l][pieces][flags].
-    size_t acc_bytes, ml_bytes, pieces_bytes, flags_bytes;
+    int odd_piece_relief;  // balanced: 256ths of a piece that every odd piece hands to its even neighbour
+    // Workspace regions, each 256-byte aligned: [acc][m][l][pieces][flags][first tiles].
+    size_t acc_bytes, ml_bytes, pieces_bytes, flags_bytes, first_tiles_bytes;
     size_t workspaceBytes() const {
-        return acc_bytes > 0 ? acc_bytes + 2 * ml_bytes + pieces_bytes + flags_bytes + 256 : 0;
+        return acc_bytes > 0 ? acc_bytes + 2 * ml_bytes + pieces_bytes + flags_bytes + first_tiles_bytes + 256 : 0;
     }
 };
 
@@ -68,7 +70,8 @@ inline bool launchable(const PagedAttentionInfo &in) {
 
 // Environment knobs (all optional, read at descriptor creation only): INFINIOP_AMD_PA_KERNEL=generic,
 // INFINIOP_AMD_PA_SCHEDULE=grid|balanced, INFINIOP_AMD_PA_LATENT_KERNEL=wide|narrow,
-// INFINIOP_AMD_PA_PARTITION=<tokens>, INFINIOP_AMD_PA_WAVES_PER_CU=<n>, INFINIOP_AMD_PA_MERGE=kernel|fused.
+// INFINIOP_AMD_PA_PARTITION=<tokens>, INFINIOP_AMD_PA_WAVES_PER_CU=<n>, INFINIOP_AMD_PA_MERGE=kernel|fused,
+// INFINIOP_AMD_PA_ODD_RELIEF=<256ths>.
 inline Plan makePlan(const PagedAttentionInfo &in, const device::amd::DeviceInfo &dev) {
     Plan plan{};
     const long long bs = static_cast<long long>(in.page_block_size);
@@ -170,7 +173,10 @@ inline Plan makePlan(const PagedAttentionInfo &in, const device::amd::DeviceInfo
     // as long as possible), each with an equal share of the tiles. The flat tile axis of a stream (all
     // tiles of the batch plus a start cost per sequence) is indexed with 32-bit integers.
     const bool flat_axis_fits = static_cast<long long>(in.num_seqs) * (max_tiles + kBalancedMaxStartCost) < (1LL << 30);
-    const bool can_balance = plan.tiled && !latent_head && flat_axis_fits && in.num_seqs <= static_cast<size_t>(kBalancedMaxSeqs);
+    // (an empty batch or a tensor without heads is a legal call that launches nothing: no plan to make, and the
+    // arithmetic below divides by both counts)
+    const bool can_balance = plan.tiled && !latent_head && flat_axis_fits && in.num_seqs <= static_cast<size_t>(kBalancedMaxSeqs)
+                          && in.num_seqs > 0 && stream_count > 0;
     plan.balanced = can_balance && !small_job;
     if (const char *env = std::getenv("INFINIOP_AMD_PA_SCHEDULE")) {
         if (std::strcmp(env, "grid") == 0) {
@@ -193,12 +199,30 @@ inline Plan makePlan(const PagedAttentionInfo &in, const device::amd::DeviceInfo
         plan.waves_per_stream = static_cast<int>(wps < 1 ? 1 : wps);
         rows = static_cast<size_t>(plan.waves_per_stream) + in.num_seqs;
         plan.pieces_bytes = alignUp(in.num_seqs * 2 * sizeof(int), 256);
+        // Workgroups go to the eight accelerator dies round-robin by linear id, so with an even number of pieces
+        // per stream the odd pieces run on the odd dies, and on every MI355X measured (four of them) the odd die
+        // of each pair streams the head-128 and head-192 kernels 5 - 9 % slower than the even one (per-die median
+        // time in the tile loop at the Llama-3-8B batch-32 shape: 41.5 vs 44.5 us at head 128, 63 vs 66 us at
+        // head 192; none at heads 64 and 256). Every odd piece therefore hands a fixed share of its slots, in
+        // 256ths, to its even neighbour (head 128: 55.45 -> 54.9 us at that shape, 122.0 -> 120.2 us at the
+        // long-context shape, 370 -> 362 us at the 70B share; head 192: 78.4 -> 77.4 us; heads 64 and 256 lose with
+        // any share). INFINIOP_AMD_PA_ODD_RELIEF=<0..64> overrides it, 0 switches it off.
+        plan.odd_piece_relief = in.head_size == 128 ? 16 : (in.head_size == 192 ? 12 : 0);
+        if (const char *env = std::getenv("INFINIOP_AMD_PA_ODD_RELIEF")) {
+            const int forced = std::atoi(env);
+            plan.odd_piece_relief = forced >= 0 && forced <= 64 ? forced : plan.odd_piece_relief;
+        }
+        if (plan.waves_per_stream % 2 != 0) {
+            plan.odd_piece_relief = 0; // pieces do not come in (even die, odd die) pairs
+        }
         plan.fused_merge = false;
         if (const char *env = std::getenv("INFINIOP_AMD_PA_MERGE")) {
             plan.fused_merge = std::strcmp(env, "fused") == 0;
         }
         // one flag per (row, stream), whichever way the merge runs (the knob must not change the size)
         plan.flags_bytes = alignUp(rows * static_cast<size_t>(stream_count) * sizeof(unsigned long long), 256);
+        plan.first_tiles_bytes = alignUp(static_cast<size_t>(plan.waves_per_stream) * static_cast<size_t>(stream_count)
+                                             * kFirstTileInts * sizeof(int), 256);
         // the element-wise kernel's rows are (sequence, partition): as many partitions as those rows hold
         long long fallback = static_cast<long long>(rows / in.num_seqs);
         fallback = fallback > plan.max_partitions ? plan.max_partitions : fallback;

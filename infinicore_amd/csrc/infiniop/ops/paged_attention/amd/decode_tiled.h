@@ -154,10 +154,15 @@ __device__ __forceinline__ float maxOf(float a, float b) { return __builtin_elem
 // double-buffered tile apart - is preceded by a wait for all of these loads, which serialises the loads of the
 // next tile with the arithmetic on the current one.
 // Source as (wave-uniform base, 32-bit lane offset) or as a pointer per lane.
+// The statements write M0 and say so in their clobber lists, so that the compiler never carries a value of its
+// own in M0 across them (it uses M0 for indexed register moves, lane reads and messages). M0 is a register the
+// compiler reserves, for which it warns about any clobber; the clobber is still recorded on the statement.
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
 __device__ __forceinline__ void loadLane16ToLds(const char *uniform_base, uint32_t lane_offset, uint4 *lds_base) {
     const uint32_t lds_address = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) void *)lds_base));
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                 :: "v"(lane_offset), "s"(uniform_base), "s"(lds_address) : "memory");
+                 :: "v"(lane_offset), "s"(uniform_base), "s"(lds_address) : "memory", "m0");
 }
 // the same with the lanes of `lanes` only (an EXEC mask: all ones, or zero for an instruction that does nothing)
 __device__ __forceinline__ void loadLane16ToLdsMasked(const char *uniform_base, uint32_t lane_offset, uint4 *lds_base,
@@ -165,13 +170,14 @@ __device__ __forceinline__ void loadLane16ToLdsMasked(const char *uniform_base, 
     const uint32_t lds_address = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) void *)lds_base));
     unsigned long long saved;
     asm volatile("s_mov_b32 m0, %3\n\ts_and_saveexec_b64 %0, %4\n\tglobal_load_lds_dwordx4 %1, %2\n\ts_mov_b64 exec, %0"
-                 : "=&s"(saved) : "v"(lane_offset), "s"(uniform_base), "s"(lds_address), "s"(lanes) : "memory", "scc");
+                 : "=&s"(saved) : "v"(lane_offset), "s"(uniform_base), "s"(lds_address), "s"(lanes) : "memory", "scc", "m0");
 }
 __device__ __forceinline__ void loadLane16ToLds(const char *lane_pointer, uint4 *lds_base) {
     const uint32_t lds_address = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) void *)lds_base));
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
-                 :: "v"(lane_pointer), "s"(lds_address) : "memory");
+                 :: "v"(lane_pointer), "s"(lds_address) : "memory", "m0");
 }
+#pragma clang diagnostic pop
 
 // max over the four lanes {c, c+16, c+32, c+48}; every one of them gets the result (two lane swaps,
 // no LDS traffic)

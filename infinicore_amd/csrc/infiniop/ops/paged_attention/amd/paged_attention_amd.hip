@@ -299,6 +299,7 @@ infiniStatus_t Descriptor::launch(void *workspace, void *out, const void *q, con
         a.part_l = reinterpret_cast<float *>(ws + plan.acc_bytes + plan.ml_bytes);
         a.seq_pieces = reinterpret_cast<int2 *>(ws + plan.acc_bytes + 2 * plan.ml_bytes);
         a.seg_flags = reinterpret_cast<unsigned long long *>(ws + plan.acc_bytes + 2 * plan.ml_bytes + plan.pieces_bytes);
+        a.first_tiles = reinterpret_cast<int32_t *>(ws + plan.acc_bytes + 2 * plan.ml_bytes + plan.pieces_bytes + plan.flags_bytes);
         a.token = nextToken();
         // the 64-head latent-attention kernel plans its units per call from the actual lengths and leaves the
         // partition size it chose in the first word of the pieces region, for the merge kernel
@@ -327,6 +328,7 @@ infiniStatus_t Descriptor::launch(void *workspace, void *out, const void *q, con
     a.partition_tokens = tiled ? plan.partition_tokens : plan.fallback_partition_tokens;
     a.max_partitions = tiled ? plan.max_partitions : plan.fallback_max_partitions;
     a.compute_units = device::amd::deviceInfo(device_id).compute_units;
+    a.odd_piece_relief = plan.odd_piece_relief;
     a.q_stride = in.q_stride;
     a.q_head_stride = in.q_head_stride;
     a.o_stride = in.o_stride;

@@ -93,7 +93,8 @@ def test_workspace_is_that_of_the_chosen_schedule(probe):
     c2 = probe(32, 32, 8, 128, 16, 256)
     rows = 128 + 32
     flags = rows * 8 * 8  # one 8-byte flag per (row, KV-head stream)
-    assert c2["workspace_bytes"] == rows * 32 * 128 * 4 + 2 * rows * 32 * 4 + 256 + flags + 256
+    first_tiles = 128 * 8 * 32  # 32 bytes per wavefront: where its first tiles were in the previous call
+    assert c2["workspace_bytes"] == rows * 32 * 128 * 4 + 2 * rows * 32 * 4 + 256 + flags + first_tiles + 256
     assert c2["workspace_bytes"] < 8 * 32 * 32 * 130 * 4
     # the element-wise fallback (operands that are not 16-byte aligned at run time) fits the same rows
     assert c2["fallback_max_partitions"] * 32 <= rows
@@ -106,3 +107,14 @@ def test_shapes_beyond_the_launch_limits_are_not_launchable(probe):
     assert probe(65535, 8, 8, 128, 16, 4)["launchable"]
     assert not probe(65536, 8, 8, 128, 16, 4)["launchable"]
     assert not probe(4, 65536, 65536, 128, 16, 4)["launchable"]
+
+
+@pytest.mark.parametrize("schedule", [None, "balanced", "grid"])
+def test_empty_batches_and_headless_tensors_plan_nothing(probe, monkeypatch, schedule):
+    """No sequences, or no heads: a legal call that launches nothing. The plan must not divide by either count,
+    whichever schedule the knob asks for."""
+    if schedule:
+        monkeypatch.setenv("INFINIOP_AMD_PA_SCHEDULE", schedule)
+    for seqs, heads, kv in ((0, 32, 8), (4, 0, 8), (0, 0, 8)):  # (no KV heads at all is refused at validation)
+        pl = probe(seqs, heads, kv, 128, 16, 256)
+        assert not pl["balanced"] and pl["workspace_bytes"] >= 0

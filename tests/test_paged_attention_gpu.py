@@ -733,12 +733,62 @@ def test_many_calls_on_one_workspace(gpu_handle, oracle, monkeypatch, pools, mer
     L.check_error(L.LIBINFINIOP.infiniopDestroyPagedAttentionDescriptor(op))
 
 
-@pytest.mark.parametrize("shape", ["head128", "latent64heads"])
-def test_capture_and_replay(gpu_handle, oracle, shape):
+def test_remembered_first_tiles_never_leak_into_another_batch(gpu_handle, oracle):
+    """The work-equalising kernel starts its pipeline with the tiles it guesses from what the previous call left
+    in the workspace, and checks the guess against the block table. One descriptor and workspace; between calls
+    the pages move (same lengths, another table and pool: every guess names a page that now holds other tokens),
+    then the lengths change too, then the first batch returns: every call must match the oracle of its own batch."""
+    base = custom("guess_a", torch.bfloat16, 12, 32, 8, 128, 16, 300, 2500, seed=77)
+    a = workloads.make_decode_inputs(base)
+    moved = workloads.make_decode_inputs(custom("guess_b", torch.bfloat16, 12, 32, 8, 128, 16, 300, 2500, seed=78))
+    # same lengths as `a`, the table and pool contents of `moved` where they are long enough: rebuild from a's lengths
+    b = workloads.make_decode_inputs(base)
+    perm = torch.randperm(b.k_cache.shape[0], generator=torch.Generator().manual_seed(5))
+    inverse = torch.empty_like(perm)
+    inverse[perm] = torch.arange(perm.numel())
+    b.k_cache, b.v_cache = b.k_cache[perm].contiguous(), b.v_cache[perm].contiguous()  # page i now lives at inverse[i]
+    b.block_tables = inverse[b.block_tables]
+    b.q = moved.q
+    q, k, v, bt, sl = to_device(a)
+    out = torch.zeros_like(q)
+    status, op = create_paged_attention(gpu_handle, out, q, k, v, bt, sl, None, a.scale)
+    assert status == 0
+    size = workspace_size_attention(op)
+    ws = torch.empty(size, dtype=torch.uint8, device=DEV).random_(0, 255)
+    shorter = workloads.make_decode_inputs(base)
+    shorter.seq_lens = (shorter.seq_lens * 2) // 3
+    for step, inp in enumerate([a, a, b, b, shorter, a, b]):
+        qd, kd, vd, btd, sld = to_device(inp)
+        out.zero_()
+        L.check_error(L.LIBINFINIOP.infiniopPagedAttention(op, ptr(ws), size, ptr(out), ptr(qd), ptr(kd), ptr(vd),
+                                                           ptr(btd), ptr(sld), None, None))
+        torch.cuda.synchronize()
+        want, want_f32 = oracle_of(oracle, inp, return_fp32=True)
+        assert_close(out, want, f"step {step}", want_f32)
+    L.check_error(L.LIBINFINIOP.infiniopDestroyPagedAttentionDescriptor(op))
+
+
+@pytest.mark.parametrize("relief", [0, 16, 40, 64])
+@pytest.mark.parametrize("D", [64, 128, 192])
+def test_uneven_piece_pairs(gpu_handle, oracle, monkeypatch, D, relief):
+    """Odd pieces hand a share of their slots to their even neighbours (a fixed share by default where the odd
+    accelerator dies stream slower): any share from none to a quarter of a piece must cut the batch into pieces
+    that cover every tile exactly once, and tell the merge kernel the right piece range of every sequence."""
+    monkeypatch.setenv("INFINIOP_AMD_PA_ODD_RELIEF", str(relief))
+    inp = workloads.make_decode_inputs(custom(f"relief{relief}_d{D}", torch.float16, 9, 16, 4, D, 16, 1, 4000, seed=900 + relief))
+    inp.seq_lens[0], inp.seq_lens[3] = 1, 0
+    run_case(gpu_handle, oracle, inp)
+
+
+@pytest.mark.parametrize("shape", ["head128", "head128_fused_merge", "latent64heads"])
+def test_capture_and_replay(gpu_handle, oracle, monkeypatch, shape):
     """The run call allocates nothing and never synchronises, so it can be recorded into a graph;
     every replay (with eager work in between) must reproduce the eager result. The latent-attention case
-    plans its units inside the kernel, from the lengths in device memory."""
-    if shape == "head128":
+    plans its units inside the kernel, from the lengths in device memory; with the segments merged inside the
+    decode kernel every replay carries the token of the captured call, so each must find the flags cleared."""
+    if shape == "head128_fused_merge":
+        monkeypatch.setenv("INFINIOP_AMD_PA_MERGE", "fused")
+    if shape.startswith("head128"):
         inp = workloads.make_decode_inputs(custom("graph", torch.float16, 6, 32, 8, 128, 16, 50, 1500, seed=59))
     else:
         inp = workloads.make_decode_inputs(mla("graph_latent", torch.bfloat16, 6, 64, 16, 50, 1500, seed=60))
@@ -765,10 +815,11 @@ def test_capture_and_replay(gpu_handle, oracle, shape):
     call()
     L.check_error(rt.infinirtStreamEndCapture(stream, ctypes.byref(graph)))
     L.check_error(rt.infinirtGraphInstantiate(ctypes.byref(graph_exec), graph, None, None, 0))
-    for replay in range(3):
+    for replay in range(4):
         out.zero_()
-        ws.random_(0, 255)  # eager work between replays; the workspace content must not matter
-        torch.cuda.synchronize()
+        if replay != 2:
+            ws.random_(0, 255)  # eager work between replays; the workspace content must not matter
+        torch.cuda.synchronize()  # (replay 2 runs on what replay 1 left: cleared flags, first-tile entries that match)
         L.check_error(rt.infinirtGraphLuanch(graph_exec, stream))
         L.check_error(rt.infinirtStreamSynchronize(stream))
         assert torch.equal(out, eager), f"replay {replay}"

@@ -151,7 +151,7 @@ def test_paged_attention_workspace_is_sized_for_the_planned_schedule(lib, host_a
     assert status == OK
     size = ctypes.c_size_t(0)
     lib.check_error(lib.LIBINFINIOP.infiniopGetPagedAttentionWorkspaceSize(op, ctypes.byref(size)))
-    assert 2_600_000 < size.value < 2_700_000
+    assert 2_600_000 < size.value < 2_720_000  # incl. 32 KB of first-tile entries
     lib.check_error(lib.LIBINFINIOP.infiniopDestroyPagedAttentionDescriptor(op))
 
 
