@@ -58,9 +58,10 @@ MEASURED_TRAFFIC = {
 def traffic_fields(workload):
     """``roofline.traffic`` and where the figure comes from (both None for a workload without a counter run)."""
     if workload not in MEASURED_TRAFFIC:
-        return {"traffic": None, "traffic_source": None}
+        return {"traffic": None, "traffic_profile": None, "traffic_commit": None}
     nbytes, summary, commit = MEASURED_TRAFFIC[workload]
-    return {"traffic": nbytes, "traffic_source": {"profile": "profiles/" + summary, "kernel_commit": commit}}
+    # flat string fields (not a nested object): they survive tools that keep only scalars of this line
+    return {"traffic": nbytes, "traffic_profile": "profiles/" + summary, "traffic_commit": commit}
 
 
 def parse_args():

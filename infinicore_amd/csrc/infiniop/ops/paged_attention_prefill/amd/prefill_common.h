@@ -53,6 +53,7 @@ struct SeqSpan {
     int32_t q_len;   // <= 0: nothing to do
     int32_t history; // may be negative: the first -history query tokens then see nothing
     int32_t capacity; // max_blocks_per_seq * block_size, the most tokens a row may see
+    int32_t kv_len;   // K/V tokens the sequence holds, forced into [0, capacity]
 };
 
 template <typename Tindex>
@@ -72,6 +73,7 @@ __device__ __forceinline__ SeqSpan loadSeqSpan(const PrefillArgs &a, int seq) {
     s.history = static_cast<int32_t>(history);
     const int64_t cap = static_cast<int64_t>(a.max_blocks_per_seq) * a.block_size;
     s.capacity = static_cast<int32_t>(cap > lim ? lim : cap);
+    s.kv_len = static_cast<int32_t>(kv < 0 ? 0 : (kv > s.capacity ? s.capacity : kv));
     return s;
 }
 

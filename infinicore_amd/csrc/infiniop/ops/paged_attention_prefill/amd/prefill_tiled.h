@@ -77,15 +77,19 @@ __host__ __device__ constexpr int prefillBlockRows(int r) { return 64 * r; }
 // block of the last sequence backwards, so that within a sequence the blocks that see the most
 // tokens start first. Every wavefront runs this on its own (no LDS, no barrier); all values are
 // wave-uniform. Returns false for a workgroup beyond the last block.
+// `span` receives the sequence's span as the lane that looked at it read it (lane reads: loading it again
+// would be one more memory round trip at the head of every workgroup).
 template <typename Tindex>
-__device__ __forceinline__ bool findRowBlock(const PrefillArgs &a, int lane, int block_rows, int x, int &seq, int &block) {
+__device__ __forceinline__ bool findRowBlock(const PrefillArgs &a, int lane, int block_rows, int x, int &seq, int &block,
+                                             SeqSpan &span_out) {
     int running = 0;
     for (int base = 0; base < a.num_seqs; base += 64) {
         const int idx = base + lane;
         const int s = a.num_seqs - 1 - idx;
         int nb = 0;
+        SeqSpan span{0, 0, 0, 0, 0};
         if (idx < a.num_seqs) {
-            const SeqSpan span = loadSeqSpan<Tindex>(a, s);
+            span = loadSeqSpan<Tindex>(a, s);
             const int64_t rows = static_cast<int64_t>(span.q_len) * a.group;
             nb = rows > 0 ? static_cast<int>((rows + block_rows - 1) / block_rows) : 0;
         }
@@ -103,6 +107,11 @@ __device__ __forceinline__ bool findRowBlock(const PrefillArgs &a, int lane, int
             const int nb_f = __builtin_amdgcn_readlane(nb, first);
             seq = a.num_seqs - 1 - (base + first);
             block = nb_f - 1 - (x - (incl_f - nb_f));
+            span_out.q_start = __builtin_amdgcn_readlane(span.q_start, first);
+            span_out.q_len = __builtin_amdgcn_readlane(span.q_len, first);
+            span_out.history = __builtin_amdgcn_readlane(span.history, first);
+            span_out.capacity = __builtin_amdgcn_readlane(span.capacity, first);
+            span_out.kv_len = __builtin_amdgcn_readlane(span.kv_len, first);
             return true;
         }
         running = __builtin_amdgcn_readlane(incl, 63);
@@ -176,10 +185,10 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<KHE
     const int block_index = blockIdx.x / a.num_kv_heads;
 
     int seq = 0, block = 0;
-    if (!findRowBlock<Tindex>(a, lane, BM, block_index, seq, block)) {
+    SeqSpan span;
+    if (!findRowBlock<Tindex>(a, lane, BM, block_index, seq, block, span)) {
         return;
     }
-    const SeqSpan span = loadSeqSpan<Tindex>(a, seq);
     const int total_rows = span.q_len * a.group; // > 0 here
     const int block_row0 = block * BM;
     const int last_row = min(block_row0 + BM, total_rows) - 1;
@@ -188,10 +197,8 @@ __global__ void __launch_bounds__(kPrefillThreads, (prefillWorkgroupsPerUnit<KHE
     if (block_visible <= 0) {
         return;
     }
-    int64_t kv_len64 = loadIndex<Tindex>(a.kv_lens, seq);
-    kv_len64 = kv_len64 < 0 ? 0 : (kv_len64 > span.capacity ? span.capacity : kv_len64);
     // tokens that exist; rows beyond it are zeroed in V (they may hold anything, NaN included)
-    const int kv_len = __builtin_amdgcn_readfirstlane(max(static_cast<int>(kv_len64), block_visible));
+    const int kv_len = __builtin_amdgcn_readfirstlane(max(span.kv_len, block_visible));
     const int n_steps = (block_visible + BN - 1) / BN;
 
     // ---- this lane's columns: row c of each of the wavefront's R column groups ----

@@ -226,6 +226,145 @@ __global__ void __launch_bounds__(256) ropeScatterQueryKernel(Args a, QueryArgs<
     ropeScatter<T, VEC, true>(a, qa);
 }
 
+// ---- the kernel for operands made of 16-byte units (the usual case) ----
+// The box kernel above spends a token's life waiting: position -> table rows -> stores are dependent round
+// trips, and the bulk of the bytes (the vectors themselves) is only requested in the second. Here a workgroup of
+// 256 threads takes a few whole tokens and treats their work as one flat list of items of two 16-byte units each -
+// per token the rotate items of the query heads (the unit holding the first elements of its pairs and the unit
+// holding their partners), those of the KV heads, then the copy items of V (two neighbouring units) - of which
+// thread t takes items t, t + 256, ... (ITEMS of them, all in registers). Straight-line code, no branch around
+// a load:
+//   1. the first threads ask for position and slot of the workgroup's tokens, then every thread asks for the
+//      units of all its items (none of these addresses depends on the position or the slot);
+//   2. positions and slots go through LDS to everybody; every item asks for its 16 bytes of each table row
+//      (copy items too: one instruction stream for all lanes);
+//   3. rotate (copy items pass through), store: query items to q_out, KV items to the page row the slot names.
+// So a token's bytes are in flight from the first round trip on and a thread holds ITEMS x 32 bytes of them.
+struct FlatShape {
+    int32_t items_per_token;  // (query heads + KV heads) x rotate_steps + KV heads x copy_steps
+    int32_t q_items, k_items; // query heads x rotate_steps, KV heads x rotate_steps
+    int32_t rotate_steps, copy_steps; // items of one rotated vector (table_dim / elements per unit), of one V row (units / 2)
+    int32_t tokens_per_group; // whole tokens per workgroup
+    uint32_t inv_items, inv_rotate, inv_copy; // ceil(2^32 / x): floor(n / x) = n * inv >> 32 for n, x < 2^16
+};
+
+constexpr int kFlatThreads = 256;
+constexpr int kFlatMaxTokens = 16; // tokens of one workgroup (their positions and slots sit in LDS)
+
+__device__ __forceinline__ int divideSmall(int n, uint32_t inverse) {
+    return static_cast<int>(__umulhi(static_cast<uint32_t>(n), inverse));
+}
+
+template <typename T, bool QUERY, int ITEMS>
+__global__ void __launch_bounds__(kFlatThreads) ropeScatterFlatKernel(Args a, QueryArgs<QUERY> qa, FlatShape f) {
+    using S = typename T::storage;
+    using U = Unit16<S>;
+    constexpr int kPer = U::kElements;
+    __shared__ int32_t token_pos[kFlatMaxTokens];
+    __shared__ int64_t token_slot[kFlatMaxTokens];
+    const int tid = threadIdx.x;
+    const int64_t first_token = static_cast<int64_t>(blockIdx.x) * f.tokens_per_group;
+    const int tokens_here = static_cast<int>(min(static_cast<int64_t>(f.tokens_per_group), a.num_tokens - first_token));
+
+    // 1a. position and slot of the workgroup's tokens (one thread each; the others re-read the first token's)
+    const int64_t my_token = first_token + (tid < tokens_here ? tid : 0);
+    const int64_t my_slot = a.slot_mapping[my_token];
+    const int64_t my_pos = loadPosition(a, my_token);
+    // 1b. the units of this thread's items
+    const int table_dim = a.head_size / 2;
+    const bool neox = a.neox != 0;
+    int tok[ITEMS], kind[ITEMS], head[ITEMS], first[ITEMS], second[ITEMS], table_at[ITEMS]; // kind: 0 query, 1 key, 2 value
+    bool live[ITEMS];
+    uint4 lo[ITEMS], hi[ITEMS];
+#pragma unroll
+    for (int j = 0; j < ITEMS; ++j) {
+        const int w = tid + kFlatThreads * j;
+        const int t = divideSmall(w, f.inv_items);
+        live[j] = t < tokens_here;
+        tok[j] = live[j] ? t : 0; // an item past the end re-reads the first token's and stores nothing
+        int r = w - t * f.items_per_token;
+        kind[j] = r < f.q_items ? 0 : (r < f.q_items + f.k_items ? 1 : 2);
+        r -= kind[j] == 0 ? 0 : (kind[j] == 1 ? f.q_items : f.q_items + f.k_items);
+        head[j] = divideSmall(r, kind[j] == 2 ? f.inv_copy : f.inv_rotate);
+        const int step = r - head[j] * (kind[j] == 2 ? f.copy_steps : f.rotate_steps);
+        // element offsets of the item's two units inside its vector
+        first[j] = kind[j] == 2 ? 2 * step * kPer : (neox ? step * kPer : 2 * step * kPer);
+        second[j] = kind[j] == 2 ? (2 * step + 1) * kPer : (neox ? table_dim + step * kPer : 2 * step * kPer + kPer);
+        table_at[j] = kind[j] == 2 ? 0 : step * kPer;
+        const int64_t token = first_token + tok[j];
+        const S *src = static_cast<const S *>(a.v) + token * a.v_src_token_stride + static_cast<int64_t>(head[j]) * a.value_size;
+        if (kind[j] == 1) {
+            src = static_cast<const S *>(a.k) + token * a.k_src_token_stride + static_cast<int64_t>(head[j]) * a.head_size;
+        }
+        if constexpr (QUERY) {
+            if (kind[j] == 0) {
+                src = static_cast<const S *>(qa.q) + token * qa.q_token_stride + head[j] * qa.q_head_stride;
+            }
+        }
+        lo[j] = *reinterpret_cast<const uint4 *>(src + first[j]);
+        hi[j] = *reinterpret_cast<const uint4 *>(src + second[j]);
+    }
+    // 2. positions (forced into the table) and slots to everybody
+    if (tid < tokens_here) {
+        token_pos[tid] = static_cast<int32_t>(my_pos < 0 ? 0 : (my_pos >= a.table_len ? a.table_len - 1 : my_pos));
+        token_slot[tid] = (my_slot >= 0 && my_slot < a.num_slots) ? my_slot : -1; // padding, or outside the pool: dropped
+    }
+    __syncthreads();
+    uint4 sn[ITEMS], cs[ITEMS];
+#pragma unroll
+    for (int j = 0; j < ITEMS; ++j) {
+        const int64_t at = static_cast<int64_t>(token_pos[tok[j]]) * table_dim + table_at[j];
+        sn[j] = *reinterpret_cast<const uint4 *>(static_cast<const S *>(a.sin_table) + at);
+        cs[j] = *reinterpret_cast<const uint4 *>(static_cast<const S *>(a.cos_table) + at);
+    }
+    // 3. rotate and store
+#pragma unroll
+    for (int j = 0; j < ITEMS; ++j) {
+        const U x_lo = __builtin_bit_cast(U, lo[j]), x_hi = __builtin_bit_cast(U, hi[j]);
+        const U s_ = __builtin_bit_cast(U, sn[j]), c_ = __builtin_bit_cast(U, cs[j]);
+        U y_lo, y_hi;
+        if (neox) {
+#pragma unroll
+            for (int i = 0; i < kPer; ++i) {
+                rotatePair(x_lo.e[i], x_hi.e[i], s_.e[i], c_.e[i], y_lo.e[i], y_hi.e[i]);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < kPer / 2; ++i) {
+                rotatePair(x_lo.e[2 * i], x_lo.e[2 * i + 1], s_.e[i], c_.e[i], y_lo.e[2 * i], y_lo.e[2 * i + 1]);
+                rotatePair(x_hi.e[2 * i], x_hi.e[2 * i + 1], s_.e[kPer / 2 + i], c_.e[kPer / 2 + i], y_hi.e[2 * i], y_hi.e[2 * i + 1]);
+            }
+        }
+        const uint4 out_lo = kind[j] == 2 ? lo[j] : __builtin_bit_cast(uint4, y_lo);
+        const uint4 out_hi = kind[j] == 2 ? hi[j] : __builtin_bit_cast(uint4, y_hi);
+        const int64_t token = first_token + tok[j];
+        const int64_t slot = token_slot[tok[j]];
+        int64_t page, row;
+        if (a.block_shift >= 0) {
+            page = slot >> a.block_shift;
+            row = slot & (a.block_size - 1);
+        } else {
+            page = slot / a.block_size;
+            row = slot % a.block_size;
+        }
+        S *dst = static_cast<S *>(a.v_cache) + page * a.v_block_stride + head[j] * a.v_head_stride + row * a.v_slot_stride;
+        if (kind[j] == 1) {
+            dst = static_cast<S *>(a.k_cache) + page * a.k_block_stride + head[j] * a.k_head_stride + row * a.k_slot_stride;
+        }
+        bool stores = live[j] && slot >= 0;
+        if constexpr (QUERY) {
+            if (kind[j] == 0) {
+                dst = static_cast<S *>(qa.q_out) + token * qa.q_out_token_stride + head[j] * qa.q_out_head_stride;
+                stores = live[j]; // the query of a padding token is rotated all the same
+            }
+        }
+        if (stores) {
+            *reinterpret_cast<uint4 *>(dst + first[j]) = out_lo;
+            *reinterpret_cast<uint4 *>(dst + second[j]) = out_hi;
+        }
+    }
+}
+
 // Smallest power of two >= x, at most 2^30.
 int ceilPow2(int x) {
     int p = 1;
@@ -237,8 +376,68 @@ int ceilPow2(int x) {
 
 bool multipleOf16(uint64_t x) { return (x & 15u) == 0; }
 
+uint32_t inverseOf(int x) { return static_cast<uint32_t>(((uint64_t{1} << 32) + static_cast<uint64_t>(x) - 1) / static_cast<uint64_t>(x)); }
+
+// The flat kernel if the shape fits it (16-byte units, a token's items within one workgroup's reach): true when launched.
+template <typename T>
+bool launchFlat(const Args &a, const QueryArgs<true> &qa, int rotate_steps, int copy_steps, hipStream_t stream) {
+    if (rotate_steps <= 0 || copy_steps <= 0) {
+        return false;
+    }
+    if (copy_steps % 2 != 0) {
+        return false; // a V row is an odd number of units: no pairs
+    }
+    FlatShape f{};
+    f.rotate_steps = rotate_steps;
+    f.copy_steps = copy_steps / 2;
+    const long long q_items = static_cast<long long>(qa.num_q_heads) * rotate_steps;
+    const long long k_items = static_cast<long long>(a.num_kv_heads) * rotate_steps;
+    const long long items = q_items + k_items + static_cast<long long>(a.num_kv_heads) * f.copy_steps;
+    constexpr int kMaxItems = 6; // per thread
+    if (items > kFlatThreads * kMaxItems || a.table_len > 0x7fffffff) {
+        return false;
+    }
+    f.q_items = static_cast<int32_t>(q_items);
+    f.k_items = static_cast<int32_t>(k_items);
+    f.items_per_token = static_cast<int32_t>(items);
+    // Items per thread: as few as hold one token when the call is short (a decode step is one round of workgroups
+    // whatever it does: latency counts), else about three (96 bytes in flight per thread).
+    const int at_least = static_cast<int>((items + kFlatThreads - 1) / kFlatThreads);
+    int per_thread = at_least;
+    if (a.num_tokens > 1024 && per_thread < 3) {
+        per_thread = 3;
+    }
+    per_thread = per_thread <= 3 ? per_thread : (per_thread <= 4 ? 4 : kMaxItems);
+    long long tokens = static_cast<long long>(kFlatThreads) * per_thread / items;
+    tokens = tokens > kFlatMaxTokens ? kFlatMaxTokens : tokens;
+    f.tokens_per_group = static_cast<int32_t>(tokens);
+    f.inv_items = inverseOf(f.items_per_token);
+    f.inv_rotate = inverseOf(rotate_steps);
+    f.inv_copy = inverseOf(f.copy_steps);
+    const dim3 grid(static_cast<unsigned>((a.num_tokens + tokens - 1) / tokens));
+    const bool query = qa.num_q_heads > 0;
+#define LAUNCH_FLAT(N)                                                                                              \
+    if (query) {                                                                                                    \
+        ropeScatterFlatKernel<T, true, N><<<grid, kFlatThreads, 0, stream>>>(a, qa, f);                              \
+    } else {                                                                                                        \
+        ropeScatterFlatKernel<T, false, N><<<grid, kFlatThreads, 0, stream>>>(a, QueryArgs<false>{}, f);             \
+    }
+    switch (per_thread) {
+    case 1: LAUNCH_FLAT(1) break;
+    case 2: LAUNCH_FLAT(2) break;
+    case 3: LAUNCH_FLAT(3) break;
+    case 4: LAUNCH_FLAT(4) break;
+    default: LAUNCH_FLAT(6) break;
+    }
+#undef LAUNCH_FLAT
+    return true;
+}
+
 template <typename T>
 void launch(const Args &a, QueryArgs<true> qa, bool vec, int row_steps, int rotate_steps, hipStream_t stream) {
+    if (vec && launchFlat<T>(a, qa, rotate_steps, static_cast<int>(a.value_size / (16 / sizeof(typename T::storage))), stream)) {
+        return;
+    }
     // 256-thread box: x = steps along a row, y = heads, z = tokens
     int bx = ceilPow2(row_steps);
     bx = bx > 64 ? 64 : bx;

@@ -41,8 +41,10 @@ def test_every_recorded_traffic_figure_names_a_workload_and_a_committed_profile_
         text = (ROOT / "profiles" / summary).read_text()
         assert "FETCH_SIZE" in text and "rocprofv3 --pmc" in text
         fields = bench.traffic_fields(name)
-        assert fields["traffic"] == nbytes and fields["traffic_source"]["profile"] == "profiles/" + summary
-    assert bench.traffic_fields("no_such_workload") == {"traffic": None, "traffic_source": None}
+        assert fields["traffic"] == nbytes and fields["traffic_profile"] == "profiles/" + summary
+        assert fields["traffic_commit"] == commit
+        assert all(not isinstance(v, (dict, list)) for v in fields.values())  # flat: scalars only
+    assert bench.traffic_fields("no_such_workload") == {"traffic": None, "traffic_profile": None, "traffic_commit": None}
 
 
 @pytest.mark.parametrize("name", sorted(workloads.DECODE_CONFIGS))
