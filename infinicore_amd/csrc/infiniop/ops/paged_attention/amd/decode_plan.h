@@ -215,9 +215,22 @@ inline Plan makePlan(const PagedAttentionInfo &in, const device::amd::DeviceInfo
         if (plan.waves_per_stream % 2 != 0) {
             plan.odd_piece_relief = 0; // pieces do not come in (even die, odd die) pairs
         }
-        plan.fused_merge = false;
+        // Merging inside the decode kernel saves the second launch and pays for it with the readers' dependent
+        // round trips at the end of the kernel, one batch of four segments after the other: it wins where a
+        // sequence is cut into few segments and the call is short. Measured, second kernel vs merged inside
+        // (us per call): 128 sequences of 1 024 - 8 192 tokens on 128 pieces per stream 362.3 vs 360.7 at head
+        // 128, 193.1 vs 190.9 at head 64; 32 sequences of 512 - 4 096 tokens 34.3 vs 33.1 at head 64 but 55.0 vs
+        // 56.8 at head 128 and 77.4 vs 79.6 at head 192; 8 sequences of 16 384 - 32 768 tokens 67.8 vs 70.4 at
+        // head 64; head 256 always loses (102 vs 133).
+        const long long pieces = plan.waves_per_stream;
+        plan.fused_merge = (in.head_size == 64 && pieces <= 4LL * static_cast<long long>(in.num_seqs))
+                        || (in.head_size == 128 && pieces <= static_cast<long long>(in.num_seqs));
         if (const char *env = std::getenv("INFINIOP_AMD_PA_MERGE")) {
-            plan.fused_merge = std::strcmp(env, "fused") == 0;
+            if (std::strcmp(env, "fused") == 0) {
+                plan.fused_merge = true;
+            } else if (std::strcmp(env, "kernel") == 0) {
+                plan.fused_merge = false;
+            }
         }
         // one flag per (row, stream), whichever way the merge runs (the knob must not change the size)
         plan.flags_bytes = alignUp(rows * static_cast<size_t>(stream_count) * sizeof(unsigned long long), 256);

@@ -768,6 +768,31 @@ def test_remembered_first_tiles_never_leak_into_another_batch(gpu_handle, oracle
     L.check_error(L.LIBINFINIOP.infiniopDestroyPagedAttentionDescriptor(op))
 
 
+@pytest.mark.parametrize("D,B", [(64, 40), (128, 136), (64, 136)])
+def test_batches_whose_segments_are_merged_inside_the_decode_kernel_by_default(gpu_handle, oracle, monkeypatch, D, B):
+    """No merge knob set: batches of many sequences per piece (and, at head 64, of a few pieces per sequence) are
+    merged by the decode kernel itself; they must agree with the oracle like the others, call after call on
+    one workspace."""
+    monkeypatch.delenv("INFINIOP_AMD_PA_MERGE", raising=False)
+    inp = workloads.make_decode_inputs(custom(f"default_merge_d{D}_b{B}", torch.bfloat16, B, 16, 4, D, 16, 1, 700, seed=640 + B + D))
+    inp.seq_lens[1], inp.seq_lens[5] = 0, 1
+    q, k, v, bt, sl = to_device(inp)
+    out = torch.zeros_like(q)
+    status, op = create_paged_attention(gpu_handle, out, q, k, v, bt, sl, None, inp.scale)
+    assert status == 0
+    size = workspace_size_attention(op)
+    ws = torch.empty(size, dtype=torch.uint8, device=DEV).random_(0, 255)
+    want, want_f32 = oracle.paged_attention(inp.q, inp.k_cache, inp.v_cache, inp.block_tables, inp.seq_lens, inp.scale,
+                                            num_threads=ORACLE_THREADS, return_fp32=True, out=torch.zeros_like(inp.q))
+    for call in range(4):
+        out.zero_()
+        L.check_error(L.LIBINFINIOP.infiniopPagedAttention(op, ptr(ws), size, ptr(out), ptr(q), ptr(k), ptr(v), ptr(bt),
+                                                           ptr(sl), None, None))
+        torch.cuda.synchronize()
+        assert_close(out, want, f"call {call}", want_f32)
+    L.check_error(L.LIBINFINIOP.infiniopDestroyPagedAttentionDescriptor(op))
+
+
 @pytest.mark.parametrize("relief", [0, 16, 40, 64])
 @pytest.mark.parametrize("D", [64, 128, 192])
 def test_uneven_piece_pairs(gpu_handle, oracle, monkeypatch, D, relief):
