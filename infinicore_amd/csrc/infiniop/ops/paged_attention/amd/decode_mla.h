@@ -274,6 +274,7 @@ constexpr int kMlaWideTileTokens = 32; // two halves of 16
 // K / V operands of the wide kernel are requested from LDS this many matrix instructions before the one that takes
 // them: every operand feeds a single instruction (16 clocks) and an LDS read takes several times that.
 constexpr int kMlaOperandsAhead = 6;
+constexpr int kMlaQuadOperandsAhead = 4; // the same for the four-wavefront kernel (one wavefront per SIMD)
 // The wide kernels feed the probabilities to P.V as one term in the storage dtype, as the prefill kernel does. They
 // are bound by instruction issue, not by memory, and the second term that the other decode kernels add for bf16
 // (decode_tiled.h: p = hi + lo) costs 16 more matrix and ~50 more vector instructions per wavefront and tile while the
@@ -284,7 +285,9 @@ constexpr bool kMlaWideSplitProbabilities = false;
 // first / second half; the rest as softmaxStep (decode_tiled.h). The probabilities come back as the A
 // operand of a 32-deep matrix instruction whose k index 8g + j stands for token 4g + j of the first
 // half (j < 4) or token 4g + j - 4 of the second.
-template <typename T, int COLS>
+// ACC_HALF: the accumulators o live in the accumulation half of the register file (where the matrix instructions of a
+// kernel that may use more than 256 registers keep their results).
+template <typename T, int COLS, bool ACC_HALF = false>
 __device__ __forceinline__ void softmaxStepPair(f32x4 (&o)[COLS], float &m, float &l, const f32x4 s0, const f32x4 s1, int g,
                                                 float scale_log2, float slope, int rel_pos0, int valid, uint4 &p_op,
                                                 uint4 &p_lo) {
@@ -316,13 +319,19 @@ __device__ __forceinline__ void softmaxStepPair(f32x4 (&o)[COLS], float &m, floa
         const float alpha = fastExp2(m - m_new);
         l *= alpha;
         m = m_new;
+        float alpha_r[4];
 #pragma unroll
         for (int rr = 0; rr < 4; ++rr) {
-            const float alpha_r = __shfl(alpha, 4 * g + rr, 64);
+            alpha_r[rr] = __shfl(alpha, 4 * g + rr, 64);
+        }
 #pragma unroll
-            for (int e = 0; e < COLS; ++e) {
-                o[e][rr] *= alpha_r;
+        for (int e = 0; e < COLS; ++e) {
+            f32x4 x = o[e];
+#pragma unroll
+            for (int rr = 0; rr < 4; ++rr) {
+                x[rr] *= alpha_r[rr];
             }
+            o[e] = x;
         }
     }
     uint32_t hi[4], lo[4] = {0, 0, 0, 0};
@@ -431,6 +440,41 @@ __device__ __forceinline__ WidePlan planWide(const DecodeArgs &a, int lane, int 
     return plan;
 }
 
+// Which (sequence, partition, stream = KV head x group of head chunks) a workgroup of the 64-head kernels works on, and
+// the partition size of the call. Everything depends on the workgroup only, so all its wavefronts get the same
+// answer. False: no unit for this workgroup. `len` = length of the sequence, clamped to what its block-table row can
+// hold.
+template <typename Tindex>
+__device__ __forceinline__ bool locateWideUnit(const DecodeArgs &a, int lane, int groups_of_chunks, int &seq, int &part,
+                                               int &stream, int &partition_tokens, int &len) {
+    if (a.chosen_partition != nullptr) {
+        // planned per call (see planWide): one-dimensional grid
+        const WidePlan plan = planWide<Tindex>(a, lane, a.num_kv_heads * groups_of_chunks, static_cast<int>(blockIdx.x));
+        if (blockIdx.x == 0 && threadIdx.x == 0) {
+            a.chosen_partition[0] = plan.partition_tokens; // for the merge kernel
+        }
+        if (plan.seq < 0) {
+            return false;
+        }
+        // wave-uniform by construction; saying so keeps the address arithmetic in scalar registers
+        seq = __builtin_amdgcn_readfirstlane(plan.seq);
+        part = __builtin_amdgcn_readfirstlane(plan.part);
+        stream = __builtin_amdgcn_readfirstlane(plan.stream);
+        partition_tokens = __builtin_amdgcn_readfirstlane(plan.partition_tokens);
+        len = __builtin_amdgcn_readfirstlane(plan.len); // the plan has read it already: no second round trip
+        return true;
+    }
+    // fixed partitions on a three-dimensional grid, rotated as in decodeMlaKernel
+    seq = blockIdx.z;
+    part = static_cast<int>((blockIdx.x + blockIdx.z) % gridDim.x);
+    stream = blockIdx.y;
+    partition_tokens = a.partition_tokens;
+    const int64_t len64 = loadIndex<Tindex>(a.seq_lens, seq);
+    const int64_t max_len = static_cast<int64_t>(a.max_blocks_per_seq) << a.block_shift;
+    len = static_cast<int>(len64 < max_len ? len64 : max_len);
+    return true;
+}
+
 // CHUNKS = 4: as described above. CHUNKS = 1 (16 query heads per KV head): the workgroup has a single
 // chunk and all eight wavefronts work for it - wavefront w computes the partial scores of token half
 // w % 2 over a quarter of the K-steps (5, 5, 4, 4 of the 18), all eight exchange them through LDS, and
@@ -464,30 +508,8 @@ __global__ void __launch_bounds__(kMlaWideThreads, 2) decodeMlaWideKernel(Decode
     // up to the first barrier depends on the workgroup only, so all wavefronts leave together.
     int seq, part, stream, partition_tokens;
     int len; // of the sequence, clamped to what its block-table row can hold
-    if (a.chosen_partition != nullptr) {
-        // planned per call (see planWide): one-dimensional grid
-        const WidePlan plan = planWide<Tindex>(a, lane, a.num_kv_heads * groups_of_chunks, static_cast<int>(blockIdx.x));
-        if (blockIdx.x == 0 && threadIdx.x == 0) {
-            a.chosen_partition[0] = plan.partition_tokens; // for the merge kernel
-        }
-        if (plan.seq < 0) {
-            return;
-        }
-        // wave-uniform by construction; saying so keeps the address arithmetic in scalar registers
-        seq = __builtin_amdgcn_readfirstlane(plan.seq);
-        part = __builtin_amdgcn_readfirstlane(plan.part);
-        stream = __builtin_amdgcn_readfirstlane(plan.stream);
-        partition_tokens = __builtin_amdgcn_readfirstlane(plan.partition_tokens);
-        len = __builtin_amdgcn_readfirstlane(plan.len); // the plan has read it already: no second round trip
-    } else {
-        // fixed partitions on a three-dimensional grid, rotated as in decodeMlaKernel
-        seq = blockIdx.z;
-        part = static_cast<int>((blockIdx.x + blockIdx.z) % gridDim.x);
-        stream = blockIdx.y;
-        partition_tokens = a.partition_tokens;
-        const int64_t len64 = loadIndex<Tindex>(a.seq_lens, seq);
-        const int64_t max_len = static_cast<int64_t>(a.max_blocks_per_seq) << a.block_shift;
-        len = static_cast<int>(len64 < max_len ? len64 : max_len);
+    if (!locateWideUnit<Tindex>(a, lane, groups_of_chunks, seq, part, stream, partition_tokens, len)) {
+        return;
     }
     const int kv_head = stream / groups_of_chunks;
     const int chunk_group = stream - kv_head * groups_of_chunks;
@@ -822,6 +844,391 @@ __global__ void __launch_bounds__(kMlaWideThreads, 2) decodeMlaWideKernel(Decode
                 a.part_l[slot] = l_h;
             }
         }
+    }
+}
+
+// ---- 16 query heads per wavefront, tiles straight into LDS -------------------------------------------------
+// The unit of work of decodeMlaWideKernel<.., 4> (a group of head chunks of a (partition, sequence); units planned per
+// call) with the tile pipeline of the prefill kernel (paged_attention_prefill/amd/prefill_tiled.h). WAVES = 4 (up
+// to 64 query heads per workgroup, one wavefront per SIMD) or 8 (up to 128 heads, two per SIMD: a tile fetched once
+// serves twice the heads).
+//   * Wavefront w serves head chunk w: all 18 K-steps of K . Q^T for both 16-token halves of a 32-token tile (its 16
+//     query rows in 72 registers), the softmax, and all 512 value columns (128 accumulator registers; P . V as 32
+//     matrix instructions of depth 32). Nothing is exchanged between wavefronts.
+//   * K and V tiles go from global memory straight into LDS (16 bytes per lane, no register in between),
+//     double-buffered; the first half of the wavefronts brings equal parts of the K tile, the second half of the V
+//     tile, one load instruction after every few K operands of the tile before. One workgroup barrier per tile.
+//   * K row-major with its 16-byte chunks XOR-swizzled by the row; V row-major in blocks of 16 columns, read back
+//     through the transposing LDS read (layouts: see the prefill kernel).
+//   * results leave through LDS (the tile buffers) as whole rows, 16 bytes per lane.
+template <typename T, typename Tindex, int WAVES>
+__global__ void __launch_bounds__(64 * WAVES) decodeMlaRowsKernel(DecodeArgs a) {
+    static_assert(WAVES == 4 || WAVES == 8, "one or two wavefronts per SIMD");
+    using S = typename T::storage;
+    constexpr int kSteps = kMlaKeySize / 32;      // 18 K-steps
+    constexpr int kRowK = kMlaKeySize / 8;        // 72 16-byte chunks in a K row
+    constexpr int kRowV = kMlaValueSize / 8;      // 64 in a V row
+    constexpr int kSwizzle = 8;                   // stays inside a K row: 72 is a multiple of 8
+    constexpr int kTileK = kTileTokens * kRowK;   // chunks of a 16-token half
+    constexpr int kTileV = kTileTokens * kRowV;
+    constexpr int kParts = WAVES / 4;             // wavefronts that share the copy of one half of one kind
+    constexpr int kLoadsK = kTileK / 64 / kParts; // load instructions of a wavefront that copies K: 18 or 9
+    constexpr int kLoadsV = kTileV / 64 / kParts; // V: 16 or 8
+    constexpr int kBlocks = kMlaValueSize / 16;   // 32 column blocks of 16
+    constexpr int kSlots = kLoadsK;               // load instructions of one wavefront per tile (V: the last ones empty)
+    constexpr int kOutRows = kHeadsPerWave / 2;   // output rows a wavefront stages in LDS at a time
+    constexpr int kOutPitch = kMlaValueSize + 4;  // floats between them (conflict-free column writes)
+    constexpr int kMainK = 64;                    // chunks of a K row kept in the main region of a half; the other 8 in its tail
+    constexpr int kTailK = kTileTokens * kMainK;  // first slot of the tail region
+    struct Tiles {
+        // [buffer][half] of {main [token][64 chunks], tail [token][8 chunks]}, chunks XOR-swizzled by token % 8: a load
+        // instruction fills 64 consecutive slots, i.e. the main part of one token or the tails of eight
+        uint4 k[2][2 * kTileK];
+        // [buffer][half][row half (8 rows)][block of 16 columns][row of the half][two 16-byte chunks]
+        uint4 v[2][2 * kTileV];
+    };
+    __shared__ Tiles tiles;
+    static_assert(sizeof(Tiles) >= WAVES * kOutRows * kOutPitch * sizeof(float), "the tile buffers hold the staged output rows of all wavefronts");
+
+    const int head_chunks = (a.group + kHeadsPerWave - 1) / kHeadsPerWave;
+    const int groups_of_chunks = (head_chunks + WAVES - 1) / WAVES;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    const int c = lane & 15;
+    const int g = lane >> 4;
+
+    int seq, part, stream, partition_tokens, len;
+    if (!locateWideUnit<Tindex>(a, lane, groups_of_chunks, seq, part, stream, partition_tokens, len)) {
+        return;
+    }
+    const int kv_head = stream / groups_of_chunks;
+    const int chunk = (stream - kv_head * groups_of_chunks) * WAVES + wave; // may lie beyond the last chunk: no heads
+    const int start = part * partition_tokens;
+    if (len <= 0 || start >= len) {
+        return;
+    }
+    const int end = min(len, start + partition_tokens);
+    const int n_tiles = (end - start + kMlaWideTileTokens - 1) / kMlaWideTileTokens;
+
+    const int first_entry = start >> a.block_shift;
+    const int last_entry = (end - 1) >> a.block_shift;
+    int page_ids = 0;
+    if (first_entry + lane <= last_entry) {
+        page_ids = clampPage(
+            loadIndex<Tindex>(a.block_tables, seq * a.block_table_batch_stride + first_entry + lane), a.num_blocks);
+    }
+
+    // Query of head (chunk*16 + c): columns 32 kk + 8g .. +7, the B operand of K-step kk
+    const int head_in_group = chunk * kHeadsPerWave + c;
+    const bool head_valid = head_in_group < a.group;
+    const int head = kv_head * a.group + head_in_group;
+    uint4 q_reg[kSteps];
+    {
+        const S *q_ptr = static_cast<const S *>(a.q) + seq * a.q_stride + (head_valid ? head : 0) * a.q_head_stride;
+        const uint32_t keep = head_valid ? 0xffffffffu : 0u;
+#pragma unroll
+        for (int kk = 0; kk < kSteps; ++kk) {
+            uint4 x = *reinterpret_cast<const uint4 *>(q_ptr + 32 * kk + 8 * g);
+            x.x &= keep, x.y &= keep, x.z &= keep, x.w &= keep;
+            q_reg[kk] = x;
+        }
+    }
+    const float slope = (a.alibi_slopes != nullptr && head_valid) ? a.alibi_slopes[head] * kLog2e : 0.0f;
+
+    // ---- copy side: wavefront w < WAVES / 2 brings part w of the K tile, wavefront WAVES / 2 + w part w of the V
+    // tile; a part is a half (16 tokens, inside one page) or, with eight wavefronts, eight rows of one ----
+    const bool copies_k = wave < WAVES / 2;
+    const int copy_part = wave % (WAVES / 2);
+    const int copy_half = copy_part / kParts;
+    const int copy_sub = copy_part % kParts;
+    const char *copy_head = copies_k
+        ? reinterpret_cast<const char *>(static_cast<const S *>(a.k_cache) + kv_head * a.k_head_stride)
+        : reinterpret_cast<const char *>(static_cast<const S *>(a.v_cache) + kv_head * a.v_head_stride);
+    const int64_t copy_batch_stride = copies_k ? a.k_batch_stride : a.v_batch_stride;
+    const int64_t copy_row_stride = copies_k ? a.k_row_stride : a.v_row_stride;
+    const int copy_loads = copies_k ? kLoadsK : kLoadsV;
+    const int block_mask = a.block_size - 1;
+    // Load instruction j of a wavefront fills LDS slots [slot0(j), slot0(j) + 64) of its half, lane i the i-th, from
+    // (row(j) of the half, uniform) + (this lane's piece). With R = 8 copy_sub the wavefront's first row:
+    //   K, j < rows:  the main part of row R + j: slot0 = 64 (R + j); lane asks for chunk lane ^ (row % 8)
+    //   K, j >= rows: the tails of rows R + 8 (j - rows) .. + 7: slot0 = tail + 8 (that row); lane asks for chunk
+    //                 64 + (lane % 8 ^ row % 8) of row (that row) + lane / 8
+    //   V:            slot0 = 512 copy_sub + 64 j: row 8 (copy_sub + j / 8) + (lane % 16) / 2, chunk 8 (j % 8) +
+    //                 2 (lane / 16) + lane % 2 (the layout at Tiles)
+    // so two registers hold every lane-dependent offset (lane_main, XORed with a constant per instruction, and
+    // lane_tail) and the rest is scalar arithmetic.
+    constexpr int kRowsK = 16 / kParts; // rows of the half this wavefront copies (K)
+    const uint32_t k_row_bytes = static_cast<uint32_t>(a.k_row_stride) * sizeof(S);
+    const uint32_t v_row_bytes = static_cast<uint32_t>(a.v_row_stride) * sizeof(S);
+    const int copy_row0 = kRowsK * copy_sub;
+    const uint32_t lane_main = copies_k ? 16u * lane : ((lane & 15) >> 1) * v_row_bytes + 16u * (2 * (lane >> 4) + (lane & 1));
+    const uint32_t lane_tail = (lane >> 3) * k_row_bytes + 16u * (kMainK + ((lane & 7) ^ (lane >> 3))); // rows R + 8 q + lane / 8: same row % 8 as lane / 8
+    auto slotLaneOffset = [&](int j) -> uint32_t {
+        if (!copies_k) {
+            return lane_main;
+        }
+        return j < kRowsK ? (lane_main ^ (16u * ((copy_row0 + j) & (kSwizzle - 1)))) : lane_tail;
+    };
+    auto slotRowOffset = [&](int j) -> uint32_t { // uniform part, bytes
+        if (!copies_k) {
+            return (8 * (copy_sub + (kParts == 1 ? j / 8 : 0))) * v_row_bytes + 128u * (j % 8);
+        }
+        return (j < kRowsK ? copy_row0 + j : copy_row0 + 8 * (j - kRowsK)) * k_row_bytes;
+    };
+    auto slotLds = [&](int j) -> int { // first slot within the half
+        if (!copies_k) {
+            return 512 * copy_sub + 64 * j;
+        }
+        return j < kRowsK ? kMainK * (copy_row0 + j) : kTailK + 8 * (copy_row0 + 8 * (j - kRowsK));
+    };
+    auto vRowOfLoad = [&](int j) { return 8 * (copy_sub + (kParts == 1 ? j / 8 : 0)) + ((lane & 15) >> 1); };
+    // The load instructions of a tile are not issued in one burst after the barrier but one at a time between the
+    // matrix instructions of the tile before (see the prefill kernel): stageTile records where they read and write,
+    // issueSlot(i) issues the i-th. A half that ends beyond the partition takes the lane-by-lane path at once: K rows
+    // beyond the end are not needed (their scores are replaced), V rows beyond it are zeroed (they may hold anything,
+    // NaN included, and 0 * NaN is NaN).
+    const char *pend_src = copy_head;
+    uint4 *pend_dst = &tiles.k[0][0];
+    unsigned long long pend_live = 0ull;
+    auto issueSlot = [&](int i) {
+        loadLane16ToLdsMasked(pend_src + slotRowOffset(i), slotLaneOffset(i), pend_dst + slotLds(i), i < copy_loads ? pend_live : 0ull);
+    };
+    // true: the stage is exactly copy_loads load instructions of this wavefront (what a counted wait relies on)
+    auto stageTile = [&](int t, bool deferred) -> bool {
+        pend_live = 0ull;
+        const int tok0 = start + t * kMlaWideTileTokens + kTileTokens * copy_half;
+        uint4 *dst = copies_k ? &tiles.k[t & 1][copy_half * kTileK] : &tiles.v[t & 1][copy_half * kTileV];
+        if (tok0 >= end) {
+            if (!copies_k) { // nothing of this half is used, but what P . V multiplies by zero has to be finite
+#pragma unroll
+                for (int j = 0; j < kLoadsV; ++j) {
+                    dst[slotLds(j) + lane] = make_uint4(0, 0, 0, 0);
+                }
+            }
+            return false;
+        }
+        const int page = __builtin_amdgcn_readlane(page_ids, (tok0 >> a.block_shift) - first_entry);
+        const char *src = copy_head + (page * copy_batch_stride + (tok0 & block_mask) * copy_row_stride) * static_cast<int64_t>(sizeof(S));
+        if (copies_k || tok0 + kTileTokens <= end) {
+            if (deferred) {
+                pend_src = src, pend_dst = dst, pend_live = ~0ull;
+            } else {
+#pragma unroll
+                for (int j = 0; j < kSlots; ++j) {
+                    if (j < copy_loads) {
+                        loadLane16ToLds(src + slotRowOffset(j), slotLaneOffset(j), dst + slotLds(j));
+                    }
+                }
+            }
+            return true;
+        }
+#pragma unroll
+        for (int j = 0; j < kLoadsV; ++j) {
+            if (tok0 + vRowOfLoad(j) < end) {
+                loadLane16ToLds(src + slotRowOffset(j) + slotLaneOffset(j), dst + slotLds(j));
+            } else {
+                dst[slotLds(j) + lane] = make_uint4(0, 0, 0, 0);
+            }
+        }
+        return false;
+    };
+
+    // o[e][r] = O[head 4g + r of the chunk][column 16 e + c]
+    f32x4 o[kBlocks];
+#pragma unroll
+    for (int e = 0; e < kBlocks; ++e) {
+        o[e] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    float m = -INFINITY; // reference point of head c's exponentials (same value in the four lanes g = 0..3)
+    float l = 0.0f;      // sum of rounded probabilities of head c over this lane's tokens only
+
+    // this lane's chunk of row c in K-step kk, within a half: chunk 4 kk + g of the row, XOR-swizzled, i.e.
+    // 8 (kk / 2) + ((4 (kk % 2) + g) ^ (c % 8)), in the main region up to K-step 15 and in the tail after
+    const int k_read_index[2] = {c * kMainK + (g ^ (c & (kSwizzle - 1))), c * kMainK + ((4 + g) ^ (c & (kSwizzle - 1)))};
+    const int k_read_tail = kTailK + c * 8 - c * kMainK; // added to k_read_index for the last two K-steps
+    // this lane's piece of a transposing V read, relative to block 0 of half 0 of buffer 0: lane (g, c) points at
+    // token 4g + c / 4, columns 16 e + 4 (c % 4) .. + 3 and receives tokens 4g .. 4g + 3 of column 16 e + c
+    typedef short s16x4 __attribute__((ext_vector_type(4)));
+    typedef __attribute__((address_space(3))) s16x4 *LdsPiece;
+    const auto v_read_base = (__attribute__((address_space(3))) char *)tiles.v
+                           + 16 * ((g >> 1) * 8 * kRowV + (4 * (g & 1) + (c >> 2)) * 2 + ((c & 3) >> 1)) + 8 * (c & 1);
+
+    f32x4 s0, s1; // raw scores of head c for tokens 4g .. 4g + 3 of the first / second half of the tile
+    auto computeScores = [&](int buf) {
+        // K . Q^T: operand idx = (K-step idx / 2, half idx % 2); independent chains: four with one wavefront per SIMD,
+        // two with two (the registers are needed, and the other wavefront fills the gaps)
+        constexpr int kChains = WAVES == 4 ? 2 : 1; // per half
+        f32x4 sp[2][2] = {{{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}}, {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}}};
+        {
+            constexpr int kAhead = WAVES == 4 ? kMlaQuadOperandsAhead : 2;
+            constexpr int kOperands = 2 * kSteps;
+            constexpr int kEvery = kOperands / kSlots; // one load instruction of the next tile after every so many operands
+            auto readK = [&](int idx) {
+                const int kk = idx >> 1;
+                const int in_half = kk < 2 * (kMainK / 8) ? 8 * (kk >> 1) + k_read_index[kk & 1] : k_read_index[kk & 1] + k_read_tail;
+                return tiles.k[buf][(idx & 1) * kTileK + in_half];
+            };
+            uint4 kf[kAhead];
+#pragma unroll
+            for (int i = 0; i < kAhead; ++i) {
+                kf[i] = readK(i);
+            }
+            __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 0);
+#pragma unroll
+            for (int idx = 0; idx < kOperands; ++idx) {
+                const uint4 cur = kf[idx % kAhead];
+                if (idx + kAhead < kOperands) {
+                    kf[idx % kAhead] = readK(idx + kAhead);
+                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                }
+                const int kk = idx >> 1;
+                sp[idx & 1][kk % kChains] = T::mfmaK32(cur, q_reg[kk], sp[idx & 1][kk % kChains]);
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                if (idx % kEvery == kEvery - 1) {
+                    issueSlot(idx / kEvery); // V wavefronts: one load instruction of the next V tile
+                }
+            }
+            static_assert(kOperands % kSlots == 0, "a place in the tile for every load instruction of the next");
+        }
+        s0 = kChains == 2 ? sp[0][0] + sp[0][1] : sp[0][0], s1 = kChains == 2 ? sp[1][0] + sp[1][1] : sp[1][0];
+    };
+    auto computeValues = [&](int buf, int t) {
+        const int tok0 = start + t * kMlaWideTileTokens;
+        const int valid = min(kMlaWideTileTokens, end - tok0);
+        uint4 p_op, p_lo;
+        softmaxStepPair<T, kBlocks>(o, m, l, s0, s1, g, a.scale_log2, slope, tok0 - (len - 1), valid, p_op, p_lo);
+
+        // P . V: operand e = V[32 tokens][columns 16 e .. 16 e + 15]: two transposing reads, one per half
+        constexpr int kAhead = WAVES == 4 ? kMlaQuadOperandsAhead : 2;
+        constexpr int kEveryV = kBlocks / kSlots; // one load instruction after every so many operands
+        auto readV = [&](int e) {
+            const auto base = v_read_base + buf * (2 * kTileV * 16) + 256 * e;
+            const uint2 lo = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<LdsPiece>(base)));
+            const uint2 hi = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<LdsPiece>(base + kTileV * 16)));
+            return make_uint4(lo.x, lo.y, hi.x, hi.y);
+        };
+        uint4 vf[kAhead];
+#pragma unroll
+        for (int i = 0; i < kAhead; ++i) {
+            vf[i] = readV(i);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x100, 2 * kAhead, 0);
+#pragma unroll
+        for (int e = 0; e < kBlocks; ++e) {
+            const uint4 cur = vf[e % kAhead];
+            if (e + kAhead < kBlocks) {
+                vf[e % kAhead] = readV(e + kAhead);
+                __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+            }
+            o[e] = T::mfmaK32(p_op, cur, o[e]);
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            if (e % kEveryV == kEveryV - 1 && e / kEveryV < kSlots) {
+                issueSlot(e / kEveryV); // K wavefronts: one load instruction of the K tile after the next
+            }
+        }
+    };
+
+    // ---- pipeline. K tiles and V tiles are double-buffered separately and a tile has two barriers:
+    //   A(t): K(t) is in LDS and everybody is past P . V of tile t - 1  -> the V wavefronts ask for V(t + 1) (between
+    //         the matrix instructions of K . Q^T), whose buffer P . V of tile t - 1 was the last to read;
+    //   B(t): V(t) is in LDS and everybody is past K . Q^T of tile t    -> the K wavefronts ask for K(t + 2) (between
+    //         the matrix instructions of P . V), whose buffer K . Q^T of tile t was the last to read.
+    // A tile is thus asked for a tile and a half before it is needed. A wavefront's loads come back in the order
+    // issued, so waiting until no more than the load instructions of the younger stage are outstanding means the
+    // older stage has landed; where the younger stage is not exactly that many instructions (the ragged end of a
+    // partition) the wait is for everything.
+    auto awaitOlderStage = [&](bool younger_is_whole) {
+        if (younger_is_whole) {
+            if (copies_k) {
+                asm volatile("s_waitcnt vmcnt(%0)" :: "n"(kLoadsK) : "memory");
+            } else {
+                asm volatile("s_waitcnt vmcnt(%0)" :: "n"(kLoadsV) : "memory");
+            }
+        } else {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        }
+    };
+    bool younger_whole = false; // of this wavefront's kind: the stage in flight behind the one it waits for next
+    stageTile(0, false);
+    if (copies_k && n_tiles > 1) {
+        younger_whole = stageTile(1, false);
+    }
+    for (int t = 0; t < n_tiles; ++t) {
+        if (copies_k) {
+            awaitOlderStage(younger_whole); // K(t); K(t + 1) may still be on its way
+        }
+        __syncthreads(); // A(t)
+        pend_live = 0ull;
+        if (!copies_k && t + 1 < n_tiles) {
+            younger_whole = stageTile(t + 1, true);
+        } else if (!copies_k) {
+            younger_whole = false;
+        }
+        computeScores(t & 1);
+        if (!copies_k) {
+            awaitOlderStage(younger_whole); // V(t); V(t + 1) has just been asked for
+        }
+        __syncthreads(); // B(t)
+        pend_live = 0ull;
+        if (copies_k && t + 2 < n_tiles) {
+            younger_whole = stageTile(t + 2, true);
+        } else if (copies_k) {
+            younger_whole = false;
+        }
+        computeValues(t & 1, t);
+    }
+    __syncthreads(); // everybody is past the last tile: the buffers are free
+
+    // ---- epilogue: a lane holds single columns (16 e + c) of heads 4g .. 4g + 3; the wavefront's 16 rows pass through
+    // LDS, eight at a time (heads 4g + 2 pass + {0, 1}), and leave as 16-byte pieces, 64 lanes on consecutive pieces ----
+    const float l_tot = sumAcrossTokenGroups(l);
+    const bool single = len <= partition_tokens;
+    float *stage = reinterpret_cast<float *>(&tiles) + wave * (kOutRows * kOutPitch);
+    const int heads_here = min(kHeadsPerWave, a.group - chunk * kHeadsPerWave); // <= 0: a chunk beyond the last
+    const int out_head0 = kv_head * a.group + chunk * kHeadsPerWave;
+#pragma unroll
+    for (int pass = 0; pass < 2; ++pass) {
+#pragma unroll
+        for (int rr = 0; rr < 2; ++rr) {
+            float *row = stage + (2 * g + rr) * kOutPitch + c;
+#pragma unroll
+            for (int e = 0; e < kBlocks; ++e) {
+                row[16 * e] = o[e][2 * pass + rr];
+            }
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // the wavefront's own stores have landed before its lanes read each other's
+#pragma unroll
+        for (int lr = 0; lr < kOutRows; ++lr) {
+            const int r = 4 * (lr >> 1) + 2 * pass + (lr & 1); // head of the chunk in staged row lr
+            if (r >= heads_here) {
+                continue;
+            }
+            if (single) { // one row per instruction: 64 lanes x 8 columns
+                const float inv_l = 1.0f / (__shfl(l_tot, r, 64) + 1e-6f);
+                const float4 x = *reinterpret_cast<const float4 *>(stage + lr * kOutPitch + 8 * lane);
+                const float4 y = *reinterpret_cast<const float4 *>(stage + lr * kOutPitch + 8 * lane + 4);
+                uint4 w;
+                w.x = T::pack2(x.x * inv_l, x.y * inv_l);
+                w.y = T::pack2(x.z * inv_l, x.w * inv_l);
+                w.z = T::pack2(y.x * inv_l, y.y * inv_l);
+                w.w = T::pack2(y.z * inv_l, y.w * inv_l);
+                S *o_ptr = static_cast<S *>(a.out) + seq * a.o_stride + (out_head0 + r) * a.o_head_stride;
+                *reinterpret_cast<uint4 *>(o_ptr + 8 * lane) = w;
+            } else { // half a row per instruction: 64 lanes x 4 columns
+                const int64_t slot = (static_cast<int64_t>(seq) * a.num_heads + out_head0 + r) * a.max_partitions + part;
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const int col = 256 * h + 4 * lane;
+                    *reinterpret_cast<float4 *>(a.part_acc + slot * kMlaValueSize + col) = *reinterpret_cast<const float4 *>(stage + lr * kOutPitch + col);
+                }
+            }
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // read back before the second pass overwrites the rows
+    }
+    if (!single && g == 0 && c < heads_here) {
+        const int64_t slot = (static_cast<int64_t>(seq) * a.num_heads + out_head0 + c) * a.max_partitions + part;
+        a.part_m[slot] = m;
+        a.part_l[slot] = l_tot;
     }
 }
 

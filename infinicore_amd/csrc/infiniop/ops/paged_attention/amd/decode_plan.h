@@ -27,6 +27,15 @@ constexpr int kMlaValueSize = 512;     // latent attention: value / output vecto
 constexpr int kMlaWideChunks = 4;      // latent attention: head chunks of 16 per workgroup of the 64-head kernel
 constexpr size_t kGridLimitYZ = 65535; // largest y / z extent of a launch
 
+// Latent attention, more than 16 query heads per KV head: head chunks of 16 that share a workgroup (and with it every
+// K / V tile it fetches), one wavefront each.
+inline int latentChunksPerWorkgroup(long long head_chunks) {
+    if (const char *env = std::getenv("PA_MLA_CHUNKS")) {
+        return std::atoi(env) == 8 ? 8 : 4;
+    }
+    return head_chunks > kMlaWideChunks ? 8 : kMlaWideChunks;
+}
+
 struct Plan {
     bool tiled;            // tiled matrix-core kernel (head 64 / 128 / 192 / 256 or 576 with values of 512, power-of-two pages >= 16, 16-byte aligned strides)
     bool balanced;         // tiled kernel under the work-equalising schedule (decode_balanced.h)
@@ -128,12 +137,16 @@ inline Plan makePlan(const PagedAttentionInfo &in, const device::amd::DeviceInfo
             plan.latent_wide = false;
         }
     }
+    const long long chunks_per_group = latentChunksPerWorkgroup(head_chunks);
     const long long wide_units = static_cast<long long>(in.num_seqs) * in.num_kv_heads
-                               * ((head_chunks + kMlaWideChunks - 1) / kMlaWideChunks);
+                               * ((head_chunks + chunks_per_group - 1) / chunks_per_group);
     long long want = plan.latent_wide ? wide_units * max_tokens / dev.compute_units
                    : latent_head      ? units * max_tokens * 3 / (16LL * dev.compute_units)
                    : small_job        ? units * max_tokens / (8LL * dev.compute_units)
                                       : units * max_tokens / (16LL * dev.compute_units);
+    if (const char *env = std::getenv("PA_MLA_WANT_DIV")) {
+        want /= std::atoi(env) > 0 ? std::atoi(env) : 1;
+    }
     long long p = floorPow2(want < 1 ? 1 : want);
     const long long p_min = plan.latent_wide ? 128 : (latent_head ? 256 : 64);
     p = p < p_min ? p_min : (p > 512 ? 512 : p);

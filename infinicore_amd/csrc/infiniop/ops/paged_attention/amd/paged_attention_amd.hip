@@ -97,9 +97,10 @@ void launchAll(const DecodeArgs &a, const Plan &plan, bool tiled, hipStream_t st
             const int head_chunks = (a.group + kHeadsPerWave - 1) / kHeadsPerWave;
             const dim3 grid(plan.max_partitions, a.num_kv_heads * head_chunks, a.num_seqs);
             if (plan.latent_wide) {
-                // a single chunk of 16 heads gets the whole workgroup; otherwise four chunks share one
+                // a single chunk of 16 heads gets the whole workgroup; otherwise a wavefront per chunk, four or eight
                 const bool one_chunk = head_chunks == 1;
-                const int groups_of_chunks = one_chunk ? 1 : (head_chunks + kMlaWideChunks - 1) / kMlaWideChunks;
+                const int chunks_per_group = latentChunksPerWorkgroup(head_chunks);
+                const int groups_of_chunks = (head_chunks + chunks_per_group - 1) / chunks_per_group;
                 const int streams = a.num_kv_heads * groups_of_chunks;
                 dim3 wide(plan.max_partitions, streams, a.num_seqs);
                 if (a.chosen_partition != nullptr) {
@@ -109,8 +110,12 @@ void launchAll(const DecodeArgs &a, const Plan &plan, bool tiled, hipStream_t st
                 }
                 if (one_chunk) {
                     decodeMlaWideKernel<T, Tindex, 1><<<wide, kMlaWideThreads, 0, stream>>>(a);
-                } else {
+                } else if (std::getenv("PA_MLA_OLD") != nullptr) {
                     decodeMlaWideKernel<T, Tindex, kMlaWideChunks><<<wide, kMlaWideThreads, 0, stream>>>(a);
+                } else if (chunks_per_group == 8) {
+                    decodeMlaRowsKernel<T, Tindex, 8><<<wide, 512, 0, stream>>>(a);
+                } else {
+                    decodeMlaRowsKernel<T, Tindex, 4><<<wide, 256, 0, stream>>>(a);
                 }
                 break;
             }
