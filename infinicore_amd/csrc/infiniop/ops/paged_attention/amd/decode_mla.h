@@ -1,9 +1,10 @@
 // Tiled decode kernels for latent-attention caches: head_size 576 (512 latent + 64 rotary columns),
 // value_size 512, the shape of the reference's dedicated kernel
 // (src/infiniop/ops/paged_attention/nvidia/paged_attention_mla_hd576_v512.cu). gfx950, 64-lane wavefronts.
-// Two kernels: decodeMlaKernel (16 query heads per workgroup of two wavefronts, described first) and
-// decodeMlaWideKernel (up to 64 query heads per workgroup of eight, for more than 16 heads per KV head;
-// further down).
+// Three kernels: decodeMlaKernel (16 query heads per workgroup of two wavefronts, described first),
+// decodeMlaChunkKernel (the same 16 heads on a workgroup of eight wavefronts, for batches too small to fill the
+// device with pairs) and decodeMlaRowsKernel (more than 16 heads per KV head: 64 or 128 per workgroup, a wavefront per
+// 16); further down.
 //
 // Unit of work and arithmetic are those of the head-128 tiled kernel (decode_tiled.h): one unit = one
 // (partition, KV head x 16 query heads, sequence), tiles of 16 tokens, K . Q^T and P . V on the matrix
@@ -252,33 +253,32 @@ __global__ void __launch_bounds__(kMlaThreads, 2) decodeMlaKernel(DecodeArgs a) 
     }
 }
 
-// ---- many query heads per KV head ---------------------------------------------------------------------
-// With more than 16 query heads per KV head the kernel above fetches every K / V tile once per 16 heads
-// (from L2) and each pair of wavefronts moves a whole tile through its own registers. The kernel below
-// gives a workgroup of EIGHT wavefronts 64 query heads of one (partition, sequence): a K / V tile of 32
-// tokens (two halves of 16, each inside one page) is fetched once for all of them and shared through
-// LDS, double-buffered.
+// ---- workgroups of eight wavefronts on tiles of 32 tokens ------------------------------------------------
+// decodeMlaChunkKernel gives the 16 query heads of one (partition, sequence) a workgroup of EIGHT wavefronts; a K / V
+// tile of 32 tokens (two halves of 16, each inside one page) goes through LDS, double-buffered.
 //   * copy: wavefronts 0..3 fetch the V tile, one 128-column quarter each (lane (g, c): token rows
 //     4g..4g+3 of both halves, one 8-column strip), and store it already transposed into matrix-operand
 //     order (per column, the eight tokens of a lane as one 16-byte word); wavefronts 4..7 fetch the K
 //     tile as flat 16-byte chunks (nine load instructions each, every one inside one half) and store it
 //     row-major with a pitch of 73 chunks (conflict-free for both the row-major writes and the
 //     column-of-16-rows reads).
-//   * compute: wavefront w works for head chunk w % 4 (16 heads); the two wavefronts of a chunk split
-//     the 18 K-steps of K . Q^T (9 each, their query slice in registers) and exchange the partial
-//     scores through LDS, run the same softmax, and own 256 value columns each (64 accumulator
-//     registers; P . V as 32-deep matrix instructions). Two workgroup barriers per tile.
-// Partial results and their merge are those of the kernel above.
+//   * compute: wavefront w computes the partial scores of token half w % 2 over a quarter of the K-steps (5, 5, 4, 4
+//     of the 18; its query slice in registers), all eight exchange them through LDS, run the same softmax, and each
+//     owns 64 value columns (16 accumulator registers; P . V as 32-deep matrix instructions). Two workgroup
+//     barriers per tile.
+// Partial results and their merge are those of the kernel above. (More than 16 heads per KV head: decodeMlaRowsKernel,
+// at the end of the file.)
 constexpr int kMlaWideThreads = 512;
 constexpr int kMlaWideTileTokens = 32; // two halves of 16
-// K / V operands of the wide kernel are requested from LDS this many matrix instructions before the one that takes
+// K / V operands of these kernels are requested from LDS this many matrix instructions before the one that takes
 // them: every operand feeds a single instruction (16 clocks) and an LDS read takes several times that.
-constexpr int kMlaOperandsAhead = 6;
-constexpr int kMlaQuadOperandsAhead = 4; // the same for the four-wavefront kernel (one wavefront per SIMD)
-// The wide kernels feed the probabilities to P.V as one term in the storage dtype, as the prefill kernel does. They
-// are bound by instruction issue, not by memory, and the second term that the other decode kernels add for bf16
-// (decode_tiled.h: p = hi + lo) costs 16 more matrix and ~50 more vector instructions per wavefront and tile while the
-// largest error against the fp32 oracle at the 128-head shape moves from 0.96e-3 to 1.01e-3 (77 -> 73 us per call).
+constexpr int kMlaOperandsAhead = 6;     // decodeMlaChunkKernel
+constexpr int kMlaQuadOperandsAhead = 4; // decodeMlaRowsKernel with one wavefront per SIMD (two with two)
+// The kernels on 32-token tiles feed the probabilities to P.V as one term in the storage dtype, as the prefill kernel
+// does. They are bound by LDS traffic and instruction issue, not by memory, and the second term that the other decode
+// kernels add for bf16 (decode_tiled.h: p = hi + lo) costs 16 more matrix and ~50 more vector instructions per
+// wavefront and tile while the largest error against the fp32 oracle at the 128-head shape moves from 0.96e-3 to
+// 1.01e-3 (77 -> 73 us per call with the kernel of the time).
 constexpr bool kMlaWideSplitProbabilities = false;
 
 // Online-softmax step of one 32-token tile. s0 / s1 = raw scores of head c for tokens 4g..4g+3 of the
@@ -362,7 +362,7 @@ __device__ __forceinline__ void softmaxStepPair(f32x4 (&o)[COLS], float &m, floa
 //     results);
 //   * the (sequence, partition) units are numbered densely; linear workgroup id = 8 streams (u / 8) +
 //     8 stream + u % 8, so the units that exist come first, the dies get equal shares, and the workgroups
-//     of one unit (one per 64 heads) sit on the same die and meet in its L2.
+//     of one unit (one per group of head chunks) sit on the same die and meet in its L2.
 struct WidePlan {
     int partition_tokens;
     int seq, part, stream; // this workgroup's unit; seq < 0: none
@@ -475,19 +475,12 @@ __device__ __forceinline__ bool locateWideUnit(const DecodeArgs &a, int lane, in
     return true;
 }
 
-// CHUNKS = 4: as described above. CHUNKS = 1 (16 query heads per KV head): the workgroup has a single
-// chunk and all eight wavefronts work for it - wavefront w computes the partial scores of token half
-// w % 2 over a quarter of the K-steps (5, 5, 4, 4 of the 18), all eight exchange them through LDS, and
-// each owns 64 value columns (16 accumulator registers). The copy side is the same.
-template <typename T, typename Tindex, int CHUNKS>
-__global__ void __launch_bounds__(kMlaWideThreads, 2) decodeMlaWideKernel(DecodeArgs a) {
-    static_assert(CHUNKS == 1 || CHUNKS == kMlaWideChunks, "one chunk or four per workgroup");
-    constexpr bool kOne = CHUNKS == 1;
-    constexpr int kOwnSteps = kOne ? 5 : 9;   // K-steps of one wavefront (the last of the five may be empty)
-    constexpr int kOwnBlocks = kOne ? 4 : 16; // 16-column blocks of one wavefront
+template <typename T, typename Tindex>
+__global__ void __launch_bounds__(kMlaWideThreads, 2) decodeMlaChunkKernel(DecodeArgs a) {
+    constexpr int kOwnSteps = 5;  // K-steps of one wavefront (the last of the five may be empty)
+    constexpr int kOwnBlocks = 4; // 16-column blocks of one wavefront
     using S = typename T::storage;
     constexpr int kSteps = kMlaKeySize / 32;        // 18
-    constexpr int kHalfSteps = kSteps / 2;          // K-steps per wavefront
     constexpr int kChunksPerRow = kMlaKeySize / 8;  // 72 16-byte chunks in a K row
     constexpr int kPitch = kChunksPerRow + 1;
     constexpr int kHalfChunks = kTileTokens * kChunksPerRow; // 1152 chunks in a half
@@ -495,16 +488,16 @@ __global__ void __launch_bounds__(kMlaWideThreads, 2) decodeMlaWideKernel(Decode
     constexpr int kBlocks = kMlaValueSize / 16;              // 32 column blocks of 16
     __shared__ uint4 k_lds[2][kMlaWideTileTokens * kPitch];
     __shared__ uint4 v_lds[2][kBlocks * 64];  // [column block][token group g][lane c]: .xy first half, .zw second
-    __shared__ f32x4 s_lds[8][kOne ? 1 : 2][64]; // partial scores of every wavefront (CHUNKS = 4: both halves)
+    __shared__ f32x4 s_lds[8][64]; // partial scores of every wavefront
 
     const int head_chunks = (a.group + kHeadsPerWave - 1) / kHeadsPerWave;
-    const int groups_of_chunks = (head_chunks + CHUNKS - 1) / CHUNKS;
+    const int groups_of_chunks = head_chunks; // a workgroup per chunk
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int lane = threadIdx.x & 63;
     const int c = lane & 15;
     const int g = lane >> 4;
 
-    // Which (sequence, partition, KV head x group of four head chunks) this workgroup works on. Everything
+    // Which (sequence, partition, KV head x head chunk) this workgroup works on. Everything
     // up to the first barrier depends on the workgroup only, so all wavefronts leave together.
     int seq, part, stream, partition_tokens;
     int len; // of the sequence, clamped to what its block-table row can hold
@@ -512,13 +505,11 @@ __global__ void __launch_bounds__(kMlaWideThreads, 2) decodeMlaWideKernel(Decode
         return;
     }
     const int kv_head = stream / groups_of_chunks;
-    const int chunk_group = stream - kv_head * groups_of_chunks;
-    const int chunk = kOne ? chunk_group : chunk_group * kMlaWideChunks + (wave & 3); // may lie beyond the last chunk: no heads
-    const int kh = wave >> 2; // CHUNKS = 4: half of the K-steps and half of the value columns
+    const int chunk = stream - kv_head * groups_of_chunks;
     // this wavefront's K-steps: [first_step, first_step + own_steps)
-    const int first_step = kOne ? (wave >> 1) * 5 - ((wave >> 1) == 3 ? 1 : 0) : kh * kHalfSteps;
-    const int own_steps = kOne ? ((wave >> 1) < 2 ? 5 : 4) : kHalfSteps;
-    const int th = wave & 1; // CHUNKS = 1: the token half whose scores this wavefront computes
+    const int first_step = (wave >> 1) * 5 - ((wave >> 1) == 3 ? 1 : 0);
+    const int own_steps = (wave >> 1) < 2 ? 5 : 4;
+    const int th = wave & 1; // the token half whose scores this wavefront computes
 
     const int start = part * partition_tokens;
     if (len <= 0 || start >= len) {
@@ -535,7 +526,7 @@ __global__ void __launch_bounds__(kMlaWideThreads, 2) decodeMlaWideKernel(Decode
             loadIndex<Tindex>(a.block_tables, seq * a.block_table_batch_stride + first_entry + lane), a.num_blocks);
     }
 
-    // Query of head (chunk*16 + c): columns 288 kh + 32 i + 8g .. +7, the B operand of this wavefront's K-steps
+    // Query of head (chunk*16 + c): columns 32 (first_step + i) + 8g .. +7, the B operand of this wavefront's K-steps
     const int head_in_group = chunk * kHeadsPerWave + c;
     const bool head_valid = head_in_group < a.group;
     const int head = kv_head * a.group + head_in_group;
@@ -658,14 +649,13 @@ __global__ void __launch_bounds__(kMlaWideThreads, 2) decodeMlaWideKernel(Decode
         }
     };
 
-    // CHUNKS = 4: o[e][r] = O[head 4g + r of the chunk][column 256 kh + 128 (e / 8) + 8 c + e % 8]
-    // CHUNKS = 1: o[e][r] = O[head 4g + r][column 128 (wave / 2) + 8 c + 4 (wave % 2) + e]
+    // o[e][r] = O[head 4g + r][column 128 (wave / 2) + 8 c + 4 (wave % 2) + e]
     f32x4 o[kOwnBlocks];
 #pragma unroll
     for (int e = 0; e < kOwnBlocks; ++e) {
         o[e] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
-    const int first_block = kOne ? 4 * wave : 16 * kh;
+    const int first_block = 4 * wave;
     float m = -INFINITY; // reference point of head c's exponentials (same value in the four lanes g = 0..3)
     float l = 0.0f;      // sum of rounded probabilities of head c over this lane's tokens only
 
@@ -693,37 +683,7 @@ __global__ void __launch_bounds__(kMlaWideThreads, 2) decodeMlaWideKernel(Decode
         }
         loadStage(t + 1 + kSets, next_set);
         f32x4 s0, s1;
-        if constexpr (!kOne) {
-            // partial scores of both halves over this wavefront's K-steps: four independent chains (a
-            // matrix instruction that accumulates into the result of the previous one waits ~44 cycles
-            // for it, an independent one issues after 16)
-            f32x4 sp[2][2] = {{{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}}, {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}}};
-            // operand idx = (K-step idx / 2, token half idx % 2), requested kMlaOperandsAhead uses ahead
-            constexpr int kOperands = 2 * kOwnSteps;
-            auto readK = [&](int idx) { return k_lds[buf][(16 * (idx & 1) + c) * kPitch + 4 * (first_step + (idx >> 1)) + g]; };
-            uint4 kf[kOperands];
-#pragma unroll
-            for (int idx = 0; idx < kMlaOperandsAhead; ++idx) {
-                kf[idx] = readK(idx);
-            }
-            __builtin_amdgcn_sched_group_barrier(0x100, kMlaOperandsAhead, 0);
-#pragma unroll
-            for (int idx = 0; idx < kOperands; ++idx) {
-                if (idx + kMlaOperandsAhead < kOperands) {
-                    kf[idx + kMlaOperandsAhead] = readK(idx + kMlaOperandsAhead);
-                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-                }
-                const int i = idx >> 1;
-                sp[idx & 1][i & 1] = T::mfmaK32(kf[idx], q_reg[i], sp[idx & 1][i & 1]);
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            }
-            s0 = sp[0][0] + sp[0][1], s1 = sp[1][0] + sp[1][1];
-            s_lds[wave][0][lane] = s0;
-            s_lds[wave][1][lane] = s1;
-            __syncthreads(); // partial scores of both K halves are there
-            s0 += s_lds[wave ^ 4][0][lane];
-            s1 += s_lds[wave ^ 4][1][lane];
-        } else {
+        {
             // partial scores of this wavefront's token half over its quarter of the K-steps
             f32x4 sp[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
             auto readK = [&](int i) { return k_lds[buf][(16 * th + c) * kPitch + 4 * min(first_step + i, kSteps - 1) + g]; };
@@ -743,10 +703,10 @@ __global__ void __launch_bounds__(kMlaWideThreads, 2) decodeMlaWideKernel(Decode
                 sp[i & 1] = T::mfmaK32(kf[i], q_reg[i], sp[i & 1]);
                 __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
             }
-            s_lds[wave][0][lane] = sp[0] + sp[1];
+            s_lds[wave][lane] = sp[0] + sp[1];
             __syncthreads(); // all eight partial tiles are there: wavefront 2 q + h holds quarter q of half h
-            s0 = (s_lds[0][0][lane] + s_lds[2][0][lane]) + (s_lds[4][0][lane] + s_lds[6][0][lane]);
-            s1 = (s_lds[1][0][lane] + s_lds[3][0][lane]) + (s_lds[5][0][lane] + s_lds[7][0][lane]);
+            s0 = (s_lds[0][lane] + s_lds[2][lane]) + (s_lds[4][lane] + s_lds[6][lane]);
+            s1 = (s_lds[1][lane] + s_lds[3][lane]) + (s_lds[5][lane] + s_lds[7][lane]);
         }
 
         const int tok0 = start + t * kMlaWideTileTokens;
@@ -798,48 +758,19 @@ __global__ void __launch_bounds__(kMlaWideThreads, 2) decodeMlaWideKernel(Decode
             continue;
         }
         const int out_head = kv_head * a.group + hg;
-        if constexpr (kOne) {
-            const int col0 = 128 * (wave >> 1) + 8 * c + 4 * (wave & 1);
-            if (single) {
-                const float inv_l = 1.0f / (l_h + 1e-6f);
-                S *o_ptr = static_cast<S *>(a.out) + seq * a.o_stride + out_head * a.o_head_stride + col0;
-                uint2 w;
-                w.x = T::pack2(o[0][rr] * inv_l, o[1][rr] * inv_l);
-                w.y = T::pack2(o[2][rr] * inv_l, o[3][rr] * inv_l);
-                *reinterpret_cast<uint2 *>(o_ptr) = w;
-            } else {
-                const int64_t slot = (static_cast<int64_t>(seq) * a.num_heads + out_head) * a.max_partitions + part;
-                float *dst = a.part_acc + slot * kMlaValueSize + col0;
-                *reinterpret_cast<float4 *>(dst) = make_float4(o[0][rr], o[1][rr], o[2][rr], o[3][rr]);
-                if (c == 0 && wave == 0) {
-                    a.part_m[slot] = m_h;
-                    a.part_l[slot] = l_h;
-                }
-            }
-            continue;
-        }
-        const int col0 = 256 * kh + 8 * c;
+        const int col0 = 128 * (wave >> 1) + 8 * c + 4 * (wave & 1);
         if (single) {
             const float inv_l = 1.0f / (l_h + 1e-6f);
             S *o_ptr = static_cast<S *>(a.out) + seq * a.o_stride + out_head * a.o_head_stride + col0;
-#pragma unroll
-            for (int i = 0; i < kOwnBlocks / 8; ++i) {
-                uint4 w;
-                w.x = T::pack2(o[8 * i + 0][rr] * inv_l, o[8 * i + 1][rr] * inv_l);
-                w.y = T::pack2(o[8 * i + 2][rr] * inv_l, o[8 * i + 3][rr] * inv_l);
-                w.z = T::pack2(o[8 * i + 4][rr] * inv_l, o[8 * i + 5][rr] * inv_l);
-                w.w = T::pack2(o[8 * i + 6][rr] * inv_l, o[8 * i + 7][rr] * inv_l);
-                *reinterpret_cast<uint4 *>(o_ptr + 128 * i) = w;
-            }
+            uint2 w;
+            w.x = T::pack2(o[0][rr] * inv_l, o[1][rr] * inv_l);
+            w.y = T::pack2(o[2][rr] * inv_l, o[3][rr] * inv_l);
+            *reinterpret_cast<uint2 *>(o_ptr) = w;
         } else {
             const int64_t slot = (static_cast<int64_t>(seq) * a.num_heads + out_head) * a.max_partitions + part;
             float *dst = a.part_acc + slot * kMlaValueSize + col0;
-#pragma unroll
-            for (int i = 0; i < kOwnBlocks / 8; ++i) {
-                reinterpret_cast<float4 *>(dst + 128 * i)[0] = make_float4(o[8 * i + 0][rr], o[8 * i + 1][rr], o[8 * i + 2][rr], o[8 * i + 3][rr]);
-                reinterpret_cast<float4 *>(dst + 128 * i)[1] = make_float4(o[8 * i + 4][rr], o[8 * i + 5][rr], o[8 * i + 6][rr], o[8 * i + 7][rr]);
-            }
-            if (c == 0 && kh == 0) {
+            *reinterpret_cast<float4 *>(dst) = make_float4(o[0][rr], o[1][rr], o[2][rr], o[3][rr]);
+            if (c == 0 && wave == 0) {
                 a.part_m[slot] = m_h;
                 a.part_l[slot] = l_h;
             }
@@ -848,10 +779,11 @@ __global__ void __launch_bounds__(kMlaWideThreads, 2) decodeMlaWideKernel(Decode
 }
 
 // ---- 16 query heads per wavefront, tiles straight into LDS -------------------------------------------------
-// The unit of work of decodeMlaWideKernel<.., 4> (a group of head chunks of a (partition, sequence); units planned per
-// call) with the tile pipeline of the prefill kernel (paged_attention_prefill/amd/prefill_tiled.h). WAVES = 4 (up
-// to 64 query heads per workgroup, one wavefront per SIMD) or 8 (up to 128 heads, two per SIMD: a tile fetched once
-// serves twice the heads).
+// More than 16 query heads per KV head. The unit of work is a group of WAVES head chunks of a (partition, sequence),
+// units planned per call like those of decodeMlaChunkKernel; the tile pipeline is that of the prefill kernel
+// (paged_attention_prefill/amd/prefill_tiled.h). WAVES = 4 (up to 64 query heads per workgroup, one wavefront per
+// SIMD) or 8 (up to 128 heads, two per SIMD: a tile fetched once serves twice the heads; the faster one where the
+// batch fills the device without cutting the sequences finely, decode_plan.h).
 //   * Wavefront w serves head chunk w: all 18 K-steps of K . Q^T for both 16-token halves of a 32-token tile (its 16
 //     query rows in 72 registers), the softmax, and all 512 value columns (128 accumulator registers; P . V as 32
 //     matrix instructions of depth 32). Nothing is exchanged between wavefronts.

@@ -24,23 +24,14 @@ constexpr int kBalancedMaxStartCost = 6; // largest per-sequence start cost (in 
 constexpr int kFirstTileInts = 8;      // that schedule: words per wavefront that remember where its first tiles were (32 bytes)
 constexpr int kMlaKeySize = 576;       // latent attention: key / query vector
 constexpr int kMlaValueSize = 512;     // latent attention: value / output vector
-constexpr int kMlaWideChunks = 4;      // latent attention: head chunks of 16 per workgroup of the 64-head kernel
 constexpr size_t kGridLimitYZ = 65535; // largest y / z extent of a launch
-
-// Latent attention, more than 16 query heads per KV head: head chunks of 16 that share a workgroup (and with it every
-// K / V tile it fetches), one wavefront each.
-inline int latentChunksPerWorkgroup(long long head_chunks) {
-    if (const char *env = std::getenv("PA_MLA_CHUNKS")) {
-        return std::atoi(env) == 8 ? 8 : 4;
-    }
-    return head_chunks > kMlaWideChunks ? 8 : kMlaWideChunks;
-}
 
 struct Plan {
     bool tiled;            // tiled matrix-core kernel (head 64 / 128 / 192 / 256 or 576 with values of 512, power-of-two pages >= 16, 16-byte aligned strides)
     bool balanced;         // tiled kernel under the work-equalising schedule (decode_balanced.h)
     bool fused_merge;      // balanced: segments merged inside the decode kernel (no second launch)
-    bool latent_wide;      // latent attention with more than 16 query heads per KV head: up to 64 heads per workgroup
+    bool latent_wide;      // latent attention on 32-token tiles shared through LDS, units planned per call (decode_mla.h)
+    int latent_chunks;     // that kernel: 16-head chunks that share a workgroup: 1 (eight wavefronts for the one chunk), 4 or 8 (a wavefront each)
     bool partition_forced; // INFINIOP_AMD_PA_PARTITION set: the 64-head kernel keeps exactly that size
     int partition_tokens;  // grid schedule: tokens per unit of work
     int max_partitions;    // grid schedule: partitions the longest representable sequence needs
@@ -78,7 +69,7 @@ inline bool launchable(const PagedAttentionInfo &in) {
 }
 
 // Environment knobs (all optional, read at descriptor creation only): INFINIOP_AMD_PA_KERNEL=generic,
-// INFINIOP_AMD_PA_SCHEDULE=grid|balanced, INFINIOP_AMD_PA_LATENT_KERNEL=wide|narrow,
+// INFINIOP_AMD_PA_SCHEDULE=grid|balanced, INFINIOP_AMD_PA_LATENT_KERNEL=wide|narrow, INFINIOP_AMD_PA_LATENT_HEADS=64|128,
 // INFINIOP_AMD_PA_PARTITION=<tokens>, INFINIOP_AMD_PA_WAVES_PER_CU=<n>, INFINIOP_AMD_PA_MERGE=kernel|fused,
 // INFINIOP_AMD_PA_ODD_RELIEF=<256ths>.
 inline Plan makePlan(const PagedAttentionInfo &in, const device::amd::DeviceInfo &dev) {
@@ -119,15 +110,19 @@ inline Plan makePlan(const PagedAttentionInfo &in, const device::amd::DeviceInfo
     // A unit of the latent-attention kernel leaves 32 KiB of partial results and advances one tile per
     // ~2 us however many units there are: fewer, longer units measured best there (more units end the
     // decode kernel sooner, but writing and merging their partial results costs more than that gains).
-    // Latent attention with more than one 16-head chunk per KV head runs up to 64 heads per workgroup
-    // (measured against the 16-head units, 32 sequences: 16 heads 54.4 vs 40.7 us, 32 heads 58.1 vs 62.0,
-    // 48 heads 60 vs 82, 64 heads 64 vs 104, 128 heads 83 vs 165; 128 sequences of 32 heads 163 vs 245, of
-    // 128 heads 314 vs 708). One workgroup per compute unit there, up to 128 KiB of partial results each:
-    // about one round of workgroups measured best.
+    // Latent attention with more than one 16-head chunk per KV head shares every K / V tile between the chunks of a
+    // workgroup, a wavefront per chunk (decodeMlaRowsKernel; measured against the 16-head units, 32 sequences, with
+    // the first kernel of the kind: 32 heads 58.1 vs 62.0 us, 48 heads 60 vs 82, 64 heads 64 vs 104, 128 heads 83 vs
+    // 165). One workgroup per compute unit there, up to 256 KiB of partial results each: about one round of
+    // workgroups measured best. Four chunks (64 heads) per workgroup, or eight where there are more than four and the
+    // batch fills the device without cutting the sequences finely: with eight a tile is fetched once for twice the
+    // heads, but a unit leaves twice the partial results and there are half as many units to fill the device with
+    // (128 heads, 4 vs 8 chunks: 32 sequences 70.2 vs 72.2 us, 64 sequences 136.7 vs 112.0, 128 sequences 276 vs 212,
+    // 256 sequences 523 vs 425).
     const long long head_chunks = (group + kHeadsPerWave - 1) / kHeadsPerWave;
-    // A single chunk gets all eight wavefronts of such a workgroup (decodeMlaWideKernel<.., 1>) up to 64
-    // sequences x KV heads (16 heads, 1 / 4 / 16 / 32 sequences: 16.0 / 18.9 / 26.2 / 37.8 vs 28.8 / 29.8 /
-    // 31.5 / 39.1 us on the 16-head units; 128 sequences: 135.8 vs 134.1).
+    // A single chunk gets all eight wavefronts of a workgroup (decodeMlaChunkKernel) up to 64 sequences x KV
+    // heads (16 heads, 1 / 4 / 16 / 32 sequences: 16.0 / 18.9 / 26.2 / 37.8 vs 28.8 / 29.8 / 31.5 / 39.1 us on the
+    // 16-head units; 128 sequences: 135.8 vs 134.1).
     plan.latent_wide = plan.tiled && latent_head
                     && (head_chunks > 1 || static_cast<long long>(in.num_seqs) * in.num_kv_heads <= 64);
     if (const char *env = std::getenv("INFINIOP_AMD_PA_LATENT_KERNEL")) {
@@ -137,16 +132,19 @@ inline Plan makePlan(const PagedAttentionInfo &in, const device::amd::DeviceInfo
             plan.latent_wide = false;
         }
     }
-    const long long chunks_per_group = latentChunksPerWorkgroup(head_chunks);
+    plan.latent_chunks = head_chunks <= 1 ? 1 : ((head_chunks > 4 && static_cast<long long>(in.num_seqs) * in.num_kv_heads >= 48) ? 8 : 4);
+    if (const char *env = std::getenv("INFINIOP_AMD_PA_LATENT_HEADS")) {
+        if (head_chunks > 1 && (std::atoi(env) == 64 || std::atoi(env) == 128)) {
+            plan.latent_chunks = std::atoi(env) / kHeadsPerWave;
+        }
+    }
+    const long long chunks_per_group = plan.latent_chunks;
     const long long wide_units = static_cast<long long>(in.num_seqs) * in.num_kv_heads
                                * ((head_chunks + chunks_per_group - 1) / chunks_per_group);
     long long want = plan.latent_wide ? wide_units * max_tokens / dev.compute_units
                    : latent_head      ? units * max_tokens * 3 / (16LL * dev.compute_units)
                    : small_job        ? units * max_tokens / (8LL * dev.compute_units)
                                       : units * max_tokens / (16LL * dev.compute_units);
-    if (const char *env = std::getenv("PA_MLA_WANT_DIV")) {
-        want /= std::atoi(env) > 0 ? std::atoi(env) : 1;
-    }
     long long p = floorPow2(want < 1 ? 1 : want);
     const long long p_min = plan.latent_wide ? 128 : (latent_head ? 256 : 64);
     p = p < p_min ? p_min : (p > 512 ? 512 : p);

@@ -98,9 +98,7 @@ void launchAll(const DecodeArgs &a, const Plan &plan, bool tiled, hipStream_t st
             const dim3 grid(plan.max_partitions, a.num_kv_heads * head_chunks, a.num_seqs);
             if (plan.latent_wide) {
                 // a single chunk of 16 heads gets the whole workgroup; otherwise a wavefront per chunk, four or eight
-                const bool one_chunk = head_chunks == 1;
-                const int chunks_per_group = latentChunksPerWorkgroup(head_chunks);
-                const int groups_of_chunks = (head_chunks + chunks_per_group - 1) / chunks_per_group;
+                const int groups_of_chunks = (head_chunks + plan.latent_chunks - 1) / plan.latent_chunks;
                 const int streams = a.num_kv_heads * groups_of_chunks;
                 dim3 wide(plan.max_partitions, streams, a.num_seqs);
                 if (a.chosen_partition != nullptr) {
@@ -108,11 +106,9 @@ void launchAll(const DecodeArgs &a, const Plan &plan, bool tiled, hipStream_t st
                     const long long units = static_cast<long long>(a.num_seqs) * plan.max_partitions;
                     wide = dim3(static_cast<unsigned>((units + 7) / 8 * 8 * streams));
                 }
-                if (one_chunk) {
-                    decodeMlaWideKernel<T, Tindex, 1><<<wide, kMlaWideThreads, 0, stream>>>(a);
-                } else if (std::getenv("PA_MLA_OLD") != nullptr) {
-                    decodeMlaWideKernel<T, Tindex, kMlaWideChunks><<<wide, kMlaWideThreads, 0, stream>>>(a);
-                } else if (chunks_per_group == 8) {
+                if (plan.latent_chunks == 1) {
+                    decodeMlaChunkKernel<T, Tindex><<<wide, kMlaWideThreads, 0, stream>>>(a);
+                } else if (plan.latent_chunks == 8) {
                     decodeMlaRowsKernel<T, Tindex, 8><<<wide, 512, 0, stream>>>(a);
                 } else {
                     decodeMlaRowsKernel<T, Tindex, 4><<<wide, 256, 0, stream>>>(a);

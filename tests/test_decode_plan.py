@@ -8,10 +8,11 @@ from pathlib import Path
 import pytest
 
 ROOT = Path(__file__).resolve().parents[1]
-KNOBS = ("INFINIOP_AMD_PA_KERNEL", "INFINIOP_AMD_PA_SCHEDULE", "INFINIOP_AMD_PA_LATENT_KERNEL",
+KNOBS = ("INFINIOP_AMD_PA_KERNEL", "INFINIOP_AMD_PA_SCHEDULE", "INFINIOP_AMD_PA_LATENT_KERNEL", "INFINIOP_AMD_PA_LATENT_HEADS",
          "INFINIOP_AMD_PA_PARTITION", "INFINIOP_AMD_PA_WAVES_PER_CU")
 FIELDS = ("tiled", "balanced", "latent_wide", "partition_tokens", "max_partitions", "fallback_partition_tokens",
-          "fallback_max_partitions", "waves_per_stream", "workspace_bytes", "launchable", "acc_bytes", "ml_bytes")
+          "fallback_max_partitions", "waves_per_stream", "workspace_bytes", "launchable", "acc_bytes", "ml_bytes",
+          "latent_chunks")
 
 
 def build_probe(directory):
@@ -118,3 +119,24 @@ def test_empty_batches_and_headless_tensors_plan_nothing(probe, monkeypatch, sch
     for seqs, heads, kv in ((0, 32, 8), (4, 0, 8), (0, 0, 8)):  # (no KV heads at all is refused at validation)
         pl = probe(seqs, heads, kv, 128, 16, 256)
         assert not pl["balanced"] and pl["workspace_bytes"] >= 0
+
+
+def test_head_chunks_that_share_a_latent_attention_workgroup(probe, monkeypatch):
+    """One chunk of 16 heads: eight wavefronts for it (small batches) or the pairs of wavefronts; more chunks: four per
+    workgroup, eight where there are more than four and at least 48 sequences x KV heads; the knob forces 64 or 128
+    heads per workgroup where there is more than one chunk."""
+    mla = dict(head_size=576, value_size=512, block_size=16, max_blocks=256)
+    def chunks(num_seqs, heads, kv=1):
+        plan = probe(num_seqs, heads, kv, mla["head_size"], mla["block_size"], mla["max_blocks"], value_size=mla["value_size"])
+        return plan["latent_wide"], plan["latent_chunks"]
+    assert chunks(32, 16) == (1, 1)
+    assert chunks(128, 16)[0] == 0          # many sequences of one chunk: the two-wavefront units
+    assert chunks(32, 32) == (1, 4) and chunks(32, 64) == (1, 4) and chunks(300, 64) == (1, 4)
+    assert chunks(32, 128) == (1, 4) and chunks(47, 128) == (1, 4)
+    assert chunks(48, 128) == (1, 8) and chunks(24, 256, kv=2) == (1, 8) and chunks(256, 80) == (1, 8)
+    monkeypatch.setenv("INFINIOP_AMD_PA_LATENT_HEADS", "128")
+    assert chunks(4, 128) == (1, 8) and chunks(4, 32) == (1, 8) and chunks(32, 16) == (1, 1)
+    monkeypatch.setenv("INFINIOP_AMD_PA_LATENT_HEADS", "64")
+    assert chunks(200, 128) == (1, 4)
+    monkeypatch.setenv("INFINIOP_AMD_PA_LATENT_HEADS", "96")
+    assert chunks(200, 128) == (1, 8)       # not a size the kernels have: ignored
