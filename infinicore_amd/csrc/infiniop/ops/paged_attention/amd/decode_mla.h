@@ -791,7 +791,7 @@ __global__ void __launch_bounds__(kMlaWideThreads, 2) decodeMlaChunkKernel(Decod
 //     double-buffered; the first half of the wavefronts brings equal parts of the K tile, the second half of the V
 //     tile, one load instruction after every few K operands of the tile before. One workgroup barrier per tile.
 //   * K row-major with its 16-byte chunks XOR-swizzled by the row; V row-major in blocks of 16 columns, read back
-//     through the transposing LDS read (layouts: see the prefill kernel).
+//     through the transposing LDS read, a block of 16 tokens x 16 columns at a time (512 contiguous bytes).
 //   * results leave through LDS (the tile buffers) as whole rows, 16 bytes per lane.
 template <typename T, typename Tindex, int WAVES>
 __global__ void __launch_bounds__(64 * WAVES) decodeMlaRowsKernel(DecodeArgs a) {
@@ -816,7 +816,8 @@ __global__ void __launch_bounds__(64 * WAVES) decodeMlaRowsKernel(DecodeArgs a) 
         // [buffer][half] of {main [token][64 chunks], tail [token][8 chunks]}, chunks XOR-swizzled by token % 8: a load
         // instruction fills 64 consecutive slots, i.e. the main part of one token or the tails of eight
         uint4 k[2][2 * kTileK];
-        // [buffer][half][row half (8 rows)][block of 16 columns][row of the half][two 16-byte chunks]
+        // [buffer][half][block of 16 columns][token][two 16-byte chunks]: the 64 lanes of a transposing read of one
+        // block touch 512 contiguous bytes, whichever way the hardware groups them
         uint4 v[2][2 * kTileV];
     };
     __shared__ Tiles tiles;
@@ -885,15 +886,15 @@ __global__ void __launch_bounds__(64 * WAVES) decodeMlaRowsKernel(DecodeArgs a) 
     //   K, j < rows:  the main part of row R + j: slot0 = 64 (R + j); lane asks for chunk lane ^ (row % 8)
     //   K, j >= rows: the tails of rows R + 8 (j - rows) .. + 7: slot0 = tail + 8 (that row); lane asks for chunk
     //                 64 + (lane % 8 ^ row % 8) of row (that row) + lane / 8
-    //   V:            slot0 = 512 copy_sub + 64 j: row 8 (copy_sub + j / 8) + (lane % 16) / 2, chunk 8 (j % 8) +
-    //                 2 (lane / 16) + lane % 2 (the layout at Tiles)
+    //   V:            slot0 = 64 (loads per wavefront x copy_sub + j), two blocks of 16 columns: row (lane % 32) / 2,
+    //                 chunk 4 (that j) + 2 (lane / 32) + lane % 2 (the layout at Tiles; 64 contiguous bytes of a row)
     // so two registers hold every lane-dependent offset (lane_main, XORed with a constant per instruction, and
     // lane_tail) and the rest is scalar arithmetic.
     constexpr int kRowsK = 16 / kParts; // rows of the half this wavefront copies (K)
     const uint32_t k_row_bytes = static_cast<uint32_t>(a.k_row_stride) * sizeof(S);
     const uint32_t v_row_bytes = static_cast<uint32_t>(a.v_row_stride) * sizeof(S);
     const int copy_row0 = kRowsK * copy_sub;
-    const uint32_t lane_main = copies_k ? 16u * lane : ((lane & 15) >> 1) * v_row_bytes + 16u * (2 * (lane >> 4) + (lane & 1));
+    const uint32_t lane_main = copies_k ? 16u * lane : ((lane & 31) >> 1) * v_row_bytes + 16u * (2 * (lane >> 5) + (lane & 1));
     const uint32_t lane_tail = (lane >> 3) * k_row_bytes + 16u * (kMainK + ((lane & 7) ^ (lane >> 3))); // rows R + 8 q + lane / 8: same row % 8 as lane / 8
     auto slotLaneOffset = [&](int j) -> uint32_t {
         if (!copies_k) {
@@ -903,17 +904,17 @@ __global__ void __launch_bounds__(64 * WAVES) decodeMlaRowsKernel(DecodeArgs a) 
     };
     auto slotRowOffset = [&](int j) -> uint32_t { // uniform part, bytes
         if (!copies_k) {
-            return (8 * (copy_sub + (kParts == 1 ? j / 8 : 0))) * v_row_bytes + 128u * (j % 8);
+            return 64u * (kLoadsV * copy_sub + j);
         }
         return (j < kRowsK ? copy_row0 + j : copy_row0 + 8 * (j - kRowsK)) * k_row_bytes;
     };
     auto slotLds = [&](int j) -> int { // first slot within the half
         if (!copies_k) {
-            return 512 * copy_sub + 64 * j;
+            return 64 * (kLoadsV * copy_sub + j);
         }
         return j < kRowsK ? kMainK * (copy_row0 + j) : kTailK + 8 * (copy_row0 + 8 * (j - kRowsK));
     };
-    auto vRowOfLoad = [&](int j) { return 8 * (copy_sub + (kParts == 1 ? j / 8 : 0)) + ((lane & 15) >> 1); };
+    auto vRowOfLoad = [&](int) { return (lane & 31) >> 1; };
     // The load instructions of a tile are not issued in one burst after the barrier but one at a time between the
     // matrix instructions of the tile before (see the prefill kernel): stageTile records where they read and write,
     // issueSlot(i) issues the i-th. A half that ends beyond the partition takes the lane-by-lane path at once: K rows
@@ -983,7 +984,7 @@ __global__ void __launch_bounds__(64 * WAVES) decodeMlaRowsKernel(DecodeArgs a) 
     typedef short s16x4 __attribute__((ext_vector_type(4)));
     typedef __attribute__((address_space(3))) s16x4 *LdsPiece;
     const auto v_read_base = (__attribute__((address_space(3))) char *)tiles.v
-                           + 16 * ((g >> 1) * 8 * kRowV + (4 * (g & 1) + (c >> 2)) * 2 + ((c & 3) >> 1)) + 8 * (c & 1);
+                           + 16 * ((4 * g + (c >> 2)) * 2 + ((c & 3) >> 1)) + 8 * (c & 1);
 
     f32x4 s0, s1; // raw scores of head c for tokens 4g .. 4g + 3 of the first / second half of the tile
     auto computeScores = [&](int buf) {
@@ -1034,7 +1035,7 @@ __global__ void __launch_bounds__(64 * WAVES) decodeMlaRowsKernel(DecodeArgs a) 
         constexpr int kAhead = WAVES == 4 ? kMlaQuadOperandsAhead : 2;
         constexpr int kEveryV = kBlocks / kSlots; // one load instruction after every so many operands
         auto readV = [&](int e) {
-            const auto base = v_read_base + buf * (2 * kTileV * 16) + 256 * e;
+            const auto base = v_read_base + buf * (2 * kTileV * 16) + 512 * e;
             const uint2 lo = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<LdsPiece>(base)));
             const uint2 hi = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<LdsPiece>(base + kTileV * 16)));
             return make_uint4(lo.x, lo.y, hi.x, hi.y);
