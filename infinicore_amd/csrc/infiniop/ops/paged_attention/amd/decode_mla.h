@@ -376,6 +376,9 @@ __device__ __forceinline__ WidePlan planWide(const DecodeArgs &a, int lane, int 
     // Lanes hold up to four lengths each; a batch of at most 64 sequences fills one of the four slots, and
     // the arithmetic on the empty ones (three quarters of the search below) is skipped: wave-uniform tests.
     const int slots = (a.num_seqs + 63) >> 6;
+    // what an earlier call left of its search (see below), asked for in the same round trip as the lengths
+    unsigned long long *const remembered = reinterpret_cast<unsigned long long *>(a.chosen_partition + 2);
+    const unsigned long long seen = *remembered;
     int lens[4]; // the lengths once (one round of independent loads)
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -386,9 +389,9 @@ __device__ __forceinline__ WidePlan planWide(const DecodeArgs &a, int lane, int 
         }
         lens[i] = static_cast<int>(len);
     }
+    // The search: cost(p) = (rounds of workgroups) x (tiles per partition).
     const int cap = min(64 << a.block_shift, 1024);
-    int best_cost = 0x7fffffff;
-    for (int p = a.partition_tokens; p <= cap || p == a.partition_tokens; p += 64) {
+    auto roundsAt = [&](int p) {
         // partitions of this lane's sequences: ceil(len / p) through the reciprocal, corrected to be exact
         // (lengths above 2^24 are rounded, which only blunts the estimate)
         const float pf = static_cast<float>(p), inv = 1.0f / pf;
@@ -405,14 +408,52 @@ __device__ __forceinline__ WidePlan planWide(const DecodeArgs &a, int lane, int 
             x += static_cast<int>(q) + (q * pf < lf ? 1 : 0);
         }
         const int workgroups = __builtin_amdgcn_readlane(waveInclusiveSum(x), 63) * streams;
-        const int rounds = (workgroups + a.compute_units - 1) / a.compute_units;
-        const int cost = rounds * ((p + kMlaWideTileTokens - 1) / kMlaWideTileTokens);
-        if (cost <= best_cost) {
-            best_cost = cost;
-            plan.partition_tokens = p;
+        return (workgroups + a.compute_units - 1) / a.compute_units;
+    };
+    const int first_rounds = roundsAt(a.partition_tokens);
+    // (one round at the planned size: everything runs at once, larger partitions only take longer)
+    if (first_rounds > 1 && a.partition_tokens + 64 <= cap) {
+        // The rest of the search is the same for every call on the same lengths - the layers of a model's decode
+        // step, one after the other - so its result is remembered beside the partition size left for the merge
+        // kernel: one 64-bit word, a 56-bit hash of everything the search looks at above the size in units of 64
+        // tokens (one word: a reader never sees the hash of one call with the size of another). Every workgroup of
+        // a call takes the same branch, because those that miss all arrive at the value the first one writes. A
+        // stale or colliding entry can only hold a size this search could have chosen for this shape (the hash
+        // covers the shape, the checks below the range), i.e. it costs time, never correctness.
+        unsigned h1 = 0, h2 = 0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            if (i >= slots) {
+                break;
+            }
+            unsigned x = static_cast<unsigned>(lens[i]) * 0x9E3779B1u + static_cast<unsigned>(64 * i + lane) * 0x85EBCA77u;
+            x ^= x >> 15;
+            h1 += x * 0x2C1B3C6Du;
+            h2 += (x ^ 0x27D4EB2Fu) * 0x165667B1u;
         }
-        if (rounds <= 1 && p == a.partition_tokens) {
-            break; // everything runs at once at the planned size: larger partitions only take longer
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            h1 += __shfl_xor(h1, off, 64);
+            h2 += __shfl_xor(h2, off, 64);
+        }
+        h1 += static_cast<unsigned>(a.partition_tokens) * 0x9E3779B1u + static_cast<unsigned>(streams) * 0x85EBCA77u;
+        h2 += static_cast<unsigned>(a.num_seqs) * 0xC2B2AE3Du + static_cast<unsigned>(a.compute_units) * 0x27D4EB2Fu + static_cast<unsigned>(a.block_shift);
+        const unsigned long long key = ((static_cast<unsigned long long>(h1) << 32) | h2) & ~0xffull;
+        const int seen_steps = static_cast<int>(seen & 0xff); // remembered size = planned size + 64 x this
+        if ((seen & ~0xffull) == key && a.partition_tokens + 64 * seen_steps <= cap) {
+            plan.partition_tokens = a.partition_tokens + 64 * seen_steps;
+        } else {
+            int best_cost = first_rounds * ((a.partition_tokens + kMlaWideTileTokens - 1) / kMlaWideTileTokens);
+            for (int p = a.partition_tokens + 64; p <= cap; p += 64) {
+                const int cost = roundsAt(p) * ((p + kMlaWideTileTokens - 1) / kMlaWideTileTokens);
+                if (cost <= best_cost) { // ties go to the larger size (fewer partial results)
+                    best_cost = cost;
+                    plan.partition_tokens = p;
+                }
+            }
+            if (linear_id == 0 && lane == 0) {
+                *remembered = key | static_cast<unsigned long long>((plan.partition_tokens - a.partition_tokens) / 64);
+            }
         }
     }
     // dense unit of this workgroup

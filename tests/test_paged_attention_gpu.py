@@ -384,6 +384,49 @@ def test_mla_per_call_plan_is_in_use(gpu_handle, tmp_path):
     assert 128 <= chosen <= 1024 and chosen % 64 == 0, chosen
 
 
+def test_mla_remembered_partition_search(gpu_handle, oracle, tmp_path):
+    """The search for the partition size is remembered in the workspace (a hash of the lengths and the shape with the
+    size found) and skipped by later calls on the same lengths: such calls reproduce the first one bit for bit, a
+    call on other lengths through the same workspace searches again and is right, and going back is right again."""
+    from test_decode_plan import build_probe
+
+    inp = workloads.make_decode_inputs(mla("mla_remember", torch.bfloat16, 24, 128, 16, 600, 2500, seed=466))
+    q, k, v, bt, sl = to_device(inp)
+    out = torch.zeros((24, 128, 512), dtype=torch.bfloat16, device=DEV)
+    status, op = create_paged_attention(gpu_handle, out, q, k, v, bt, sl, None, inp.scale)
+    assert status == 0
+    size = workspace_size_attention(op)
+    ws = torch.full((size,), 0xFF, dtype=torch.uint8, device=DEV)
+    plan = build_probe(tmp_path)(24, 128, 1, 576, 16, bt.shape[1], value_size=512, num_blocks=k.shape[0])
+    offset = plan["acc_bytes"] + 2 * plan["ml_bytes"]
+
+    def call():
+        out.zero_()
+        L.check_error(L.LIBINFINIOP.infiniopPagedAttention(op, ptr(ws), size, ptr(out), ptr(q), ptr(k), ptr(v), ptr(bt), ptr(sl), None, None))
+        torch.cuda.synchronize()
+        chosen = int(ws[offset:offset + 4].view(torch.int32).item())
+        word = int(ws[offset + 8:offset + 16].view(torch.int64).item()) & 0xFFFFFFFFFFFFFFFF
+        return out.clone(), chosen, word
+
+    first, chosen_a, word_a = call()
+    assert chosen_a > plan["partition_tokens"], "the case must make the kernel search beyond the planned size"
+    assert chosen_a == plan["partition_tokens"] + 64 * (word_a & 0xFF)
+    assert_close(first.cpu(), oracle.paged_attention(inp.q, inp.k_cache, inp.v_cache, inp.block_tables, inp.seq_lens, inp.scale), "mla_remember")
+    again, chosen, word = call()
+    assert (chosen, word) == (chosen_a, word_a) and torch.equal(again.view(torch.int16), first.view(torch.int16))
+    long_lens = inp.seq_lens.clone()
+    inp.seq_lens[:] = inp.seq_lens - 37  # other lengths under the same block table, still too many partitions for one round
+    sl.copy_(inp.seq_lens)
+    other, chosen_b, word_b = call()
+    assert word_b != word_a and chosen_b == plan["partition_tokens"] + 64 * (word_b & 0xFF)
+    assert_close(other.cpu(), oracle.paged_attention(inp.q, inp.k_cache, inp.v_cache, inp.block_tables, inp.seq_lens, inp.scale), "mla_remember_other")
+    inp.seq_lens[:] = long_lens
+    sl.copy_(long_lens)
+    back, chosen, word = call()
+    assert (chosen, word) == (chosen_a, word_a) and torch.equal(back.view(torch.int16), first.view(torch.int16))
+    L.check_error(L.LIBINFINIOP.infiniopDestroyPagedAttentionDescriptor(op))
+
+
 def test_mla_more_sequences_than_the_per_call_plan_handles(gpu_handle, oracle):
     """More than 256 sequences: fixed partitions on the three-dimensional grid."""
     run_case(gpu_handle, oracle, workloads.make_decode_inputs(mla("mla_b300", torch.bfloat16, 300, 32, 16, 1, 400, seed=470)))
