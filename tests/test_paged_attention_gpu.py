@@ -427,6 +427,18 @@ def test_mla_remembered_partition_search(gpu_handle, oracle, tmp_path):
     L.check_error(L.LIBINFINIOP.infiniopDestroyPagedAttentionDescriptor(op))
 
 
+def test_mla_batches_that_take_128_heads_per_workgroup_by_themselves(gpu_handle, oracle, tmp_path):
+    """From 48 sequences x KV heads on, more than 64 query heads per KV head share one workgroup of eight wavefronts
+    (no knob set): 50 ragged sequences of 128 and of 80 heads (five chunks: three wavefronts without heads)."""
+    from test_decode_plan import build_probe
+
+    for H in (128, 80):
+        inp = workloads.make_decode_inputs(mla(f"mla_b50_h{H}", torch.bfloat16, 50, H, 16, 1, 700, seed=475 + H))
+        plan = build_probe(tmp_path)(50, H, 1, 576, 16, inp.block_tables.shape[1], value_size=512, num_blocks=inp.k_cache.shape[0])
+        assert plan["latent_wide"] and plan["latent_chunks"] == 8
+        run_case(gpu_handle, oracle, inp)
+
+
 def test_mla_more_sequences_than_the_per_call_plan_handles(gpu_handle, oracle):
     """More than 256 sequences: fixed partitions on the three-dimensional grid."""
     run_case(gpu_handle, oracle, workloads.make_decode_inputs(mla("mla_b300", torch.bfloat16, 300, 32, 16, 1, 400, seed=470)))
