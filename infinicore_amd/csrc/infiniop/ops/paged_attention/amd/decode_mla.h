@@ -1,7 +1,8 @@
 // Tiled decode kernels for latent-attention caches: head_size 576 (512 latent + 64 rotary columns),
 // value_size 512, the shape of the reference's dedicated kernel
 // (src/infiniop/ops/paged_attention/nvidia/paged_attention_mla_hd576_v512.cu). gfx950, 64-lane wavefronts.
-// Three kernels: decodeMlaKernel (16 query heads per workgroup of two wavefronts, described first),
+// Three kernels: decodeMlaKernel (16 query heads per workgroup of two wavefronts, described first; with its value
+// width as a parameter it also takes heads of 576 whose values are 576 wide, MlaGeometry),
 // decodeMlaChunkKernel (the same 16 heads on a workgroup of eight wavefronts, for batches too small to fill the
 // device with pairs) and decodeMlaRowsKernel (more than 16 heads per KV head: 64 or 128 per workgroup, a wavefront per
 // 16); further down.
@@ -43,24 +44,32 @@ namespace op::paged_attention::amd {
 
 constexpr int kMlaThreads = 128; // two wavefronts per unit of work
 
+// VALUE: 512 (latent attention), or 576: plain attention with heads of 576, a shape of the reference's tests
+// (test/infiniop/paged_attention.py:106, nvidia/paged_attention_hd576.cu). A wavefront's half of the value columns is
+// then 288 wide: the two strips of 128 and a tail of 32, of which lane c owns columns 256 + 2c and 256 + 2c + 1
+// (4-byte loads and stores).
+template <int VALUE>
 struct MlaGeometry {
+    static_assert(VALUE == kMlaValueSize || VALUE == kMlaKeySize, "values as wide as the latent part or as the keys");
     static constexpr int kSteps = kMlaKeySize / 32;       // K-steps of K.Q^T
     static constexpr int kChunksPerRow = kMlaKeySize / 8; // 16-byte chunks in one K row
     static constexpr int kLoads = 8 * kChunksPerRow / 64; // K load instructions per tile and wavefront (8 rows)
     static constexpr int kLdsPitch = kChunksPerRow + 1;   // chunks between consecutive rows in LDS
-    static constexpr int kHalf = kMlaValueSize / 2;       // value columns per wavefront
+    static constexpr int kHalf = VALUE / 2;               // value columns per wavefront
     static constexpr int kStrips = kHalf / 128;           // 16-byte strips of one V row per lane
-    static constexpr int kCols = kHalf / 16;              // V / output columns per lane
+    static constexpr int kTail = kHalf - 128 * kStrips;   // columns after the strips: 0 or 32
+    static constexpr int kPairs = 4 * kStrips + kTail / 32; // pairs of V / output columns per lane
+    static constexpr int kCols = 2 * kPairs;              // V / output columns per lane
     // row (0..7 of the wavefront's eight) and chunk of the piece lane `lane` fetches in instruction j
     static __device__ __forceinline__ int kRow(int j, int lane) { return (64 * j + lane) / kChunksPerRow; }
     static __device__ __forceinline__ int kChunk(int j, int lane) { return (64 * j + lane) % kChunksPerRow; }
     static __device__ __forceinline__ int ldsIndex(int row, int chunk) { return row * kLdsPitch + chunk; }
 };
 
-template <typename T, typename Tindex>
+template <typename T, typename Tindex, int VALUE>
 __global__ void __launch_bounds__(kMlaThreads, 2) decodeMlaKernel(DecodeArgs a) {
     using S = typename T::storage;
-    using G = MlaGeometry;
+    using G = MlaGeometry<VALUE>;
     __shared__ uint4 k_lds[kTileTokens * G::kLdsPitch];   // one K tile
     __shared__ uint4 q_lds[kHeadsPerWave * G::kLdsPitch]; // the 16 query rows
 
@@ -124,7 +133,7 @@ __global__ void __launch_bounds__(kMlaThreads, 2) decodeMlaKernel(DecodeArgs a) 
     const int block_mask = a.block_size - 1;
 
     // Byte offsets of this lane's pieces inside a tile; the same for every tile.
-    uint32_t k_off[G::kLoads], v_off[4];
+    uint32_t k_off[G::kLoads], v_off[4], v_tail_off[4];
     {
         const uint32_t k_row_bytes = static_cast<uint32_t>(a.k_row_stride) * sizeof(S);
         const uint32_t v_row_bytes = static_cast<uint32_t>(a.v_row_stride) * sizeof(S);
@@ -135,6 +144,7 @@ __global__ void __launch_bounds__(kMlaThreads, 2) decodeMlaKernel(DecodeArgs a) 
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             v_off[j] = (4 * g + j) * v_row_bytes + 16 * c;
+            v_tail_off[j] = (4 * g + j) * v_row_bytes + 256 * G::kStrips + 4 * c;
         }
     }
 
@@ -155,7 +165,7 @@ __global__ void __launch_bounds__(kMlaThreads, 2) decodeMlaKernel(DecodeArgs a) 
         }
     };
     // Strip i of a V tile: v[j][4 i + w] = token row 4g + j, columns (256 wave) + 128 i + 8 c + 2 w, + 2 w + 1
-    auto loadVStrip = [&](int t, int i, uint32_t (&v)[4][4 * G::kStrips]) {
+    auto loadVStrip = [&](int t, int i, uint32_t (&v)[4][G::kPairs]) {
         const uint32_t lane_mask = t < n_tiles ? 0xffffffffu : 0u;
         const char *tile = tileAddress(t, v_head, a.v_batch_stride, a.v_row_stride);
 #pragma unroll
@@ -164,8 +174,20 @@ __global__ void __launch_bounds__(kMlaThreads, 2) decodeMlaKernel(DecodeArgs a) 
             v[j][4 * i] = x.x, v[j][4 * i + 1] = x.y, v[j][4 * i + 2] = x.z, v[j][4 * i + 3] = x.w;
         }
     };
+    // The tail: v[j][4 kStrips] = token row 4g + j, columns (kHalf wave) + 128 kStrips + 2 c, + 2 c + 1
+    auto loadVTail = [&](int t, uint32_t (&v)[4][G::kPairs]) {
+        if constexpr (G::kTail != 0) {
+            const uint32_t lane_mask = t < n_tiles ? 0xffffffffu : 0u;
+            const char *tile = tileAddress(t, v_head, a.v_batch_stride, a.v_row_stride);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                v[j][4 * G::kStrips] = loadLane4(tile, v_tail_off[j] & lane_mask);
+            }
+        }
+    };
 
-    // o[8 i + e][r] = O[head 4g + r of the chunk][column (256 wave) + 128 i + 8 c + e]
+    // o[8 i + e][r] = O[head 4g + r of the chunk][column (kHalf wave) + 128 i + 8 c + e]; the tail: o[8 kStrips + e],
+    // column (kHalf wave) + 128 kStrips + 2 c + e
     f32x4 o[G::kCols];
 #pragma unroll
     for (int e = 0; e < G::kCols; ++e) {
@@ -175,12 +197,13 @@ __global__ void __launch_bounds__(kMlaThreads, 2) decodeMlaKernel(DecodeArgs a) 
     float l = 0.0f;      // sum of rounded probabilities of head c over this lane's tokens only
 
     uint4 k[G::kLoads];
-    uint32_t v[4][4 * G::kStrips];
+    uint32_t v[4][G::kPairs];
     loadK(0, k);
 #pragma unroll
     for (int i = 0; i < G::kStrips; ++i) {
         loadVStrip(0, i, v);
     }
+    loadVTail(0, v);
     for (int t = 0; t < n_tiles; ++t) {
         // K: registers -> LDS -> matrix-operand layout (token c, columns 32*kk + 8g .. +7)
 #pragma unroll
@@ -207,6 +230,11 @@ __global__ void __launch_bounds__(kMlaThreads, 2) decodeMlaKernel(DecodeArgs a) 
                 accumulatePair<T>(o[2 * w], o[2 * w + 1], v[0][w], v[1][w], v[2][w], v[3][w], p_op, p_lo, g, valid);
             }
             loadVStrip(t + 1, i, v); // the strip's registers are free again
+        }
+        if constexpr (G::kTail != 0) {
+            constexpr int w = 4 * G::kStrips;
+            accumulatePair<T>(o[2 * w], o[2 * w + 1], v[0][w], v[1][w], v[2][w], v[3][w], p_op, p_lo, g, valid);
+            loadVTail(t + 1, v);
         }
     }
 
@@ -237,13 +265,21 @@ __global__ void __launch_bounds__(kMlaThreads, 2) decodeMlaKernel(DecodeArgs a) 
                 w.w = T::pack2(o[8 * i + 6][rr] * inv_l, o[8 * i + 7][rr] * inv_l);
                 *reinterpret_cast<uint4 *>(o_ptr + 128 * i) = w;
             }
+            if constexpr (G::kTail != 0) {
+                constexpr int e = 8 * G::kStrips;
+                *reinterpret_cast<uint32_t *>(o_ptr + 128 * G::kStrips - 6 * c) = T::pack2(o[e][rr] * inv_l, o[e + 1][rr] * inv_l);
+            }
         } else {
             const int64_t slot = (static_cast<int64_t>(seq) * a.num_heads + out_head) * a.max_partitions + part;
-            float *dst = a.part_acc + slot * kMlaValueSize + col0;
+            float *dst = a.part_acc + slot * VALUE + col0;
 #pragma unroll
             for (int i = 0; i < G::kStrips; ++i) {
                 reinterpret_cast<float4 *>(dst + 128 * i)[0] = make_float4(o[8 * i + 0][rr], o[8 * i + 1][rr], o[8 * i + 2][rr], o[8 * i + 3][rr]);
                 reinterpret_cast<float4 *>(dst + 128 * i)[1] = make_float4(o[8 * i + 4][rr], o[8 * i + 5][rr], o[8 * i + 6][rr], o[8 * i + 7][rr]);
+            }
+            if constexpr (G::kTail != 0) {
+                constexpr int e = 8 * G::kStrips;
+                *reinterpret_cast<float2 *>(dst + 128 * G::kStrips - 6 * c) = make_float2(o[e][rr], o[e + 1][rr]);
             }
             if (c == 0 && wave == 0) {
                 a.part_m[slot] = m_h;

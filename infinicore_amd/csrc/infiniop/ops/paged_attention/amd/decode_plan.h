@@ -79,7 +79,10 @@ inline Plan makePlan(const PagedAttentionInfo &in, const device::amd::DeviceInfo
     const bool pow2_page = bs >= 16 && (bs & (bs - 1)) == 0;
 
     const bool tiled_head = in.head_size == 64 || in.head_size == 128 || in.head_size == 192 || in.head_size == 256;
-    const bool latent_head = in.head_size == kMlaKeySize && in.value_size == kMlaValueSize;
+    // heads of 576: latent attention (values of 512), or values as wide as the keys (a shape of the reference's tests,
+    // test/infiniop/paged_attention.py:106), which only the kernel on 16-head units of two wavefronts takes
+    const bool latent_head = in.head_size == kMlaKeySize && (in.value_size == kMlaValueSize || in.value_size == kMlaKeySize);
+    const bool latent_tiles_in_lds = latent_head && in.value_size == kMlaValueSize;
     plan.tiled = ((tiled_head && in.value_size == in.head_size) || latent_head) && pow2_page
               && multipleOf8(in.q_stride) && multipleOf8(in.q_head_stride) && multipleOf8(in.o_stride)
               && multipleOf8(in.o_head_stride) && multipleOf8(in.k_batch_stride) && multipleOf8(in.k_head_stride)
@@ -123,11 +126,11 @@ inline Plan makePlan(const PagedAttentionInfo &in, const device::amd::DeviceInfo
     // A single chunk gets all eight wavefronts of a workgroup (decodeMlaChunkKernel) up to 64 sequences x KV
     // heads (16 heads, 1 / 4 / 16 / 32 sequences: 16.0 / 18.9 / 26.2 / 37.8 vs 28.8 / 29.8 / 31.5 / 39.1 us on the
     // 16-head units; 128 sequences: 135.8 vs 134.1).
-    plan.latent_wide = plan.tiled && latent_head
+    plan.latent_wide = plan.tiled && latent_tiles_in_lds
                     && (head_chunks > 1 || static_cast<long long>(in.num_seqs) * in.num_kv_heads <= 64);
     if (const char *env = std::getenv("INFINIOP_AMD_PA_LATENT_KERNEL")) {
         if (std::strcmp(env, "wide") == 0) {
-            plan.latent_wide = plan.tiled && latent_head;
+            plan.latent_wide = plan.tiled && latent_tiles_in_lds;
         } else if (std::strcmp(env, "narrow") == 0) {
             plan.latent_wide = false;
         }

@@ -203,6 +203,11 @@ __device__ __forceinline__ uint2 loadLane8(const char *uniform_base, uint32_t la
     const u32x2 v = __builtin_nontemporal_load(reinterpret_cast<const u32x2 *>(uniform_base + lane_offset));
     return make_uint2(v[0], v[1]);
 }
+// and the 4-byte one (two columns)
+__device__ __forceinline__ uint32_t loadLane4(const char *uniform_base, uint32_t lane_offset) {
+    asm volatile("" : "+v"(lane_offset));
+    return __builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(uniform_base + lane_offset));
+}
 
 // This lane's strip of one V row: the first piece at uniform_base + first_offset, the rest piece (heads above
 // 128) at uniform_base + rest_offset; 16-byte loads, 8-byte ones for pieces of four columns

@@ -115,7 +115,11 @@ void launchAll(const DecodeArgs &a, const Plan &plan, bool tiled, hipStream_t st
                 }
                 break;
             }
-            decodeMlaKernel<T, Tindex><<<grid, kMlaThreads, 0, stream>>>(a);
+            if (a.value_size == kMlaKeySize) {
+                decodeMlaKernel<T, Tindex, kMlaKeySize><<<grid, kMlaThreads, 0, stream>>>(a);
+            } else {
+                decodeMlaKernel<T, Tindex, kMlaValueSize><<<grid, kMlaThreads, 0, stream>>>(a);
+            }
             break;
         }
         }

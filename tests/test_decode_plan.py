@@ -121,6 +121,18 @@ def test_empty_batches_and_headless_tensors_plan_nothing(probe, monkeypatch, sch
         assert not pl["balanced"] and pl["workspace_bytes"] >= 0
 
 
+def test_heads_of_576_with_values_of_576_take_the_tiled_kernel_on_two_wavefront_units(probe, monkeypatch):
+    """The kernels that keep tiles in LDS are for values of 512 only, whatever the knob says; the partial results are
+    sized for 576 columns."""
+    for num_seqs, heads, kv in ((1, 16, 16), (32, 128, 1), (8, 40, 2)):
+        plan = probe(num_seqs, heads, kv, 576, 16, 256)
+        assert plan["tiled"] == 1 and plan["latent_wide"] == 0 and plan["balanced"] == 0
+        assert plan["acc_bytes"] >= num_seqs * plan["max_partitions"] * heads * 576 * 4
+    monkeypatch.setenv("INFINIOP_AMD_PA_LATENT_KERNEL", "wide")
+    assert probe(32, 128, 1, 576, 16, 256)["latent_wide"] == 0
+    assert probe(32, 128, 1, 576, 16, 256, value_size=512)["latent_wide"] == 1
+
+
 def test_head_chunks_that_share_a_latent_attention_workgroup(probe, monkeypatch):
     """One chunk of 16 heads: eight wavefronts for it (small batches) or the pairs of wavefronts; more chunks: four per
     workgroup, eight where there are more than four and at least 48 sequences x KV heads; the knob forces 64 or 128

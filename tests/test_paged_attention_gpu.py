@@ -340,6 +340,61 @@ def test_mla_padded_cache_rows(gpu_handle, oracle, latent_kernel):
     assert_close(got, want, "mla_strided", want_f32)
 
 
+# ---- heads of 576 with values of 576 (test/infiniop/paged_attention.py:106): the two-wavefront kernel of the latent
+# shape with 288 value columns per wavefront -----------------------------------------------------------------------
+
+def head576(name, dtype, B, H, Hkv, bs, lo, hi, seed, **kw):
+    return workloads.DecodeConfig(name, dtype, B, H, Hkv, 576, bs, lo, hi, seed=seed, **kw)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("H,Hkv", [(16, 16), (20, 1), (40, 2)])
+def test_head_576_with_values_of_576(gpu_handle, oracle, tmp_path, dtype, H, Hkv):
+    """One head per KV head (the reference's row), a group of 20 (two chunks of 16, one partly filled) and two KV heads;
+    lengths of one token, one page and enough for several partitions. The plan takes the tiled kernel."""
+    from test_decode_plan import build_probe
+    inp = workloads.make_decode_inputs(head576(f"h576_{H}_{Hkv}", dtype, 4, H, Hkv, 16, 1, 2500, seed=900 + H))
+    inp.seq_lens[0], inp.seq_lens[1] = 1, 16
+    plan = build_probe(tmp_path)(4, H, Hkv, 576, 16, inp.block_tables.shape[1], num_blocks=inp.k_cache.shape[0])
+    assert plan["tiled"] == 1 and plan["latent_wide"] == 0 and plan["max_partitions"] > 1
+    got, _ = run_case(gpu_handle, oracle, inp)
+    assert got.shape == (4, H, 576)
+
+
+@pytest.mark.parametrize("partition", [16, 48, 1024])
+def test_head_576_partition_sizes(gpu_handle, oracle, monkeypatch, partition):
+    monkeypatch.setenv("INFINIOP_AMD_PA_PARTITION", str(partition))
+    run_case(gpu_handle, oracle, workloads.make_decode_inputs(head576(f"h576_p{partition}", torch.bfloat16, 3, 16, 4, 16, 1, 1200, seed=910)))
+
+
+def test_head_576_matches_the_elementwise_kernel_in_layout(gpu_handle):
+    """Every one of the 576 output columns lands in its place (see the latent-attention test of the same name), for
+    sequences written by the decode kernel and for merged ones."""
+    inp = workloads.make_decode_inputs(head576("h576_cols", torch.float16, 4, 16, 2, 16, 40, 1500, seed=920))
+    inp.seq_lens[0] = 33
+    ramp = (torch.arange(576, dtype=torch.float32) - 288) / 16
+    inp.v_cache[:] = ramp.to(torch.float16)
+    got = run_paged_attention(gpu_handle, *to_device(inp), inp.scale).float().cpu()
+    want = ramp.to(torch.float16).float().expand_as(got)
+    assert torch.allclose(got, want, atol=2e-3 * float(ramp.abs().max()), rtol=0), (got - want).abs().max()
+
+
+def test_head_576_alibi_pages_of_64_int32_indices_and_garbage_beyond_the_sequences(gpu_handle, oracle):
+    inp = workloads.make_decode_inputs(head576("h576_mix", torch.bfloat16, 4, 32, 2, 64, 1, 1500, seed=930))
+    slopes = torch.tensor([2.0 ** (-(i % 8 + 1)) for i in range(32)], dtype=torch.float32)
+    want, want_f32 = oracle_of(oracle, inp, alibi_slopes=slopes, return_fp32=True)
+    k, v = inp.k_cache.clone(), inp.v_cache.clone()
+    for s in range(4):
+        n = int(inp.seq_lens[s])
+        if n % 64:
+            page = inp.block_tables[s, (n - 1) // 64]
+            k[page, :, n % 64:, :] = float("nan")
+            v[page, :, n % 64:, :] = float("nan")
+    got = run_paged_attention(gpu_handle, inp.q.to(DEV), k.to(DEV), v.to(DEV), inp.block_tables.to(DEV).to(torch.int32),
+                              inp.seq_lens.to(DEV).to(torch.int32), inp.scale, alibi=slopes.to(DEV))
+    assert_close(got, want, "h576_mix", want_f32)
+
+
 @pytest.mark.parametrize("workload", ["m1_mla_16_heads_b32", "m2_mla_128_heads_b32"])
 def test_mla_full_size_against_oracle(gpu_handle, oracle, workload):
     run_case(gpu_handle, oracle, workloads.make_decode_inputs(workloads.DECODE_CONFIGS[workload]))
