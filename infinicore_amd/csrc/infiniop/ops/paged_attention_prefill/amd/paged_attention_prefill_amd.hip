@@ -25,7 +25,7 @@ using op::paged_attention::amd::IndexU32;
 // Decided once, at descriptor creation, from shapes and the device alone (sequence lengths live in
 // device memory and are never read on the host).
 struct Plan {
-    bool tiled;          // matrix-core kernel (head 64 / 128 / 192 / 256 or keys 576 with values 512, power-of-two pages >= 8, 16-byte aligned strides)
+    bool tiled;          // matrix-core kernel (head 64 / 128 / 192 / 256 or keys 576 with values 512 / 576, power-of-two pages >= 8, 16-byte aligned strides)
     int groups_per_wave; // tiled: R = 1 or 2 column groups per wavefront -> 64 R rows per workgroup
     int dims_per_lane;   // element-wise kernel: ceil(max(head_size, value_size) / 64)
 };
@@ -40,7 +40,9 @@ Plan makePlan(const PagedAttentionPrefillInfo &in, const device::amd::DeviceInfo
     const long long rows = static_cast<long long>(in.total_q_tokens) * group; // per KV head
     const bool equal_sizes = in.value_size == in.head_size
                           && (in.head_size == 64 || in.head_size == 128 || in.head_size == 192 || in.head_size == 256);
-    const bool latent = in.head_size == 576 && in.value_size == 512; // keys 576, values 512
+    // keys 576 with values 512 (latent attention) or 576 (a shape of the reference's decode tests,
+    // test/infiniop/paged_attention.py:106, taken here as well so that prompt and decode run the same class of kernel)
+    const bool latent = in.head_size == 576 && (in.value_size == 512 || in.value_size == 576);
     plan.tiled = (equal_sizes || latent) && pow2_page
               && multipleOf8(in.q_stride) && multipleOf8(in.q_head_stride) && multipleOf8(in.o_stride)
               && multipleOf8(in.o_head_stride) && multipleOf8(in.k_batch_stride) && multipleOf8(in.k_head_stride)
@@ -73,7 +75,7 @@ Plan makePlan(const PagedAttentionPrefillInfo &in, const device::amd::DeviceInfo
         }
     }
     if (latent) {
-        // the accumulators of 64 rows x 512 columns are half the register file: there is no kernel with two
+        // the accumulators of 64 rows x 512 (576) columns are half the register file: there is no kernel with two
         // groups, whatever the knob says (grid and kernel must agree on the rows per workgroup)
         r = 1;
     }
@@ -102,7 +104,7 @@ void launchTiledHead(const PrefillArgs &a, const Plan &plan, hipStream_t stream)
     const int groups = plan.groups_per_wave;
     const int block_rows = prefillBlockRows(groups);
     const dim3 grid(static_cast<unsigned>((rows / block_rows + a.num_seqs) * a.num_kv_heads));
-    if constexpr (KHEAD == VHEAD) {
+    if constexpr (KHEAD == VHEAD && KHEAD <= 256) {
         if (groups == 2) {
             prefillTiledKernel<T, Tindex, KHEAD, VHEAD, 2, PLAIN><<<grid, kPrefillThreads, 0, stream>>>(a);
             return;
@@ -118,7 +120,13 @@ void launchTiledPlain(const PrefillArgs &a, const Plan &plan, hipStream_t stream
     case 128: launchTiledHead<T, Tindex, 128, 128, PLAIN>(a, plan, stream); break;
     case 192: launchTiledHead<T, Tindex, 192, 192, PLAIN>(a, plan, stream); break;
     case 256: launchTiledHead<T, Tindex, 256, 256, PLAIN>(a, plan, stream); break;
-    default: launchTiledHead<T, Tindex, 576, 512, PLAIN>(a, plan, stream); break;
+    default:
+        if (a.value_size == 576) {
+            launchTiledHead<T, Tindex, 576, 576, PLAIN>(a, plan, stream);
+        } else {
+            launchTiledHead<T, Tindex, 576, 512, PLAIN>(a, plan, stream);
+        }
+        break;
     }
 }
 

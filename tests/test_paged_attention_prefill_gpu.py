@@ -176,6 +176,44 @@ def test_mla_column_layout_and_garbage(gpu_handle, oracle):
     assert torch.allclose(got, want, atol=2e-3 * float(ramp.float().abs().max()), rtol=0), (got - want).abs().max()
 
 
+# ---- heads of 576 with values of 576 (the decode test list of the reference has the shape,
+# test/infiniop/paged_attention.py:106): the matrix-core kernel of the latent shape with 36 value blocks -------------
+
+@pytest.mark.parametrize("kernel", ["tiled", "generic"])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("H,Hkv", [(16, 16), (20, 1), (8, 2)])
+def test_head_576_with_values_of_576(gpu_handle, oracle, monkeypatch, dtype, H, Hkv, kernel):
+    if kernel == "generic":
+        monkeypatch.setenv("INFINIOP_AMD_PREFILL_KERNEL", "generic")
+    small = kernel == "generic"
+    cfg = prefill_config(f"h576_{H}_{Hkv}_{kernel}", dtype, 3, H, Hkv, 576, 16, (1, 30 if small else 150), (0, 80 if small else 400), seed=600 + H)
+    got, _ = run_case(gpu_handle, oracle, workloads.make_prefill_inputs(cfg))
+    assert got.shape[-1] == 576
+
+
+def test_head_576_column_layout_garbage_alibi_and_int32(gpu_handle, oracle):
+    """Every one of the 576 output columns lands where it belongs (V with a distinct constant per column), NaN beyond the
+    sequences does not leak in; then the same inputs with random values, ALiBi and 32-bit indices against the oracle."""
+    inp = workloads.make_prefill_inputs(prefill_config("h576_cols", torch.float16, 3, 8, 2, 576, 16, (5, 90), (3, 200), seed=640))
+    values = inp.v_cache.clone()
+    ramp = ((torch.arange(576, dtype=torch.float32) - 288) / 16).to(torch.float16)
+    inp.v_cache[:] = ramp
+    for s in range(inp.config.num_seqs):
+        L = int(inp.seq_lens[s])
+        if L % 16:
+            page = int(inp.block_tables[s, (L - 1) // 16])
+            inp.k_cache[page, :, L % 16:, :] = float("nan")
+            inp.v_cache[page, :, L % 16:, :] = float("nan")
+            values[page, :, L % 16:, :] = float("nan")
+    dev = [t.to(DEV) for t in (inp.q, inp.k_cache, inp.v_cache, inp.block_tables, inp.seq_lens, inp.cum_seq_lens_q)]
+    got = run_paged_attention_prefill(gpu_handle, *dev, inp.scale).float().cpu()
+    want = ramp.float().expand_as(got)
+    assert torch.allclose(got, want, atol=2e-3 * float(ramp.float().abs().max()), rtol=0), (got - want).abs().max()
+    inp.v_cache = values
+    slopes = torch.tensor([2.0 ** -(i % 5 + 1) for i in range(8)], dtype=torch.float32)
+    run_case(gpu_handle, oracle, inp, alibi=slopes, index_dtype=torch.int32)
+
+
 # ---- kernel variants --------------------------------------------------------------------------------------
 
 @pytest.mark.parametrize("groups", ["1", "2"])
