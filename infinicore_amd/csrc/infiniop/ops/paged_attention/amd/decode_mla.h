@@ -1242,6 +1242,385 @@ __global__ void __launch_bounds__(64 * WAVES) decodeMlaRowsKernel(DecodeArgs a) 
     }
 }
 
+// ---- 64 query heads per workgroup, K . Q^T and P . V in different wavefronts ----------------------------------------
+// The unit of work, its planning per call and the LDS layouts are those of decodeMlaRowsKernel with four chunks. That
+// kernel runs one wavefront per SIMD, and such a wavefront does the steps of a tile one after the other: the matrix
+// instructions of K . Q^T, the softmax, those of P . V, each behind the latency of its LDS operands, with two barriers;
+// the 128 accumulator and 72 query registers of a chunk leave no room for a second wavefront on the SIMD. Here a chunk
+// of 16 heads has TWO wavefronts on its SIMD with different roles:
+//   * the score wavefront (0..3) holds the query (72 registers), computes K . Q^T of tile t and its softmax step, and
+//     leaves the probabilities (512 bytes), the factor by which the reference point of each head moved and the sums
+//     in LDS;
+//   * the value wavefront (4..7) holds the accumulators (128 registers) and in the same period multiplies the
+//     probabilities of tile t - 1 by its V tile, rescaling first where a reference point moved; at the end it writes
+//     the unit's result.
+// Tiles are 16 tokens; K and V tiles each go round a ring of four LDS buffers (136 KiB as in the kernel above), one
+// workgroup barrier per tile. In period t the score wavefronts ask for V(t + 2) and the value wavefronts for K(t + 3),
+// one load instruction (global memory straight into LDS) between matrix instructions; both are first read in period
+// t + 3, so before a barrier every wavefront waits until no more than its load instructions of the last two periods
+// are outstanding (a wavefront's loads come back in the order issued). Every period issues whole tiles so that these
+// counts are exact: rows beyond the end of the partition are fetched all the same (a tile lies inside one page), their
+// scores are replaced and their V values zeroed in the operand registers; tiles beyond the last one are not needed and
+// the last one is fetched again in their place.
+template <typename T, typename Tindex>
+__global__ void __launch_bounds__(512) decodeMlaRolesKernel(DecodeArgs a) {
+    using S = typename T::storage;
+    constexpr int kChunks = 4;                    // 16-head chunks of a workgroup
+    constexpr int kRing = 4;                      // LDS buffers of either kind
+    constexpr int kSteps = kMlaKeySize / 32;      // 18 K-steps
+    constexpr int kRowK = kMlaKeySize / 8;        // 72 16-byte chunks in a K row
+    constexpr int kRowV = kMlaValueSize / 8;      // 64 in a V row
+    constexpr int kSwizzle = 8;                   // stays inside a K row: 72 is a multiple of 8
+    constexpr int kTileK = kTileTokens * kRowK;   // chunks of a tile
+    constexpr int kTileV = kTileTokens * kRowV;
+    constexpr int kBlocks = kMlaValueSize / 16;   // 32 column blocks of 16
+    constexpr int kLoadsV = kTileV / 64 / kChunks; // load instructions per period of a score wavefront: 4 of the V tile
+    constexpr int kLoadsKMost = 5;                // of a value wavefront: 4 main parts of K rows, and for two of them one of tails
+    constexpr int kOutRows = kHeadsPerWave / 2;   // output rows a wavefront stages in LDS at a time
+    constexpr int kOutPitch = kMlaValueSize + 4;  // floats between them (conflict-free column writes)
+    constexpr int kMainK = 64;                    // chunks of a K row kept in the main region of a tile; the other 8 in its tail
+    constexpr int kTailK = kTileTokens * kMainK;  // first slot of the tail region
+    struct Tiles {
+        uint4 k[kRing][kTileK]; // {main [token][64 chunks], tail [token][8 chunks]}, chunks XOR-swizzled by token % 8
+        uint4 v[kRing][kTileV]; // [block of 16 columns][token][two 16-byte chunks]
+    };
+    __shared__ Tiles tiles;
+    __shared__ uint2 p_lds[2][kChunks][64];                 // probabilities of a tile as the A operand of P . V
+    __shared__ float alpha_lds[2][kChunks][kHeadsPerWave];  // factor of head c where the reference point moved
+    __shared__ int moved_lds[2][kChunks];                   // whether any did
+    __shared__ float ml_lds[kChunks][2][kHeadsPerWave];     // at the end: reference points and sums
+    static_assert(sizeof(Tiles) >= kChunks * kOutRows * kOutPitch * sizeof(float), "the tile buffers hold the staged output rows");
+
+    const int head_chunks = (a.group + kHeadsPerWave - 1) / kHeadsPerWave;
+    const int groups_of_chunks = (head_chunks + kChunks - 1) / kChunks;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const bool scores_role = wave < kChunks;
+    const int cw = wave & (kChunks - 1); // chunk of the workgroup
+    const int lane = threadIdx.x & 63;
+    const int c = lane & 15;
+    const int g = lane >> 4;
+
+    int seq, part, stream, partition_tokens, len;
+    if (!locateWideUnit<Tindex>(a, lane, groups_of_chunks, seq, part, stream, partition_tokens, len)) {
+        return;
+    }
+    const int kv_head = stream / groups_of_chunks;
+    const int chunk = (stream - kv_head * groups_of_chunks) * kChunks + cw; // may lie beyond the last chunk: no heads
+    const int start = part * partition_tokens;
+    if (len <= 0 || start >= len) {
+        return;
+    }
+    const int end = min(len, start + partition_tokens);
+    const int n_tiles = (end - start + kTileTokens - 1) / kTileTokens;
+
+    const int first_entry = start >> a.block_shift;
+    const int last_entry = (end - 1) >> a.block_shift;
+    int page_ids = 0;
+    if (first_entry + lane <= last_entry) {
+        page_ids = clampPage(
+            loadIndex<Tindex>(a.block_tables, seq * a.block_table_batch_stride + first_entry + lane), a.num_blocks);
+    }
+    const int block_mask = a.block_size - 1;
+    // first byte of row 0 of tile t (clamped to the last tile) of K or V
+    auto tileSource = [&](int t, const char *head_base, int64_t batch_stride, int64_t row_stride) -> const char * {
+        const int tok0 = start + min(t, n_tiles - 1) * kTileTokens;
+        const int page = __builtin_amdgcn_readlane(page_ids, (tok0 >> a.block_shift) - first_entry);
+        return head_base + (page * batch_stride + (tok0 & block_mask) * row_stride) * static_cast<int64_t>(sizeof(S));
+    };
+    const int heads_here = min(kHeadsPerWave, a.group - chunk * kHeadsPerWave); // <= 0: a chunk beyond the last
+    const int n_periods = n_tiles + 1;
+
+    if (scores_role) {
+        // ================= score wavefront =================
+        // Query of head (chunk*16 + c): columns 32 kk + 8g .. +7, the B operand of K-step kk
+        const int head_in_group = chunk * kHeadsPerWave + c;
+        const bool head_valid = head_in_group < a.group;
+        const int head = kv_head * a.group + head_in_group;
+        uint4 q_reg[kSteps];
+        {
+            const S *q_ptr = static_cast<const S *>(a.q) + seq * a.q_stride + (head_valid ? head : 0) * a.q_head_stride;
+            const uint32_t keep = head_valid ? 0xffffffffu : 0u;
+#pragma unroll
+            for (int kk = 0; kk < kSteps; ++kk) {
+                uint4 x = *reinterpret_cast<const uint4 *>(q_ptr + 32 * kk + 8 * g);
+                x.x &= keep, x.y &= keep, x.z &= keep, x.w &= keep;
+                q_reg[kk] = x;
+            }
+        }
+        const float slope = (a.alibi_slopes != nullptr && head_valid) ? a.alibi_slopes[head] * kLog2e : 0.0f;
+        // copy: load instruction j (0..3) of this wavefront fills slots 64 (4 cw + j) .. + 63 of the V tile, two blocks of
+        // 16 columns: lane -> row (lane % 32) / 2, chunk 4 (4 cw + j) + 2 (lane / 32) + lane % 2
+        const char *v_head = reinterpret_cast<const char *>(static_cast<const S *>(a.v_cache) + kv_head * a.v_head_stride);
+        const uint32_t v_row_bytes = static_cast<uint32_t>(a.v_row_stride) * sizeof(S);
+        const uint32_t lane_offset = ((lane & 31) >> 1) * v_row_bytes + 16u * (2 * (lane >> 5) + (lane & 1)) + 64u * (kLoadsV * cw);
+        const char *pend_src = v_head;
+        uint4 *pend_dst = &tiles.v[0][0];
+        auto issueSlot = [&](int j) { loadLane16ToLds(pend_src + 64 * j, lane_offset, pend_dst + 64 * (kLoadsV * cw + j)); };
+        auto stageV = [&](int t) {
+            pend_src = tileSource(t, v_head, a.v_batch_stride, a.v_row_stride);
+            pend_dst = &tiles.v[t % kRing][0];
+        };
+        // this lane's chunk of row c in K-step kk: chunk 4 kk + g of the row, XOR-swizzled, i.e.
+        // 8 (kk / 2) + ((4 (kk % 2) + g) ^ (c % 8)), in the main region up to K-step 15 and in the tail after
+        const int k_read_index[2] = {c * kMainK + (g ^ (c & (kSwizzle - 1))), c * kMainK + ((4 + g) ^ (c & (kSwizzle - 1)))};
+        const int k_read_tail = kTailK + c * 8 - c * kMainK;
+
+        float m = -INFINITY; // reference point of head c's exponentials (same value in the four lanes g = 0..3)
+        float l = 0.0f;      // sum of rounded probabilities of head c over this lane's tokens only
+#pragma unroll
+        for (int t = 0; t < 2; ++t) { // V(0), V(1)
+            stageV(t);
+#pragma unroll
+            for (int j = 0; j < kLoadsV; ++j) {
+                issueSlot(j);
+            }
+        }
+        for (int t = 0; t < n_periods; ++t) {
+            asm volatile("s_waitcnt vmcnt(%0)" :: "n"(2 * kLoadsV) : "memory"); // V(t - 1) has landed
+            __syncthreads();
+            if (t == n_tiles) {
+                break;
+            }
+            stageV(t + 2);
+            // K . Q^T of tile t
+            f32x4 sp[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+            {
+                constexpr int kAhead = 4;
+                const uint4 *k_tile = &tiles.k[t % kRing][0];
+                auto readK = [&](int kk) {
+                    return k_tile[kk < 2 * (kMainK / 8) ? 8 * (kk >> 1) + k_read_index[kk & 1] : k_read_index[kk & 1] + k_read_tail];
+                };
+                uint4 kf[kAhead];
+#pragma unroll
+                for (int i = 0; i < kAhead; ++i) {
+                    kf[i] = readK(i);
+                }
+                __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 0);
+#pragma unroll
+                for (int kk = 0; kk < kSteps; ++kk) {
+                    const uint4 cur = kf[kk % kAhead];
+                    if (kk + kAhead < kSteps) {
+                        kf[kk % kAhead] = readK(kk + kAhead);
+                        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                    }
+                    sp[kk & 1] = T::mfmaK32(cur, q_reg[kk], sp[kk & 1]);
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    if (kk % 4 == 3 && kk / 4 < kLoadsV) {
+                        issueSlot(kk / 4);
+                    }
+                }
+            }
+            const f32x4 s = sp[0] + sp[1]; // raw scores of head c for tokens 4g .. 4g + 3 of the tile
+            // online softmax step (softmaxStep of decode_tiled.h with one-term probabilities, its rare branches
+            // wave-uniform, the accumulators elsewhere)
+            const int tok0 = start + t * kTileTokens;
+            const int valid = min(kTileTokens, end - tok0);
+            float sc[4];
+#pragma unroll
+            for (int rr = 0; rr < 4; ++rr) {
+                sc[rr] = s[rr] * a.scale_log2;
+            }
+            if (__builtin_amdgcn_ballot_w64(slope != 0.0f) != 0) {
+#pragma unroll
+                for (int rr = 0; rr < 4; ++rr) {
+                    sc[rr] += slope * static_cast<float>(tok0 - (len - 1) + 4 * g + rr);
+                }
+            }
+            if (valid < kTileTokens) {
+#pragma unroll
+                for (int rr = 0; rr < 4; ++rr) {
+                    sc[rr] = (4 * g + rr >= valid) ? -INFINITY : sc[rr];
+                }
+            }
+            const float mx_lane = maxOf(maxOf(sc[0], sc[1]), maxOf(sc[2], sc[3]));
+            const bool moved = __builtin_amdgcn_ballot_w64(mx_lane > m + kLazyRescaleLog2) != 0;
+            if (moved) {
+                const float m_new = maxOf(m, maxAcrossTokenGroups(mx_lane));
+                const float alpha = fastExp2(m - m_new);
+                l *= alpha;
+                m = m_new;
+                if (g == 0) {
+                    alpha_lds[t & 1][cw][c] = alpha;
+                }
+            }
+            if (lane == 0) {
+                moved_lds[t & 1][cw] = moved ? 1 : 0;
+            }
+            uint2 p_op;
+            p_op.x = T::pack2(fastExp2(sc[0] - m), fastExp2(sc[1] - m));
+            p_op.y = T::pack2(fastExp2(sc[2] - m), fastExp2(sc[3] - m));
+            l += (T::unpackLo(p_op.x) + T::unpackHi(p_op.x)) + (T::unpackLo(p_op.y) + T::unpackHi(p_op.y));
+            p_lds[t & 1][cw][lane] = p_op;
+        }
+        // (the break above leaves after the barrier of the last period: every P . V but the last has been done)
+        const float l_tot = sumAcrossTokenGroups(l);
+        if (g == 0) {
+            ml_lds[cw][0][c] = m;
+            ml_lds[cw][1][c] = l_tot;
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // this wavefront's last V tiles have landed: the buffers are free
+        __syncthreads();
+        return;
+    }
+
+    // ================= value wavefront =================
+    // copy: main parts of K rows 4 cw .. 4 cw + 3 (slot 64 row, lane asks for chunk lane ^ row % 8), and for cw < 2 the
+    // tails of rows 8 cw .. 8 cw + 7 (slot tail + 64 cw: lane -> row 8 cw + lane / 8, chunk 64 + (lane % 8 ^ lane / 8))
+    const char *k_head = reinterpret_cast<const char *>(static_cast<const S *>(a.k_cache) + kv_head * a.k_head_stride);
+    const uint32_t k_row_bytes = static_cast<uint32_t>(a.k_row_stride) * sizeof(S);
+    const uint32_t lane_main = 16u * lane;
+    const uint32_t lane_tail = (8 * cw + (lane >> 3)) * k_row_bytes + 16u * (kMainK + ((lane & 7) ^ (lane >> 3)));
+    const bool copies_tail = cw < 2;
+    const char *pend_src = k_head;
+    uint4 *pend_dst = &tiles.k[0][0];
+    auto issueSlot = [&](int j) { // j < 4: a main part; j == 4: the tails, for the wavefronts that have them
+        if (j < 4) {
+            const int row = 4 * cw + j;
+            loadLane16ToLds(pend_src + row * k_row_bytes, lane_main ^ (16u * (row & (kSwizzle - 1))), pend_dst + kMainK * row);
+        } else if (copies_tail) {
+            loadLane16ToLds(pend_src, lane_tail, pend_dst + kTailK + 64 * cw);
+        }
+    };
+    auto stageK = [&](int t) {
+        pend_src = tileSource(t, k_head, a.k_batch_stride, a.k_row_stride);
+        pend_dst = &tiles.k[t % kRing][0];
+    };
+    auto awaitPeriodBeforeLast = [&]() { // no more than the loads of the last two periods outstanding
+        if (copies_tail) {
+            asm volatile("s_waitcnt vmcnt(%0)" :: "n"(2 * kLoadsKMost) : "memory");
+        } else {
+            asm volatile("s_waitcnt vmcnt(%0)" :: "n"(2 * (kLoadsKMost - 1)) : "memory");
+        }
+    };
+    // o[e][r] = O[head 4g + r of the chunk][column 16 e + c]
+    f32x4 o[kBlocks];
+#pragma unroll
+    for (int e = 0; e < kBlocks; ++e) {
+        o[e] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    // this lane's piece of a transposing V read, relative to block 0 of buffer 0: lane (g, c) points at token
+    // 4g + c / 4, columns 16 e + 4 (c % 4) .. + 3 and receives tokens 4g .. 4g + 3 of column 16 e + c
+    typedef short s16x4 __attribute__((ext_vector_type(4)));
+    typedef __attribute__((address_space(3))) s16x4 *LdsPiece;
+    const auto v_read_base = (__attribute__((address_space(3))) char *)&tiles.v[0][0]
+                           + 16 * ((4 * g + (c >> 2)) * 2 + ((c & 3) >> 1)) + 8 * (c & 1);
+#pragma unroll
+    for (int t = 0; t < 3; ++t) { // K(0), K(1), K(2)
+        stageK(t);
+#pragma unroll
+        for (int j = 0; j < kLoadsKMost; ++j) {
+            issueSlot(j);
+        }
+    }
+    for (int t = 0; t < n_periods; ++t) {
+        awaitPeriodBeforeLast(); // K(t) has landed
+        __syncthreads();
+        if (t == 0) {
+            stageK(3);
+#pragma unroll
+            for (int j = 0; j < kLoadsKMost; ++j) {
+                issueSlot(j);
+            }
+            continue;
+        }
+        const bool more = t < n_tiles; // the last period asks for nothing
+        stageK(t + 3);
+        // P . V of tile t - 1
+        const int u = t - 1;
+        const int valid = min(kTileTokens, end - (start + u * kTileTokens));
+        const uint2 p_op = p_lds[u & 1][cw][lane];
+        if (__builtin_amdgcn_readfirstlane(moved_lds[u & 1][cw]) != 0) { // rare after the first tiles
+            const float4 al = *reinterpret_cast<const float4 *>(&alpha_lds[u & 1][cw][4 * g]);
+#pragma unroll
+            for (int e = 0; e < kBlocks; ++e) {
+                o[e][0] *= al.x, o[e][1] *= al.y, o[e][2] *= al.z, o[e][3] *= al.w;
+            }
+        }
+        // rows of the tile beyond the end of the sequence may hold anything, NaN included, and 0 * NaN is NaN
+        const uint32_t keep_lo = (4 * g + 0 < valid ? 0x0000ffffu : 0u) | (4 * g + 1 < valid ? 0xffff0000u : 0u);
+        const uint32_t keep_hi = (4 * g + 2 < valid ? 0x0000ffffu : 0u) | (4 * g + 3 < valid ? 0xffff0000u : 0u);
+        constexpr int kAhead = 4;
+        const auto v_tile = v_read_base + (u % kRing) * (kTileV * 16);
+        auto readV = [&](int e) {
+            return __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<LdsPiece>(v_tile + 512 * e)));
+        };
+        uint2 vf[kAhead];
+#pragma unroll
+        for (int i = 0; i < kAhead; ++i) {
+            vf[i] = readV(i);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 0);
+#pragma unroll
+        for (int e = 0; e < kBlocks; ++e) {
+            uint2 cur = vf[e % kAhead];
+            if (e + kAhead < kBlocks) {
+                vf[e % kAhead] = readV(e + kAhead);
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            }
+            if (valid < kTileTokens) { // wave-uniform: only the last tile of a partition can be short
+                cur.x &= keep_lo, cur.y &= keep_hi;
+            }
+            o[e] = T::mfmaK16(p_op, cur, o[e]);
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            if (more && e % 6 == 5) {
+                issueSlot(e / 6); // five places: one load instruction of K(t + 3) each
+            }
+        }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // this wavefront's last K tiles have landed: the buffers are free
+    __syncthreads();
+
+    // ---- epilogue (that of decodeMlaRowsKernel): the wavefront's 16 rows pass through LDS, eight at a time ----
+    const float m_c = ml_lds[cw][0][c], l_c = ml_lds[cw][1][c]; // of head c
+    const bool single = len <= partition_tokens;
+    float *stage = reinterpret_cast<float *>(&tiles) + cw * (kOutRows * kOutPitch);
+    const int out_head0 = kv_head * a.group + chunk * kHeadsPerWave;
+#pragma unroll
+    for (int pass = 0; pass < 2; ++pass) {
+#pragma unroll
+        for (int rr = 0; rr < 2; ++rr) {
+            float *row = stage + (2 * g + rr) * kOutPitch + c;
+#pragma unroll
+            for (int e = 0; e < kBlocks; ++e) {
+                row[16 * e] = o[e][2 * pass + rr];
+            }
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // the wavefront's own stores have landed before its lanes read each other's
+#pragma unroll
+        for (int lr = 0; lr < kOutRows; ++lr) {
+            const int r = 4 * (lr >> 1) + 2 * pass + (lr & 1); // head of the chunk in staged row lr
+            if (r >= heads_here) {
+                continue;
+            }
+            if (single) { // one row per instruction: 64 lanes x 8 columns
+                const float inv_l = 1.0f / (__shfl(l_c, r, 64) + 1e-6f);
+                const float4 x = *reinterpret_cast<const float4 *>(stage + lr * kOutPitch + 8 * lane);
+                const float4 y = *reinterpret_cast<const float4 *>(stage + lr * kOutPitch + 8 * lane + 4);
+                uint4 w;
+                w.x = T::pack2(x.x * inv_l, x.y * inv_l);
+                w.y = T::pack2(x.z * inv_l, x.w * inv_l);
+                w.z = T::pack2(y.x * inv_l, y.y * inv_l);
+                w.w = T::pack2(y.z * inv_l, y.w * inv_l);
+                S *o_ptr = static_cast<S *>(a.out) + seq * a.o_stride + (out_head0 + r) * a.o_head_stride;
+                *reinterpret_cast<uint4 *>(o_ptr + 8 * lane) = w;
+            } else { // half a row per instruction: 64 lanes x 4 columns
+                const int64_t slot = (static_cast<int64_t>(seq) * a.num_heads + out_head0 + r) * a.max_partitions + part;
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const int col = 256 * h + 4 * lane;
+                    *reinterpret_cast<float4 *>(a.part_acc + slot * kMlaValueSize + col) = *reinterpret_cast<const float4 *>(stage + lr * kOutPitch + col);
+                }
+            }
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // read back before the second pass overwrites the rows
+    }
+    if (!single && g == 0 && c < heads_here) {
+        const int64_t slot = (static_cast<int64_t>(seq) * a.num_heads + out_head0 + c) * a.max_partitions + part;
+        a.part_m[slot] = m_c;
+        a.part_l[slot] = l_c;
+    }
+}
+
 } // namespace op::paged_attention::amd
 
 #endif
