@@ -1,11 +1,11 @@
 // Tiled decode kernels for latent-attention caches: head_size 576 (512 latent + 64 rotary columns),
 // value_size 512, the shape of the reference's dedicated kernel
 // (src/infiniop/ops/paged_attention/nvidia/paged_attention_mla_hd576_v512.cu). gfx950, 64-lane wavefronts.
-// Three kernels: decodeMlaKernel (16 query heads per workgroup of two wavefronts, described first; with its value
+// Four kernels: decodeMlaKernel (16 query heads per workgroup of two wavefronts, described first; with its value
 // width as a parameter it also takes heads of 576 whose values are 576 wide, MlaGeometry),
 // decodeMlaChunkKernel (the same 16 heads on a workgroup of eight wavefronts, for batches too small to fill the
-// device with pairs) and decodeMlaRowsKernel (more than 16 heads per KV head: 64 or 128 per workgroup, a wavefront per
-// 16); further down.
+// device with pairs), decodeMlaRowsKernel (more than 16 heads per KV head: 64 or 128 per workgroup, a wavefront per
+// 16) and decodeMlaRolesKernel (64 heads per workgroup, a score and a value wavefront per SIMD); further down.
 //
 // Unit of work and arithmetic are those of the head-128 tiled kernel (decode_tiled.h): one unit = one
 // (partition, KV head x 16 query heads, sequence), tiles of 16 tokens, K . Q^T and P . V on the matrix
@@ -1246,14 +1246,15 @@ __global__ void __launch_bounds__(64 * WAVES) decodeMlaRowsKernel(DecodeArgs a) 
 // The unit of work, its planning per call and the LDS layouts are those of decodeMlaRowsKernel with four chunks. That
 // kernel runs one wavefront per SIMD, and such a wavefront does the steps of a tile one after the other: the matrix
 // instructions of K . Q^T, the softmax, those of P . V, each behind the latency of its LDS operands, with two barriers;
-// the 128 accumulator and 72 query registers of a chunk leave no room for a second wavefront on the SIMD. Here a chunk
-// of 16 heads has TWO wavefronts on its SIMD with different roles:
-//   * the score wavefront (0..3) holds the query (72 registers), computes K . Q^T of tile t and its softmax step, and
-//     leaves the probabilities (512 bytes), the factor by which the reference point of each head moved and the sums
-//     in LDS;
-//   * the value wavefront (4..7) holds the accumulators (128 registers) and in the same period multiplies the
-//     probabilities of tile t - 1 by its V tile, rescaling first where a reference point moved; at the end it writes
-//     the unit's result.
+// the 128 accumulator and 72 query registers of a chunk leave no room for a second wavefront on the SIMD. Here every
+// SIMD has TWO wavefronts with different roles:
+//   * score wavefront w (0..3) holds the query of chunk w (72 registers), computes K . Q^T of tile t and its softmax
+//     step, and leaves in LDS the probabilities (512 bytes), the factor by which the reference point of each head
+//     moved and, at the end, the sums;
+//   * value wavefront w (4..7) holds the accumulators of ALL 64 heads for value columns 128 w .. 128 w + 127 (128
+//     registers) and in the same period multiplies the probabilities of tile t - 1 of the four chunks by its quarter
+//     of the V tile: a V operand read from LDS (a transposing read, the slow kind) serves four matrix instructions;
+//     where a reference point moved it rescales first; at the end it writes its columns of the unit's result.
 // Tiles are 16 tokens; K and V tiles each go round a ring of four LDS buffers (136 KiB as in the kernel above), one
 // workgroup barrier per tile. In period t the score wavefronts ask for V(t + 2) and the value wavefronts for K(t + 3),
 // one load instruction (global memory straight into LDS) between matrix instructions; both are first read in period
@@ -1262,6 +1263,9 @@ __global__ void __launch_bounds__(64 * WAVES) decodeMlaRowsKernel(DecodeArgs a) 
 // counts are exact: rows beyond the end of the partition are fetched all the same (a tile lies inside one page), their
 // scores are replaced and their V values zeroed in the operand registers; tiles beyond the last one are not needed and
 // the last one is fetched again in their place.
+// Measured (128 heads, 32 sequences of 512 - 4 096 tokens): 60.1 us per call against 66.5 us with a wavefront per
+// chunk; a period takes 0.89 us, either role is busy for 0.8 of it. Not kept: the operands of the next tile read from
+// LDS a period ahead (62.5 us), the load instructions of a period in one burst after the barrier (61.2 - 62.3 us).
 template <typename T, typename Tindex>
 __global__ void __launch_bounds__(512) decodeMlaRolesKernel(DecodeArgs a) {
     using S = typename T::storage;
@@ -1276,8 +1280,10 @@ __global__ void __launch_bounds__(512) decodeMlaRolesKernel(DecodeArgs a) {
     constexpr int kBlocks = kMlaValueSize / 16;   // 32 column blocks of 16
     constexpr int kLoadsV = kTileV / 64 / kChunks; // load instructions per period of a score wavefront: 4 of the V tile
     constexpr int kLoadsKMost = 5;                // of a value wavefront: 4 main parts of K rows, and for two of them one of tails
-    constexpr int kOutRows = kHeadsPerWave / 2;   // output rows a wavefront stages in LDS at a time
-    constexpr int kOutPitch = kMlaValueSize + 4;  // floats between them (conflict-free column writes)
+    constexpr int kOwn = kBlocks / kChunks;       // column blocks of a value wavefront: 8
+    constexpr int kOwnCols = 16 * kOwn;           // 128 columns
+    constexpr int kOutRows = kChunks * kHeadsPerWave; // output rows a value wavefront stages in LDS: all 64 heads
+    constexpr int kOutPitch = kOwnCols + 4;       // floats between them (conflict-free column writes)
     constexpr int kMainK = 64;                    // chunks of a K row kept in the main region of a tile; the other 8 in its tail
     constexpr int kTailK = kTileTokens * kMainK;  // first slot of the tail region
     struct Tiles {
@@ -1287,7 +1293,7 @@ __global__ void __launch_bounds__(512) decodeMlaRolesKernel(DecodeArgs a) {
     __shared__ Tiles tiles;
     __shared__ uint2 p_lds[2][kChunks][64];                 // probabilities of a tile as the A operand of P . V
     __shared__ float alpha_lds[2][kChunks][kHeadsPerWave];  // factor of head c where the reference point moved
-    __shared__ int moved_lds[2][kChunks];                   // whether any did
+    __shared__ __align__(16) int moved_lds[2][kChunks];     // whether any did
     __shared__ float ml_lds[kChunks][2][kHeadsPerWave];     // at the end: reference points and sums
     static_assert(sizeof(Tiles) >= kChunks * kOutRows * kOutPitch * sizeof(float), "the tile buffers hold the staged output rows");
 
@@ -1492,11 +1498,14 @@ __global__ void __launch_bounds__(512) decodeMlaRolesKernel(DecodeArgs a) {
             asm volatile("s_waitcnt vmcnt(%0)" :: "n"(2 * (kLoadsKMost - 1)) : "memory");
         }
     };
-    // o[e][r] = O[head 4g + r of the chunk][column 16 e + c]
-    f32x4 o[kBlocks];
+    // o[h][e][r] = O[head 4g + r of the workgroup's chunk h][column 16 (kOwn cw + e) + c]
+    f32x4 o[kChunks][kOwn];
 #pragma unroll
-    for (int e = 0; e < kBlocks; ++e) {
-        o[e] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int h = 0; h < kChunks; ++h) {
+#pragma unroll
+        for (int e = 0; e < kOwn; ++e) {
+            o[h][e] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
     }
     // this lane's piece of a transposing V read, relative to block 0 of buffer 0: lane (g, c) points at token
     // 4g + c / 4, columns 16 e + 4 (c % 4) .. + 3 and receives tokens 4g .. 4g + 3 of column 16 e + c
@@ -1528,19 +1537,30 @@ __global__ void __launch_bounds__(512) decodeMlaRolesKernel(DecodeArgs a) {
         // P . V of tile t - 1
         const int u = t - 1;
         const int valid = min(kTileTokens, end - (start + u * kTileTokens));
-        const uint2 p_op = p_lds[u & 1][cw][lane];
-        if (__builtin_amdgcn_readfirstlane(moved_lds[u & 1][cw]) != 0) { // rare after the first tiles
-            const float4 al = *reinterpret_cast<const float4 *>(&alpha_lds[u & 1][cw][4 * g]);
+        uint2 p[kChunks];
 #pragma unroll
-            for (int e = 0; e < kBlocks; ++e) {
-                o[e][0] *= al.x, o[e][1] *= al.y, o[e][2] *= al.z, o[e][3] *= al.w;
+        for (int h = 0; h < kChunks; ++h) {
+            p[h] = p_lds[u & 1][h][lane];
+        }
+        const int4 moved = *reinterpret_cast<const int4 *>(&moved_lds[u & 1][0]);
+        if (__builtin_amdgcn_readfirstlane(moved.x | moved.y | moved.z | moved.w) != 0) { // rare after the first tiles
+            const int of_chunk[kChunks] = {moved.x, moved.y, moved.z, moved.w};
+#pragma unroll
+            for (int h = 0; h < kChunks; ++h) {
+                if (__builtin_amdgcn_readfirstlane(of_chunk[h]) != 0) {
+                    const float4 al = *reinterpret_cast<const float4 *>(&alpha_lds[u & 1][h][4 * g]);
+#pragma unroll
+                    for (int e = 0; e < kOwn; ++e) {
+                        o[h][e][0] *= al.x, o[h][e][1] *= al.y, o[h][e][2] *= al.z, o[h][e][3] *= al.w;
+                    }
+                }
             }
         }
         // rows of the tile beyond the end of the sequence may hold anything, NaN included, and 0 * NaN is NaN
         const uint32_t keep_lo = (4 * g + 0 < valid ? 0x0000ffffu : 0u) | (4 * g + 1 < valid ? 0xffff0000u : 0u);
         const uint32_t keep_hi = (4 * g + 2 < valid ? 0x0000ffffu : 0u) | (4 * g + 3 < valid ? 0xffff0000u : 0u);
         constexpr int kAhead = 4;
-        const auto v_tile = v_read_base + (u % kRing) * (kTileV * 16);
+        const auto v_tile = v_read_base + (u % kRing) * (kTileV * 16) + 512 * (kOwn * cw);
         auto readV = [&](int e) {
             return __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<LdsPiece>(v_tile + 512 * e)));
         };
@@ -1549,70 +1569,73 @@ __global__ void __launch_bounds__(512) decodeMlaRolesKernel(DecodeArgs a) {
         for (int i = 0; i < kAhead; ++i) {
             vf[i] = readV(i);
         }
-        __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, kChunks + 1 + kAhead, 0);
 #pragma unroll
-        for (int e = 0; e < kBlocks; ++e) {
+        for (int e = 0; e < kOwn; ++e) {
             uint2 cur = vf[e % kAhead];
-            if (e + kAhead < kBlocks) {
+            if (e + kAhead < kOwn) {
                 vf[e % kAhead] = readV(e + kAhead);
                 __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
             }
             if (valid < kTileTokens) { // wave-uniform: only the last tile of a partition can be short
                 cur.x &= keep_lo, cur.y &= keep_hi;
             }
-            o[e] = T::mfmaK16(p_op, cur, o[e]);
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            if (more && e % 6 == 5) {
-                issueSlot(e / 6); // five places: one load instruction of K(t + 3) each
+#pragma unroll
+            for (int h = 0; h < kChunks; ++h) { // the operand serves the heads of every chunk
+                o[h][e] = T::mfmaK16(p[h], cur, o[h][e]);
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                constexpr int kEvery = 6;
+                const int done = kChunks * e + h;
+                if (more && done % kEvery == kEvery - 1) {
+                    issueSlot(done / kEvery); // five places: one load instruction of K(t + 3) each
+                }
             }
         }
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // this wavefront's last K tiles have landed: the buffers are free
     __syncthreads();
 
-    // ---- epilogue (that of decodeMlaRowsKernel): the wavefront's 16 rows pass through LDS, eight at a time ----
-    const float m_c = ml_lds[cw][0][c], l_c = ml_lds[cw][1][c]; // of head c
+    // ---- epilogue: a lane holds single columns (16 e + c of the wavefront's 128) of heads 4g .. 4g + 3 of every chunk;
+    // the 64 rows pass through LDS and leave as 16-byte pieces, a row on 32 consecutive lanes ----
+    const float m_c = ml_lds[cw][0][c], l_c = ml_lds[cw][1][c]; // of head c of this wavefront's own chunk
     const bool single = len <= partition_tokens;
     float *stage = reinterpret_cast<float *>(&tiles) + cw * (kOutRows * kOutPitch);
+    const int chunk0 = chunk - cw; // the workgroup's first chunk
     const int out_head0 = kv_head * a.group + chunk * kHeadsPerWave;
 #pragma unroll
-    for (int pass = 0; pass < 2; ++pass) {
+    for (int h = 0; h < kChunks; ++h) {
 #pragma unroll
-        for (int rr = 0; rr < 2; ++rr) {
-            float *row = stage + (2 * g + rr) * kOutPitch + c;
+        for (int rr = 0; rr < 4; ++rr) {
+            float *row = stage + (kHeadsPerWave * h + 4 * g + rr) * kOutPitch + c;
 #pragma unroll
-            for (int e = 0; e < kBlocks; ++e) {
-                row[16 * e] = o[e][2 * pass + rr];
+            for (int e = 0; e < kOwn; ++e) {
+                row[16 * e] = o[h][e][rr];
             }
         }
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // the wavefront's own stores have landed before its lanes read each other's
-#pragma unroll
-        for (int lr = 0; lr < kOutRows; ++lr) {
-            const int r = 4 * (lr >> 1) + 2 * pass + (lr & 1); // head of the chunk in staged row lr
-            if (r >= heads_here) {
-                continue;
-            }
-            if (single) { // one row per instruction: 64 lanes x 8 columns
-                const float inv_l = 1.0f / (__shfl(l_c, r, 64) + 1e-6f);
-                const float4 x = *reinterpret_cast<const float4 *>(stage + lr * kOutPitch + 8 * lane);
-                const float4 y = *reinterpret_cast<const float4 *>(stage + lr * kOutPitch + 8 * lane + 4);
-                uint4 w;
-                w.x = T::pack2(x.x * inv_l, x.y * inv_l);
-                w.y = T::pack2(x.z * inv_l, x.w * inv_l);
-                w.z = T::pack2(y.x * inv_l, y.y * inv_l);
-                w.w = T::pack2(y.z * inv_l, y.w * inv_l);
-                S *o_ptr = static_cast<S *>(a.out) + seq * a.o_stride + (out_head0 + r) * a.o_head_stride;
-                *reinterpret_cast<uint4 *>(o_ptr + 8 * lane) = w;
-            } else { // half a row per instruction: 64 lanes x 4 columns
-                const int64_t slot = (static_cast<int64_t>(seq) * a.num_heads + out_head0 + r) * a.max_partitions + part;
-#pragma unroll
-                for (int h = 0; h < 2; ++h) {
-                    const int col = 256 * h + 4 * lane;
-                    *reinterpret_cast<float4 *>(a.part_acc + slot * kMlaValueSize + col) = *reinterpret_cast<const float4 *>(stage + lr * kOutPitch + col);
-                }
-            }
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // the wavefront's own stores have landed before its lanes read each other's
+    constexpr int kLanesPerRow = kOwnCols / 4; // 32 lanes on one staged row
+    const int col = kOwnCols * cw + 4 * (lane % kLanesPerRow);
+#pragma unroll 4
+    for (int i = 0; i < kOutRows * kLanesPerRow / 64; ++i) {
+        const int r = (64 / kLanesPerRow) * i + lane / kLanesPerRow;  // staged row: head r % 16 of chunk r / 16
+        const int head_in_group = chunk0 * kHeadsPerWave + r;         // chunks are consecutive, so are their heads
+        if (head_in_group >= a.group) {
+            continue;
         }
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // read back before the second pass overwrites the rows
+        const float4 x = *reinterpret_cast<const float4 *>(stage + r * kOutPitch + 4 * (lane % kLanesPerRow));
+        const int out_head = kv_head * a.group + head_in_group;
+        if (single) {
+            const float inv_l = 1.0f / (ml_lds[r >> 4][1][r & 15] + 1e-6f);
+            uint2 w;
+            w.x = T::pack2(x.x * inv_l, x.y * inv_l);
+            w.y = T::pack2(x.z * inv_l, x.w * inv_l);
+            S *o_ptr = static_cast<S *>(a.out) + seq * a.o_stride + out_head * a.o_head_stride;
+            *reinterpret_cast<uint2 *>(o_ptr + col) = w;
+        } else {
+            const int64_t slot = (static_cast<int64_t>(seq) * a.num_heads + out_head) * a.max_partitions + part;
+            *reinterpret_cast<float4 *>(a.part_acc + slot * kMlaValueSize + col) = x;
+        }
     }
     if (!single && g == 0 && c < heads_here) {
         const int64_t slot = (static_cast<int64_t>(seq) * a.num_heads + out_head0 + c) * a.max_partitions + part;

@@ -32,6 +32,7 @@ struct Plan {
     bool fused_merge;      // balanced: segments merged inside the decode kernel (no second launch)
     bool latent_wide;      // latent attention on 32-token tiles shared through LDS, units planned per call (decode_mla.h)
     int latent_chunks;     // that kernel: 16-head chunks that share a workgroup: 1 (eight wavefronts for the one chunk), 4 or 8 (a wavefront each)
+    bool latent_roles;     // four chunks: a wavefront for the scores and a wavefront for the values of each (decodeMlaRolesKernel)
     bool partition_forced; // INFINIOP_AMD_PA_PARTITION set: the 64-head kernel keeps exactly that size
     int partition_tokens;  // grid schedule: tokens per unit of work
     int max_partitions;    // grid schedule: partitions the longest representable sequence needs
@@ -69,7 +70,7 @@ inline bool launchable(const PagedAttentionInfo &in) {
 }
 
 // Environment knobs (all optional, read at descriptor creation only): INFINIOP_AMD_PA_KERNEL=generic,
-// INFINIOP_AMD_PA_SCHEDULE=grid|balanced, INFINIOP_AMD_PA_LATENT_KERNEL=wide|narrow, INFINIOP_AMD_PA_LATENT_HEADS=64|128,
+// INFINIOP_AMD_PA_SCHEDULE=grid|balanced, INFINIOP_AMD_PA_LATENT_KERNEL=wide|rows|narrow, INFINIOP_AMD_PA_LATENT_HEADS=64|128,
 // INFINIOP_AMD_PA_PARTITION=<tokens>, INFINIOP_AMD_PA_WAVES_PER_CU=<n>, INFINIOP_AMD_PA_MERGE=kernel|fused,
 // INFINIOP_AMD_PA_ODD_RELIEF=<256ths>.
 inline Plan makePlan(const PagedAttentionInfo &in, const device::amd::DeviceInfo &dev) {
@@ -128,8 +129,10 @@ inline Plan makePlan(const PagedAttentionInfo &in, const device::amd::DeviceInfo
     // 16-head units; 128 sequences: 135.8 vs 134.1).
     plan.latent_wide = plan.tiled && latent_tiles_in_lds
                     && (head_chunks > 1 || static_cast<long long>(in.num_seqs) * in.num_kv_heads <= 64);
+    bool latent_rows_forced = false;
     if (const char *env = std::getenv("INFINIOP_AMD_PA_LATENT_KERNEL")) {
-        if (std::strcmp(env, "wide") == 0) {
+        latent_rows_forced = std::strcmp(env, "rows") == 0;
+        if (std::strcmp(env, "wide") == 0 || latent_rows_forced) {
             plan.latent_wide = plan.tiled && latent_tiles_in_lds;
         } else if (std::strcmp(env, "narrow") == 0) {
             plan.latent_wide = false;
@@ -141,6 +144,10 @@ inline Plan makePlan(const PagedAttentionInfo &in, const device::amd::DeviceInfo
             plan.latent_chunks = std::atoi(env) / kHeadsPerWave;
         }
     }
+    // Four chunks per workgroup: K . Q^T with the softmax, and P . V, in different wavefronts of a SIMD, unless the knob
+    // asks for one wavefront per chunk (128 heads, 32 sequences: 60.1 vs 66.5 us; 32 / 48 / 64 heads: 46.8 / 51.9 / 53.5
+    // vs 48.0 / 51.0 / 55.4; 64 heads, 8 / 64 / 128 sequences: 25.5 / 86.2 / 169 vs 26.2 / 88.2 / 175).
+    plan.latent_roles = plan.latent_wide && plan.latent_chunks == 4 && !latent_rows_forced;
     const long long chunks_per_group = plan.latent_chunks;
     const long long wide_units = static_cast<long long>(in.num_seqs) * in.num_kv_heads
                                * ((head_chunks + chunks_per_group - 1) / chunks_per_group);

@@ -110,7 +110,7 @@ void launchAll(const DecodeArgs &a, const Plan &plan, bool tiled, hipStream_t st
                     decodeMlaChunkKernel<T, Tindex><<<wide, kMlaWideThreads, 0, stream>>>(a);
                 } else if (plan.latent_chunks == 8) {
                     decodeMlaRowsKernel<T, Tindex, 8><<<wide, 512, 0, stream>>>(a);
-                } else if (std::getenv("INFINIOP_AMD_PA_LATENT_STREAMS") == nullptr) {
+                } else if (plan.latent_roles) {
                     decodeMlaRolesKernel<T, Tindex><<<wide, 512, 0, stream>>>(a);
                 } else {
                     decodeMlaRowsKernel<T, Tindex, 4><<<wide, 256, 0, stream>>>(a);

@@ -4,7 +4,7 @@
 
 // in:  {num_seqs, num_heads, num_kv_heads, head_size, value_size, block_size, max_blocks_per_seq, num_blocks, compute_units}
 // out: {tiled, balanced, latent_wide, partition_tokens, max_partitions, fallback_partition_tokens,
-//       fallback_max_partitions, waves_per_stream, workspace_bytes, launchable, acc_bytes, ml_bytes, latent_chunks}
+//       fallback_max_partitions, waves_per_stream, workspace_bytes, launchable, acc_bytes, ml_bytes, latent_chunks, latent_roles}
 extern "C" void planProbe(const long long *in, long long *out) {
     using namespace op::paged_attention;
     PagedAttentionInfo info{};
@@ -46,4 +46,5 @@ extern "C" void planProbe(const long long *in, long long *out) {
     out[10] = static_cast<long long>(plan.acc_bytes);
     out[11] = static_cast<long long>(plan.ml_bytes);
     out[12] = plan.latent_chunks;
+    out[13] = plan.latent_roles ? 1 : 0;
 }

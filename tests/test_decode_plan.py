@@ -12,7 +12,7 @@ KNOBS = ("INFINIOP_AMD_PA_KERNEL", "INFINIOP_AMD_PA_SCHEDULE", "INFINIOP_AMD_PA_
          "INFINIOP_AMD_PA_PARTITION", "INFINIOP_AMD_PA_WAVES_PER_CU")
 FIELDS = ("tiled", "balanced", "latent_wide", "partition_tokens", "max_partitions", "fallback_partition_tokens",
           "fallback_max_partitions", "waves_per_stream", "workspace_bytes", "launchable", "acc_bytes", "ml_bytes",
-          "latent_chunks")
+          "latent_chunks", "latent_roles")
 
 
 def build_probe(directory):
@@ -119,6 +119,20 @@ def test_empty_batches_and_headless_tensors_plan_nothing(probe, monkeypatch, sch
     for seqs, heads, kv in ((0, 32, 8), (4, 0, 8), (0, 0, 8)):  # (no KV heads at all is refused at validation)
         pl = probe(seqs, heads, kv, 128, 16, 256)
         assert not pl["balanced"] and pl["workspace_bytes"] >= 0
+
+
+def test_four_chunks_per_workgroup_split_scores_and_values_between_wavefronts(probe, monkeypatch):
+    """Latent attention with four 16-head chunks per workgroup runs the kernel whose wavefronts have roles, unless the
+    knob asks for a wavefront per chunk; one chunk or eight chunks per workgroup never do."""
+    def roles(num_seqs, heads):
+        plan = probe(num_seqs, heads, 1, 576, 16, 256, value_size=512)
+        return plan["latent_chunks"], plan["latent_roles"]
+    assert roles(32, 128) == (4, 1) and roles(32, 48) == (4, 1) and roles(8, 32) == (4, 1)
+    assert roles(32, 16) == (1, 0) and roles(64, 128) == (8, 0)
+    monkeypatch.setenv("INFINIOP_AMD_PA_LATENT_KERNEL", "rows")
+    plan = probe(32, 128, 1, 576, 16, 256, value_size=512)
+    assert (plan["latent_wide"], plan["latent_chunks"], plan["latent_roles"]) == (1, 4, 0)
+    assert probe(200, 16, 1, 576, 16, 256, value_size=512)["latent_wide"] == 1  # "rows" implies the kernels on LDS tiles
 
 
 def test_heads_of_576_with_values_of_576_take_the_tiled_kernel_on_two_wavefront_units(probe, monkeypatch):

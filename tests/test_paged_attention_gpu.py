@@ -254,15 +254,15 @@ def mla(name, dtype, B, H, bs, lo, hi, seed, **kw):
     return workloads.DecodeConfig(name, dtype, B, H, 1, 576, bs, lo, hi, seed=seed, value_size=512, **kw)
 
 
-@pytest.fixture(params=[None, "narrow", "wide", "wide128"], ids=["auto", "narrow", "wide", "wide128"])
+@pytest.fixture(params=[None, "narrow", "wide", "rows", "wide128"], ids=["auto", "narrow", "wide", "rows", "wide128"])
 def latent_kernel(request, monkeypatch):
-    """The latent-attention kernels: 16 query heads per workgroup of two wavefronts ("narrow"); 32-token tiles shared
-    through LDS ("wide": a workgroup of eight wavefronts for a single chunk of 16 heads, otherwise a wavefront per chunk,
-    four per workgroup, or eight with "wide128"). Left alone, more than 16 heads per KV head and small batches take
-    the wide ones."""
+    """The latent-attention kernels: 16 query heads per workgroup of two wavefronts ("narrow"); tiles shared through LDS
+    ("wide": a workgroup of eight wavefronts for a single chunk of 16 heads, otherwise four chunks per workgroup with
+    a score and a value wavefront each; "rows": a wavefront per chunk, four per workgroup, or eight with "wide128").
+    Left alone, more than 16 heads per KV head and small batches take the wide ones."""
     if request.param:
         monkeypatch.setenv("INFINIOP_AMD_PA_LATENT_KERNEL", "wide" if request.param == "wide128" else request.param)
-        if request.param.startswith("wide"):
+        if request.param != "narrow":
             monkeypatch.setenv("INFINIOP_AMD_PA_LATENT_HEADS", "128" if request.param == "wide128" else "64")
     return request.param
 
@@ -285,7 +285,7 @@ def test_mla_partition_sizes(gpu_handle, oracle, monkeypatch, partition, latent_
     """Partitions of one 16-token half tile, of one and a half 32-token tiles, and of the most one page-id
     load covers."""
     monkeypatch.setenv("INFINIOP_AMD_PA_PARTITION", str(partition))
-    H = 48 if latent_kernel in ("wide", "wide128") else 16
+    H = 48 if latent_kernel in ("wide", "rows", "wide128") else 16
     run_case(gpu_handle, oracle, workloads.make_decode_inputs(mla(f"mla_p{partition}", torch.bfloat16, 3, H, 16, 1, 1200, seed=410)))
 
 
