@@ -46,7 +46,7 @@ MEASURED_TRAFFIC = {
     # workload: (bytes, summary under profiles/, commit of the measured kernel)
     "c2_llama3_8b_b32": (322_400_000, "decode_balanced_c2_llama3_8b_b32_hbm_traffic.md", "afe7af1"),
     "m1_mla_16_heads_b32": (153_400_000, "decode_mla_m1_m2_kernel_stats_and_traffic.md", "4349d98"),
-    "m2_mla_128_heads_b32": (205_500_000, "decode_mla_m1_m2_kernel_stats_and_traffic.md", "4349d98"),
+    "m2_mla_128_heads_b32": (205_500_000, "decode_mla_m1_m2_kernel_stats_and_traffic.md", "3b94ee4"),
     "c5_prefill_scatter": (32_100_000, "paged_caching_c5_prefill_scatter_kernel_stats_and_traffic.md", "a636ea0"),
     "k2_append_prefill_chunk": (33_600_000, "kv_caching_k2_append_prefill_chunk_kernel_stats_and_traffic.md", "f6351eb"),
     "r2_rope_scatter_prefill_chunk": (34_170_000, "rope_paged_caching_r1_r2_kernel_stats_and_traffic.md", "afe7af1"),
