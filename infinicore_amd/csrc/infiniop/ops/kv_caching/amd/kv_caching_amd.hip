@@ -11,6 +11,7 @@
 // there and are dropped here.
 #include "kv_caching_amd.h"
 #include "../../../handle.h"
+#include "../../../devices/amd/amd_streaming.h"
 #include "../../../../utils/check.h"
 #include <cstdint>
 #include <hip/hip_runtime.h>
@@ -66,11 +67,12 @@ __global__ void __launch_bounds__(256) kvCachingAppendKernel(AppendArgs a) {
     Unit *vd = static_cast<Unit *>(a.v_cache) + b * a.v_cache_strides[0] + h * a.v_cache_strides[1] + pos * a.v_cache_strides[2];
     for (int c = threadIdx.x; c < a.units_per_row; c += blockDim.x) {
         if constexpr (PACKED_ROWS) {
-            kd[c] = ks[c];
-            vd[c] = vs[c];
+            // streamed stores (the cache rows are not read again by this kernel; see amd_streaming.h)
+            device::amd::storeStreamed(kd + c, ks[c]);
+            device::amd::storeStreamed(vd + c, vs[c]);
         } else {
-            kd[c * a.k_cache_strides[3]] = ks[c * a.k_strides[3]];
-            vd[c * a.v_cache_strides[3]] = vs[c * a.v_strides[3]];
+            device::amd::storeStreamed(kd + c * a.k_cache_strides[3], ks[c * a.k_strides[3]]);
+            device::amd::storeStreamed(vd + c * a.v_cache_strides[3], vs[c * a.v_strides[3]]);
         }
     }
 }

@@ -10,6 +10,7 @@
 // (negative slot = padding, page = slot / block_size, row = slot % block_size, source heads packed).
 #include "paged_caching_amd.h"
 #include "../../../handle.h"
+#include "../../../devices/amd/amd_streaming.h"
 #include "../../../../utils/check.h"
 #include <cstdint>
 #include <hip/hip_runtime.h>
@@ -88,11 +89,12 @@ pagedCachingScatterKernel(const int64_t *early_slot_mapping, int64_t early_num_t
 
     Unit *k_dst = static_cast<Unit *>(a.k_cache) + page * a.k_block_stride + row * a.k_slot_stride;
     Unit *v_dst = static_cast<Unit *>(a.v_cache) + page * a.v_block_stride + row * a.v_slot_stride;
+    // streamed stores (the cache rows are not read again by this kernel; see amd_streaming.h)
     if (k_first) {
-        k_dst[head0 * a.k_head_stride + c0] = k0;
+        device::amd::storeStreamed(k_dst + head0 * a.k_head_stride + c0, k0);
     }
     if (v_first) {
-        v_dst[head0 * a.v_head_stride + c0] = v0;
+        device::amd::storeStreamed(v_dst + head0 * a.v_head_stride + c0, v0);
     }
     // whatever the box does not cover in one step
     for (int head = head0; head < a.num_kv_heads; head += blockDim.y) {
@@ -102,10 +104,10 @@ pagedCachingScatterKernel(const int64_t *early_slot_mapping, int64_t early_num_t
         Unit *kd = k_dst + head * a.k_head_stride;
         Unit *vd = v_dst + head * a.v_head_stride;
         for (int c = c_begin; c < a.k_units_per_row; c += blockDim.x) {
-            kd[c] = ks[c];
+            device::amd::storeStreamed(kd + c, ks[c]);
         }
         for (int c = c_begin; c < a.v_units_per_row; c += blockDim.x) {
-            vd[c] = vs[c];
+            device::amd::storeStreamed(vd + c, vs[c]);
         }
     }
 }

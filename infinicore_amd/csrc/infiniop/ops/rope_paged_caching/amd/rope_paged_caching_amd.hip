@@ -13,6 +13,7 @@
 // memory round trips long; fusing saves the second launch and the round trip of the rotated K through memory.
 #include "rope_paged_caching_amd.h"
 #include "../../../handle.h"
+#include "../../../devices/amd/amd_streaming.h"
 #include "../../../../utils/check.h"
 #include <cstdint>
 #include <hip/hip_runtime.h>
@@ -131,8 +132,8 @@ __device__ __forceinline__ void rotateRow(const S *src, S *dst, const S *sin_row
                                y_hi.e[2 * i + 1]);
                 }
             }
-            *reinterpret_cast<U *>(dst + first) = y_lo;
-            *reinterpret_cast<U *>(dst + second) = y_hi;
+            device::amd::storeStreamed(dst + first, y_lo);
+            device::amd::storeStreamed(dst + second, y_hi);
         }
     } else {
         for (int j = step0; j < table_dim; j += step) {
@@ -207,7 +208,7 @@ __device__ __forceinline__ void ropeScatter(const Args &a, const QueryArgs<QUERY
         rotateRow<S, VEC>(k_src, k_dst, sin_row, cos_row, table_dim, a.neox != 0, x0, x_step);
         if constexpr (VEC) {
             for (int u = x0; u < a.value_size / kPer; u += x_step) {
-                *reinterpret_cast<U *>(v_dst + u * kPer) = *reinterpret_cast<const U *>(v_src + u * kPer);
+                device::amd::storeStreamed(v_dst + u * kPer, *reinterpret_cast<const U *>(v_src + u * kPer));
             }
         } else {
             for (int j = x0; j < a.value_size; j += x_step) {
@@ -359,8 +360,10 @@ __global__ void __launch_bounds__(kFlatThreads) ropeScatterFlatKernel(Args a, Qu
             }
         }
         if (stores) {
-            *reinterpret_cast<uint4 *>(dst + first[j]) = out_lo;
-            *reinterpret_cast<uint4 *>(dst + second[j]) = out_hi;
+            // streamed stores: 4 096 tokens with 32 query heads 24.5 -> 18.0 us, without a query 8.7 -> 7.95 us
+            // (streamed loads on top cost 3.3 / 1.0 us: the sources are what the projection has just written)
+            device::amd::storeStreamed(dst + first[j], out_lo);
+            device::amd::storeStreamed(dst + second[j], out_hi);
         }
     }
 }
