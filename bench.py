@@ -47,10 +47,10 @@ MEASURED_TRAFFIC = {
     "c2_llama3_8b_b32": (322_400_000, "decode_balanced_c2_llama3_8b_b32_hbm_traffic.md", "afe7af1"),
     "m1_mla_16_heads_b32": (153_400_000, "decode_mla_m1_m2_kernel_stats_and_traffic.md", "4349d98"),
     "m2_mla_128_heads_b32": (205_500_000, "decode_mla_m1_m2_kernel_stats_and_traffic.md", "3b94ee4"),
-    "c5_prefill_scatter": (32_100_000, "paged_caching_c5_prefill_scatter_kernel_stats_and_traffic.md", "a636ea0"),
-    "k2_append_prefill_chunk": (33_600_000, "kv_caching_k2_append_prefill_chunk_kernel_stats_and_traffic.md", "f6351eb"),
-    "r2_rope_scatter_prefill_chunk": (34_170_000, "rope_paged_caching_r1_r2_kernel_stats_and_traffic.md", "afe7af1"),
-    "r4_rope_qk_scatter_prefill_chunk": (101_510_000, "rope_paged_caching_r1_r2_kernel_stats_and_traffic.md", "afe7af1"),
+    "c5_prefill_scatter": (33_000_000, "paged_caching_c5_prefill_scatter_kernel_stats_and_traffic.md", "3fbf320"),
+    "k2_append_prefill_chunk": (33_600_000, "kv_caching_k2_append_prefill_chunk_kernel_stats_and_traffic.md", "3fbf320"),
+    "r2_rope_scatter_prefill_chunk": (35_300_000, "rope_paged_caching_r1_r2_kernel_stats_and_traffic.md", "3fbf320"),
+    "r4_rope_qk_scatter_prefill_chunk": (103_250_000, "rope_paged_caching_r1_r2_kernel_stats_and_traffic.md", "3fbf320"),
     "p3_llama3_8b_chunked": (552_500_000, "prefill_tiled_p3_llama3_8b_chunked_counters.md", "60c46ff"),  # fetched 508.1 MB + written 44.35 MB
 }
 
