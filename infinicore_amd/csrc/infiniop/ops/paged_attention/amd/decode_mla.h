@@ -870,7 +870,9 @@ __global__ void __launch_bounds__(kMlaWideThreads, 2) decodeMlaChunkKernel(Decod
 //   * K row-major with its 16-byte chunks XOR-swizzled by the row; V row-major in blocks of 16 columns, read back
 //     through the transposing LDS read, a block of 16 tokens x 16 columns at a time (512 contiguous bytes).
 //   * results leave through LDS (the tile buffers) as whole rows, 16 bytes per lane.
-template <typename T, typename Tindex, int WAVES>
+// ONCE: the unit has this one workgroup (all the head chunks of the KV head fit it), so nobody else asks for its tiles
+// and they are fetched with the non-temporal form of the load (see loadLane16ToLds).
+template <typename T, typename Tindex, int WAVES, bool ONCE>
 __global__ void __launch_bounds__(64 * WAVES) decodeMlaRowsKernel(DecodeArgs a) {
     static_assert(WAVES == 4 || WAVES == 8, "one or two wavefronts per SIMD");
     using S = typename T::storage;
@@ -1001,7 +1003,7 @@ __global__ void __launch_bounds__(64 * WAVES) decodeMlaRowsKernel(DecodeArgs a) 
     uint4 *pend_dst = &tiles.k[0][0];
     unsigned long long pend_live = 0ull;
     auto issueSlot = [&](int i) {
-        loadLane16ToLdsMasked(pend_src + slotRowOffset(i), slotLaneOffset(i), pend_dst + slotLds(i), i < copy_loads ? pend_live : 0ull);
+        loadLane16ToLdsMasked<ONCE>(pend_src + slotRowOffset(i), slotLaneOffset(i), pend_dst + slotLds(i), i < copy_loads ? pend_live : 0ull);
     };
     // true: the stage is exactly copy_loads load instructions of this wavefront (what a counted wait relies on)
     auto stageTile = [&](int t, bool deferred) -> bool {
@@ -1026,7 +1028,7 @@ __global__ void __launch_bounds__(64 * WAVES) decodeMlaRowsKernel(DecodeArgs a) 
 #pragma unroll
                 for (int j = 0; j < kSlots; ++j) {
                     if (j < copy_loads) {
-                        loadLane16ToLds(src + slotRowOffset(j), slotLaneOffset(j), dst + slotLds(j));
+                        loadLane16ToLds<ONCE>(src + slotRowOffset(j), slotLaneOffset(j), dst + slotLds(j));
                     }
                 }
             }
@@ -1035,7 +1037,7 @@ __global__ void __launch_bounds__(64 * WAVES) decodeMlaRowsKernel(DecodeArgs a) 
 #pragma unroll
         for (int j = 0; j < kLoadsV; ++j) {
             if (tok0 + vRowOfLoad(j) < end) {
-                loadLane16ToLds(src + slotRowOffset(j) + slotLaneOffset(j), dst + slotLds(j));
+                loadLane16ToLds<ONCE>(src + slotRowOffset(j) + slotLaneOffset(j), dst + slotLds(j));
             } else {
                 dst[slotLds(j) + lane] = make_uint4(0, 0, 0, 0);
             }
@@ -1266,7 +1268,7 @@ __global__ void __launch_bounds__(64 * WAVES) decodeMlaRowsKernel(DecodeArgs a) 
 // Measured (128 heads, 32 sequences of 512 - 4 096 tokens): 60.1 us per call against 66.5 us with a wavefront per
 // chunk; a period takes 0.89 us, either role is busy for 0.8 of it. Not kept: the operands of the next tile read from
 // LDS a period ahead (62.5 us), the load instructions of a period in one burst after the barrier (61.2 - 62.3 us).
-template <typename T, typename Tindex>
+template <typename T, typename Tindex, bool ONCE>
 __global__ void __launch_bounds__(512) decodeMlaRolesKernel(DecodeArgs a) {
     using S = typename T::storage;
     constexpr int kChunks = 4;                    // 16-head chunks of a workgroup
@@ -1361,7 +1363,7 @@ __global__ void __launch_bounds__(512) decodeMlaRolesKernel(DecodeArgs a) {
         const uint32_t lane_offset = ((lane & 31) >> 1) * v_row_bytes + 16u * (2 * (lane >> 5) + (lane & 1)) + 64u * (kLoadsV * cw);
         const char *pend_src = v_head;
         uint4 *pend_dst = &tiles.v[0][0];
-        auto issueSlot = [&](int j) { loadLane16ToLds(pend_src + 64 * j, lane_offset, pend_dst + 64 * (kLoadsV * cw + j)); };
+        auto issueSlot = [&](int j) { loadLane16ToLds<ONCE>(pend_src + 64 * j, lane_offset, pend_dst + 64 * (kLoadsV * cw + j)); };
         auto stageV = [&](int t) {
             pend_src = tileSource(t, v_head, a.v_batch_stride, a.v_row_stride);
             pend_dst = &tiles.v[t % kRing][0];
@@ -1482,9 +1484,9 @@ __global__ void __launch_bounds__(512) decodeMlaRolesKernel(DecodeArgs a) {
     auto issueSlot = [&](int j) { // j < 4: a main part; j == 4: the tails, for the wavefronts that have them
         if (j < 4) {
             const int row = 4 * cw + j;
-            loadLane16ToLds(pend_src + row * k_row_bytes, lane_main ^ (16u * (row & (kSwizzle - 1))), pend_dst + kMainK * row);
+            loadLane16ToLds<ONCE>(pend_src + row * k_row_bytes, lane_main ^ (16u * (row & (kSwizzle - 1))), pend_dst + kMainK * row);
         } else if (copies_tail) {
-            loadLane16ToLds(pend_src, lane_tail, pend_dst + kTailK + 64 * cw);
+            loadLane16ToLds<ONCE>(pend_src, lane_tail, pend_dst + kTailK + 64 * cw);
         }
     };
     auto stageK = [&](int t) {

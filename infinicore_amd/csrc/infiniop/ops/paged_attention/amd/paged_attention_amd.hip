@@ -106,14 +106,24 @@ void launchAll(const DecodeArgs &a, const Plan &plan, bool tiled, hipStream_t st
                     const long long units = static_cast<long long>(a.num_seqs) * plan.max_partitions;
                     wide = dim3(static_cast<unsigned>((units + 7) / 8 * 8 * streams));
                 }
+                // one workgroup per (partition, sequence, KV head): its tiles are fetched once
+                const bool once = groups_of_chunks == 1;
                 if (plan.latent_chunks == 1) {
                     decodeMlaChunkKernel<T, Tindex><<<wide, kMlaWideThreads, 0, stream>>>(a);
                 } else if (plan.latent_chunks == 8) {
-                    decodeMlaRowsKernel<T, Tindex, 8><<<wide, 512, 0, stream>>>(a);
+                    if (once) {
+                        decodeMlaRowsKernel<T, Tindex, 8, true><<<wide, 512, 0, stream>>>(a);
+                    } else {
+                        decodeMlaRowsKernel<T, Tindex, 8, false><<<wide, 512, 0, stream>>>(a);
+                    }
                 } else if (plan.latent_roles) {
-                    decodeMlaRolesKernel<T, Tindex><<<wide, 512, 0, stream>>>(a);
+                    if (once) {
+                        decodeMlaRolesKernel<T, Tindex, true><<<wide, 512, 0, stream>>>(a);
+                    } else {
+                        decodeMlaRolesKernel<T, Tindex, false><<<wide, 512, 0, stream>>>(a);
+                    }
                 } else {
-                    decodeMlaRowsKernel<T, Tindex, 4><<<wide, 256, 0, stream>>>(a);
+                    decodeMlaRowsKernel<T, Tindex, 4, false><<<wide, 256, 0, stream>>>(a);
                 }
                 break;
             }
