@@ -639,6 +639,94 @@ decodeBalancedKernel(const void *early_seq_lens, int early_num_seqs, int early_m
         // (and the flags cleared like any others, so that the next call starts clean).
         const int merged = arrived ? count : 0;
         const float poison = arrived ? 1.0f : __builtin_nanf("");
+        if (heads_here <= 4) {
+            // Up to four heads (the usual GQA ratios): the rows of a segment are heads_here x HEAD floats, and spread
+            // over all 64 lanes as 16-byte chunks (lane l: chunks l, l + 64, ... of the segment, 1 KiB per load
+            // instruction) they are few enough registers that eight segments are in flight at once - one round trip
+            // for most sequences, where the row-per-lane-group form below needs one per four segments and keeps the
+            // three lane groups without a real head idle. Chunk id of a segment = head x HEAD / 4 + q, and chunk q
+            // of a row holds accumulators 4 (q / 16) .. + 3 of lane q % 16 (publishSegment); the parked state of
+            // this wavefront's own segment is read from LDS in the same order, merged, and written back.
+            constexpr int kChunksPerRow = HEAD / 4;
+            constexpr int kMine = 4 * kChunksPerRow / 64; // chunks of a lane: 1 .. 4
+            constexpr int kBatch = 8;                     // segments per round trip
+            int head_of[kMine], stash_at[kMine];
+            float4 mine[kMine];
+            float m_run[kMine], l_run[kMine];
+#pragma unroll
+            for (int k = 0; k < kMine; ++k) {
+                const int id = lane + 64 * k;
+                head_of[k] = id / kChunksPerRow;
+                const int q = id - head_of[k] * kChunksPerRow;
+                stash_at[k] = (4 * (4 * (q >> 4)) + head_of[k]) * 64 + (q & 15); // accumulator 4 (q / 16), row head, lane q % 16
+                mine[k] = make_float4(reader_stash[stash_at[k]], reader_stash[stash_at[k] + 4 * 64],
+                                      reader_stash[stash_at[k] + 8 * 64], reader_stash[stash_at[k] + 12 * 64]);
+                l_run[k] = reader_stash[(4 * G::kCols) * 64 + head_of[k]];
+                m_run[k] = reader_stash[(4 * G::kCols + 1) * 64 + head_of[k]];
+            }
+            for (int i0 = 0; i0 < merged; i0 += kBatch) {
+                float2 ml[kBatch][kMine];
+                float4 v[kBatch][kMine];
+#pragma unroll
+                for (int j = 0; j < kBatch; ++j) {
+                    const int i = min(i0 + j, count - 1); // past the end: the last one again, merged with weight 0
+                    const auto rows = rowsOf(first_piece + i + s);
+                    const auto pairs = pairsOf(first_piece + i + s);
+#pragma unroll
+                    for (int k = 0; k < kMine; ++k) { // (chunks and pairs of heads beyond heads_here lie beyond the buffers: zeros)
+                        ml[j][k] = loadAgent8(pairs, 8 * head_of[k]);
+                        v[j][k] = loadAgent16(rows, 16 * (lane + 64 * k));
+                    }
+                }
+#pragma unroll
+                for (int j = 0; j < kBatch; ++j) {
+                    const bool real = i0 + j < count;
+#pragma unroll
+                    for (int k = 0; k < kMine; ++k) {
+                        const float m_i = real ? ml[j][k].x : -INFINITY;
+                        const float m_new = fmaxf(m_run[k], m_i);
+                        const float w_old = mergeWeight(m_run[k], m_new), w_i = mergeWeight(m_i, m_new);
+                        l_run[k] = l_run[k] * w_old + (real ? ml[j][k].y : 0.0f) * w_i;
+                        mine[k].x = mine[k].x * w_old + v[j][k].x * w_i;
+                        mine[k].y = mine[k].y * w_old + v[j][k].y * w_i;
+                        mine[k].z = mine[k].z * w_old + v[j][k].z * w_i;
+                        mine[k].w = mine[k].w * w_old + v[j][k].w * w_i;
+                        m_run[k] = m_new;
+                    }
+                }
+            }
+#pragma unroll
+            for (int k = 0; k < kMine; ++k) {
+                if (head_of[k] < heads_here) {
+                    reader_stash[stash_at[k]] = mine[k].x;
+                    reader_stash[stash_at[k] + 4 * 64] = mine[k].y;
+                    reader_stash[stash_at[k] + 8 * 64] = mine[k].z;
+                    reader_stash[stash_at[k] + 12 * 64] = mine[k].w;
+                    if (lane + 64 * k == head_of[k] * kChunksPerRow) { // the lane with the head's first chunk
+                        reader_stash[(4 * G::kCols) * 64 + head_of[k]] = l_run[k];
+                    }
+                }
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // the merged state is in LDS before the lanes read each other's
+            if (g == 0) { // the lanes that hold the (up to four) real heads
+                TileState<HEAD> merged_state;
+#pragma unroll
+                for (int e = 0; e < G::kCols; ++e) {
+#pragma unroll
+                    for (int rr = 0; rr < 4; ++rr) {
+                        merged_state.o[e][rr] = reader_stash[(4 * e + rr) * 64 + lane];
+                    }
+                }
+#pragma unroll
+                for (int rr = 0; rr < 4; ++rr) {
+                    if (rr < heads_here) {
+                        const float l_head = reader_stash[(4 * G::kCols) * 64 + rr];
+                        S *o_ptr = static_cast<S *>(a.out) + s * a.o_stride + (first_head + rr) * a.o_head_stride;
+                        storeOutputRow<T, HEAD>(o_ptr, c, merged_state, rr, poison / (l_head + 1e-6f));
+                    }
+                }
+            }
+        } else {
         TileState<HEAD> own;
 #pragma unroll
         for (int e = 0; e < G::kCols; ++e) {
@@ -701,6 +789,7 @@ decodeBalancedKernel(const void *early_seq_lens, int early_num_seqs, int early_m
                     storeOutputRow<T, HEAD>(o_ptr, c, own, rr, poison / (l_run[rr] + 1e-6f));
                 }
             }
+        }
         }
         // the flags are consumed: clear them, so that a replay of this call (same token) starts clean
         for (int base = 0; base < count; base += 64) {
