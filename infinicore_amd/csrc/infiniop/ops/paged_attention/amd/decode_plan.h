@@ -240,8 +240,8 @@ inline Plan makePlan(const PagedAttentionInfo &in, const device::amd::DeviceInfo
         // round trips at the end of the kernel, one batch of four segments after the other: it wins where a
         // sequence is cut into few segments and the call is short. Measured, second kernel vs merged inside
         // (us per call): 128 sequences of 1 024 - 8 192 tokens on 128 pieces per stream 362.3 vs 360.7 at head
-        // 128, 193.1 vs 190.9 at head 64; 32 sequences of 512 - 4 096 tokens 34.3 vs 33.1 at head 64 but 55.0 vs
-        // 56.8 at head 128 and 77.4 vs 79.6 at head 192; 8 sequences of 16 384 - 32 768 tokens 67.8 vs 70.4 at
+        // 128, 193.1 vs 190.9 at head 64; 32 sequences of 512 - 4 096 tokens 33.1 vs 31.6 at head 64 but 55.4 vs
+        // 55.6 at head 128 and 77.4 vs 79.6 at head 192; 8 sequences of 16 384 - 32 768 tokens 67.8 vs 70.4 at
         // head 64; head 256 always loses (102 vs 133).
         const long long pieces = plan.waves_per_stream;
         plan.fused_merge = (in.head_size == 64 && pieces <= 4LL * static_cast<long long>(in.num_seqs))
