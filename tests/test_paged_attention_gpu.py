@@ -882,6 +882,25 @@ def test_remembered_first_tiles_never_leak_into_another_batch(gpu_handle, oracle
     L.check_error(L.LIBINFINIOP.infiniopDestroyPagedAttentionDescriptor(op))
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("D", [64, 128, 192, 256])
+@pytest.mark.parametrize("H,Hkv", [(8, 8), (4, 2), (6, 2), (16, 4), (16, 2)])
+def test_merge_inside_the_decode_kernel_at_every_group_size(gpu_handle, oracle, monkeypatch, D, H, Hkv, dtype):
+    """The reader of a sequence with one to four heads per KV head (rows spread over all lanes, eight segments per
+    round trip) and with eight (a lane group per four heads, four segments per round trip); two long sequences, cut
+    into some sixty segments each, next to short ones and an empty one; work-equalising schedule forced (these
+    batches are small jobs)."""
+    monkeypatch.setenv("INFINIOP_AMD_PA_MERGE", "fused")
+    monkeypatch.setenv("INFINIOP_AMD_PA_SCHEDULE", "balanced")
+    inp = workloads.make_decode_inputs(custom(f"reader_d{D}_h{H}_{Hkv}", dtype, 6, H, Hkv, D, 16, 1, 300, seed=700 + D + H))
+    lens = inp.seq_lens.clone()
+    # make_decode_inputs sized the block table for the drawn lengths: draw again with two long sequences
+    cfg = custom(f"reader_long_d{D}_h{H}_{Hkv}", dtype, 6, H, Hkv, D, 16, 6000, 9000, seed=701 + D + H)
+    inp = workloads.make_decode_inputs(cfg)
+    inp.seq_lens[1], inp.seq_lens[2], inp.seq_lens[4], inp.seq_lens[5] = 0, int(lens[2]), 17, int(lens[5])
+    run_case(gpu_handle, oracle, inp)
+
+
 @pytest.mark.parametrize("D,B", [(64, 40), (128, 136), (64, 136)])
 def test_batches_whose_segments_are_merged_inside_the_decode_kernel_by_default(gpu_handle, oracle, monkeypatch, D, B):
     """No merge knob set: batches of many sequences per piece (and, at head 64, of a few pieces per sequence) are
