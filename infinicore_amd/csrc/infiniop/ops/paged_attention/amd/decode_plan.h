@@ -244,8 +244,13 @@ inline Plan makePlan(const PagedAttentionInfo &in, const device::amd::DeviceInfo
         // 55.6 at head 128 and 77.4 vs 79.6 at head 192; 8 sequences of 16 384 - 32 768 tokens 67.8 vs 70.4 at
         // head 64; head 256 always loses (102 vs 133).
         const long long pieces = plan.waves_per_stream;
-        plan.fused_merge = (in.head_size == 64 && pieces <= 4LL * static_cast<long long>(in.num_seqs))
-                        || (in.head_size == 128 && pieces <= static_cast<long long>(in.num_seqs));
+        // With up to four heads per KV head the reader has eight segments in flight instead of four, and sequences cut
+        // into twice as many segments still gain: head 64, 16 sequences 20.2 vs 21.3 us (8: 15.7 vs 15.8); head 128, 64
+        // sequences 102.5 vs 103.4 (32: 56.4 vs 56.8 in that run, 55.6 vs 55.4 in the benchmark: left to the second
+        // kernel; 16: 31.9 vs 31.6).
+        const long long reach = group <= 4 ? 2 : 1;
+        plan.fused_merge = (in.head_size == 64 && pieces <= 4LL * reach * static_cast<long long>(in.num_seqs))
+                        || (in.head_size == 128 && pieces <= reach * static_cast<long long>(in.num_seqs));
         if (const char *env = std::getenv("INFINIOP_AMD_PA_MERGE")) {
             if (std::strcmp(env, "fused") == 0) {
                 plan.fused_merge = true;
