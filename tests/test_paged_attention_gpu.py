@@ -645,27 +645,31 @@ def test_alibi(gpu_handle, oracle, monkeypatch, dtype, kernel):
 
 # ---- a seeded sweep over everything at once ------------------------------------------------------------
 
-@pytest.mark.parametrize("seed", range(24))
+@pytest.mark.parametrize("seed", range(int(os.environ.get("INFINICORE_AMD_TEST_SWEEP_SEEDS", "40"))))
 def test_random_shapes_schedules_and_dtypes(gpu_handle, oracle, monkeypatch, seed):
-    """Every knob drawn at random from one seed: head size (tiled sizes and 576 / 512), group size, page size,
+    """Every knob drawn at random from one seed: head size (tiled sizes, 576 / 512 and 576 / 576), group size, page size,
     batch, lengths (with empty sequences), dtype, index dtype, ALiBi, schedule and merge mode. The cases above
     vary one thing at a time; this one guards the combinations."""
     rng = np.random.default_rng(1000 + seed)
-    D, Dv = [(64, 0), (128, 0), (128, 0), (192, 0), (256, 0), (576, 512)][rng.integers(0, 6)]
-    Hkv = 1 if Dv else int(rng.choice([1, 2, 4, 8]))
-    group = int(rng.choice([1, 2, 3, 4, 7, 16, 20]))
-    bs = int(rng.choice([8, 16, 16, 32, 64, 128])) if not Dv else int(rng.choice([16, 32, 64]))
-    B = int(rng.choice([1, 2, 5, 17, 40]))
-    hi = int(rng.choice([40, 300, 1500, 5000]))
+    D, Dv = [(64, 0), (128, 0), (128, 0), (192, 0), (256, 0), (576, 512), (576, 512), (576, 576)][rng.integers(0, 8)]
+    Hkv = int(rng.choice([1, 1, 2])) if D == 576 else int(rng.choice([1, 2, 4, 8]))
+    group = int(rng.choice([1, 2, 3, 4, 7, 16, 20])) if D != 576 else int(rng.choice([1, 4, 16, 20, 48, 64, 100, 128]))
+    bs = int(rng.choice([8, 16, 16, 32, 64, 128])) if D != 576 else int(rng.choice([16, 32, 64]))
+    B = int(rng.choice([1, 2, 5, 17, 40])) if D != 576 else int(rng.choice([1, 2, 5, 9]))
+    hi = int(rng.choice([40, 300, 1500, 5000])) if D != 576 else int(rng.choice([40, 300, 1500]))
     dtype = [torch.float16, torch.bfloat16][rng.integers(0, 2)]
     index_dtype = [torch.int64, torch.int32, torch.uint32][rng.integers(0, 3)]
     schedule = [None, "balanced", "grid"][rng.integers(0, 3)]
     merge = ["kernel", "fused"][rng.integers(0, 2)]
+    latent_kernel = [None, "narrow", "wide", "rows"][rng.integers(0, 4)]
     use_alibi = bool(rng.integers(0, 2))
     monkeypatch.delenv("INFINIOP_AMD_PA_SCHEDULE", raising=False)
     if schedule:
         monkeypatch.setenv("INFINIOP_AMD_PA_SCHEDULE", schedule)
     monkeypatch.setenv("INFINIOP_AMD_PA_MERGE", merge)
+    monkeypatch.delenv("INFINIOP_AMD_PA_LATENT_KERNEL", raising=False)
+    if latent_kernel:
+        monkeypatch.setenv("INFINIOP_AMD_PA_LATENT_KERNEL", latent_kernel)
     H = Hkv * group
     inp = workloads.make_decode_inputs(custom(f"sweep{seed}", dtype, B, H, Hkv, D, bs, 1, hi, seed=700 + seed,
                                               value_size=Dv, spare_block_fraction=0.25))
@@ -674,7 +678,7 @@ def test_random_shapes_schedules_and_dtypes(gpu_handle, oracle, monkeypatch, see
         lens[int(rng.integers(0, B))] = 0  # an empty sequence in the middle of the batch
     slopes = torch.tensor(rng.uniform(0.001, 0.3, H), dtype=torch.float32) if use_alibi else None
     print(f"sweep {seed}: D={D}/{Dv or D} H={H}/{Hkv} bs={bs} B={B} hi={hi} {dtype} {index_dtype} schedule={schedule} "
-          f"merge={merge} alibi={use_alibi}", flush=True)
+          f"merge={merge} latent={latent_kernel} alibi={use_alibi}", flush=True)
     q, k, v, bt, _ = to_device(inp)
     out = torch.full((B, H, Dv or D), 7.0, dtype=dtype, device=DEV)
     got = run_paged_attention(gpu_handle, q, k, v, bt.to(index_dtype), lens.to(index_dtype).to(DEV), inp.scale,
