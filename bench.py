@@ -72,7 +72,7 @@ def parse_args():
     ap.add_argument("--layers", type=int, default=32, help="decode: calls per step, each on a KV pool of its own")
     ap.add_argument("--workload", default="c2_llama3_8b_b32")
     ap.add_argument("--head-size", type=int, default=0,
-                    help="run the workload's shape with this head size (64 / 192 / 256) instead of its own; the "
+                    help="run the workload's shape with this head size (64 / 192 / 256 / 576) instead of its own; the "
                          "workload name in the output gets a _d<head> suffix")
     ap.add_argument("--pools", type=int, default=4, help="scatter workloads: distinct cache sets the steps rotate over")
     ap.add_argument("--no-cpu-baseline", action="store_true")
